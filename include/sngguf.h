@@ -1,0 +1,140 @@
+/*
+ * sngguf.h - C ABI of the MI355X (gfx950) GGUF quantized-linear library.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its work on
+ * the HIP stream it is given (a hipStream_t passed as void*, NULL = the null
+ * stream), never synchronises, never allocates and never throws.  The return
+ * value is SNGGUF_OK or a negative SNGGUF_E_* code; sngguf_strerror() turns it
+ * into text.  Buffers are borrowed for the duration of the enqueue only: the
+ * caller keeps them alive by stream ordering.
+ *
+ * The reference (OpenSenseNova/SenseNova-U1) has no native code on this path;
+ * its arithmetic lives in the third-party packages it imports at
+ * src/sensenova_u1/utils/gguf_loader.py:24,29-33,64-66 (diffusers 0.37.1
+ * quantizers/gguf/utils.py, gguf 0.19.0).  Each declaration below names the
+ * Python-level interface it stands in for.
+ */
+#ifndef SNGGUF_H
+#define SNGGUF_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml tensor type numbers (gguf.GGMLQuantizationType, the `quant_type` that
+ * src/sensenova_u1/utils/gguf_loader.py:37-43 stores on each GGUFParameter). */
+enum {
+    SNGGUF_TYPE_Q8_0 = 8,  /* 32 elements / 34 bytes:  f16 d; i8 qs[32]                         */
+    SNGGUF_TYPE_Q4_K = 12, /* 256 elements / 144 bytes: f16 d, dmin; u8 scales[12]; u8 qs[128]  */
+    SNGGUF_TYPE_Q6_K = 14  /* 256 elements / 210 bytes: u8 ql[128]; u8 qh[64]; i8 sc[16]; f16 d */
+};
+
+/* element type of the `out` buffer of sngguf_dequantize */
+enum {
+    SNGGUF_OUT_F32 = 0,
+    SNGGUF_OUT_F16 = 1,
+    SNGGUF_OUT_BF16 = 2
+};
+
+/*
+ * Rounding chain of the block decode.
+ *  SNGGUF_NUM_GGML_FP32      exact fp32 decode (ggml dequantize_row_* semantics), rounded
+ *                            once when a narrower type is asked for.
+ *  SNGGUF_NUM_UPSTREAM_FP16  replays diffusers' dequantize_blocks_* called with dtype=None:
+ *                            every tensor op of that decode is an fp16 op (computed in fp32,
+ *                            rounded to fp16, round-to-nearest-even, subnormals kept), and the
+ *                            fp16 weight is then cast to the compute dtype.  This is what
+ *                            GGUFLinear.forward_native feeds to F.linear, so it is the mode a
+ *                            drop-in uses.
+ */
+enum {
+    SNGGUF_NUM_GGML_FP32 = 0,
+    SNGGUF_NUM_UPSTREAM_FP16 = 1
+};
+
+enum {
+    SNGGUF_OK = 0,
+    SNGGUF_E_BADTYPE = -1,   /* qtype / out_dtype / numerics not one of the enums above       */
+    SNGGUF_E_BADSHAPE = -2,  /* negative size, cols % block != 0, size beyond kernel limits   */
+    SNGGUF_E_NULLPTR = -3,   /* a required pointer is NULL                                    */
+    SNGGUF_E_ALIGN = -4,     /* a pointer violates the alignment stated for it                */
+    SNGGUF_E_LAUNCH = -5,    /* the HIP runtime refused the launch (hipGetLastError != 0)     */
+    SNGGUF_E_NODEVICE = -6   /* no usable gfx950 device / code object                         */
+};
+
+/* Library version (major*10000 + minor*100 + patch) and error text. */
+int sngguf_version(void);
+const char* sngguf_strerror(int code);
+
+/* Bytes per block and elements per block of a ggml type (gguf.GGML_QUANT_SIZES);
+ * 0 for a type this library does not decode. */
+int64_t sngguf_type_size(int qtype);
+int64_t sngguf_block_size(int qtype);
+
+/*
+ * Standalone dequantize.  Replaces diffusers.quantizers.gguf.utils.dequantize_gguf_tensor
+ * (+ dequantize_blocks_Q8_0 / _Q4_K / _Q6_K), the function GGUFLinear.forward_native calls
+ * on the GGUFParameter built at src/sensenova_u1/utils/gguf_loader.py:43, and the upstream
+ * operator seam ops.ggml_dequantize(qweight, qtype, rows, cols).
+ *
+ *  q      packed blocks, row-major [rows][cols / block * type_size] bytes, 2-byte aligned
+ *  out    [rows][cols] elements of out_dtype, aligned to its element size
+ * With SNGGUF_OUT_F32 + SNGGUF_NUM_GGML_FP32 the result is the exact ggml value; with
+ * SNGGUF_OUT_F16 + SNGGUF_NUM_UPSTREAM_FP16 it is bit-identical to the upstream fp16 tensor.
+ */
+int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols,
+                      void* out, int out_dtype, int numerics, void* stream);
+
+/*
+ * y[M][N] = x[M][K] . dequant(q)[N][K]^T (+ bias[N]).  Replaces GGUFLinear.forward
+ * (diffusers quantizers/gguf/utils.py: dequantize -> .to(compute_dtype) -> F.linear), i.e.
+ * what every `module(x)` call at src/sensenova_u1/models/neo_unify/modeling_qwen3.py:214-216,
+ * 444,450,456,504,602,608,614,709,744 executes once the loader has swapped the module.
+ *
+ *  x, y, bias   bf16, row-major, x and y 16-byte aligned, bias may be NULL
+ *  q            packed blocks [N][K / block * type_size], 4-byte aligned rows
+ * The weight is rounded to bf16 exactly as `numerics` says, products are accumulated in
+ * fp32, bias is added in fp32 and the sum is rounded once to bf16.  M <= 16 takes the fused
+ * dequant-GEMV (packed bytes streamed once, nothing dequantized is written to memory);
+ * larger M takes the LDS-staged dequant-GEMM on bf16 MFMA.
+ */
+int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
+                  const void* bias, void* y, int numerics, void* stream);
+
+/*
+ * SiLU-gated pair for the decode MLP: h[M][N] = silu(x.Wg^T) * (x.Wu^T), with both
+ * projections rounded to bf16 first, silu evaluated in fp32 on the rounded gate and rounded
+ * to bf16, and the product rounded to bf16 - the rounding chain of
+ * `self.act_fn(self.gate_proj(x)) * self.up_proj(x)` at
+ * src/sensenova_u1/models/neo_unify/modeling_qwen3.py:215.  Both weights share qtype, N, K.
+ * M <= 16 only (decode); larger M returns SNGGUF_E_BADSHAPE.
+ */
+int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype,
+                        int64_t N, int64_t K, void* h, int numerics, void* stream);
+
+/*
+ * Modality-grouped linear: rows of x whose indicator is 0 use the understanding weights
+ * q_und, rows whose indicator is non-zero use the generation weights q_gen, in one pass:
+ *     y[~ind] = x[~ind] . W_und^T ;  y[ind] = x[ind] . W_gen^T
+ * which is the result the mixed branch spells out at
+ * src/sensenova_u1/models/neo_unify/modeling_qwen3.py:779-783 (and 802-806, 825-829,
+ * 879-883, 1036-1041).
+ *
+ *  indicator    M bytes (0 / non-zero), or NULL: then rows [0, n_text) are text rows and
+ *               rows [n_text, M) are image rows (the contiguous [text | image] layout)
+ *  workspace    device scratch of at least sngguf_grouped_workspace_bytes(M) bytes, 16-byte
+ *               aligned; may be NULL when indicator is NULL
+ *  bias_und / bias_gen   bf16 [N] or NULL
+ */
+int64_t sngguf_grouped_workspace_bytes(int64_t M);
+int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text,
+                          const void* q_und, int qtype_und, const void* q_gen, int qtype_gen,
+                          int64_t N, int64_t K, const void* bias_und, const void* bias_gen,
+                          void* y, void* workspace, int numerics, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SNGGUF_H */

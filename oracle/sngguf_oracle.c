@@ -1,0 +1,297 @@
+/*
+ * sngguf_oracle.c - CPU restatement of the GGUF quantized-linear path.  TEST INFRASTRUCTURE:
+ * only tests, the smoke check and the bench's cpu_baseline leg may build or call this file;
+ * the shipped library never does.
+ *
+ * What it restates.  The reference glue (src/sensenova_u1/utils/gguf_loader.py:17-85) hands
+ * every quantized tensor to diffusers 0.37.1 (uv.lock:164-165), whose GGUFLinear.forward is
+ *     w = dequantize_gguf_tensor(weight)      # dequantize_blocks_Q8_0 / _Q4_K / _Q6_K
+ *     w = w.to(compute_dtype)                 # bf16
+ *     y = F.linear(x, w, bias)
+ * and whose block decoders restate ggml's dequantize_row_q8_0 / q4_K / q6_K and
+ * get_scale_min_k4.  Neither package's source is in the reference tree, so the functions
+ * below restate the published ggml block formats (numerics 0) and the upstream torch op
+ * sequence with its fp16 intermediates (numerics 1).
+ *
+ * Pinning.  Numerics 0 is pinned by closed forms: one-hot positional blocks, scale-packing
+ * cases, encode->decode round trips through independently written packers, hand-written
+ * known-answer blocks and a bitwise cross-check against the vectorised restatement in
+ * oracle.py.  Numerics 1 (which intermediate is rounded to fp16, and when) rests on reading
+ * of the upstream package that cannot be imported here: PARITY UNPINNED for that choice; the
+ * arithmetic of each rounding is pinned against numpy's float16.
+ *
+ * No dependency beyond libc; scalar loops; fp16/bf16 conversions written out by hand so that
+ * they do not share code with numpy, torch or the device kernels.
+ */
+#include <stdint.h>
+#include <string.h>
+#include <math.h>
+
+/* ---- scalar float formats ------------------------------------------------------------ */
+
+static inline float u32_as_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline uint32_t f32_as_u32(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+/* IEEE binary16 -> binary32, exact (subnormals, inf, nan included). */
+float sno_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0) {
+        if (man == 0) return u32_as_f32(sign);
+        /* subnormal: man * 2^-24 */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return sign ? -v : v;
+    }
+    if (exp == 31) return u32_as_f32(sign | 0x7F800000u | (man << 13));
+    return u32_as_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* binary32 -> binary16, round to nearest even, subnormals produced, overflow -> inf. */
+uint16_t sno_f32_to_f16(float f) {
+    uint32_t x = f32_as_u32(f);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t ax = x & 0x7FFFFFFFu;
+    if (ax >= 0x7F800000u) { /* inf / nan */
+        return (uint16_t)(sign | 0x7C00u | ((ax > 0x7F800000u) ? (0x200u | ((ax >> 13) & 0x3FFu)) : 0u));
+    }
+    if (ax >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u); /* >= 65520 rounds to inf */
+    if (ax < 0x38800000u) { /* below the smallest normal half: result is subnormal or zero */
+        if (ax < 0x33000000u) return sign; /* < 2^-25 rounds to zero (2^-25 itself ties to even = 0) */
+        uint32_t e = ax >> 23;                         /* biased fp32 exponent, 102..112 */
+        uint32_t m = (ax & 0x7FFFFFu) | 0x800000u;     /* 24-bit significand */
+        uint32_t shift = 126u - e;                     /* drop so that the unit is 2^-24: 14..24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+    uint32_t e = (ax >> 23) - 112u;
+    uint32_t m = ax & 0x7FFFFFu;
+    uint32_t q = (e << 10) | (m >> 13);
+    uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++; /* carry into the exponent is correct */
+    return (uint16_t)(sign | q);
+}
+
+/* binary32 -> bfloat16, round to nearest even (nan kept quiet). */
+uint16_t sno_f32_to_bf16(float f) {
+    uint32_t x = f32_as_u32(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x40u);
+    uint32_t lsb = (x >> 16) & 1u;
+    x += 0x7FFFu + lsb;
+    return (uint16_t)(x >> 16);
+}
+
+float sno_bf16_to_f32(uint16_t b) { return u32_as_f32((uint32_t)b << 16); }
+
+/* one fp16 tensor-op rounding: the value an fp16 result tensor holds, widened again */
+static inline float r16(float v) { return sno_f16_to_f32(sno_f32_to_f16(v)); }
+
+static inline uint16_t rd16(const uint8_t* p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+
+/* ---- block decoders ------------------------------------------------------------------ */
+/* numerics 0: ggml fp32 semantics.  numerics 1: upstream fp16 op chain, result is the fp16
+ * tensor value widened to fp32 (exactly representable). */
+
+#define QK8_0 32
+#define QK_K 256
+
+/* ggml dequantize_row_q8_0: y[i] = d * qs[i].  Upstream: (d.view(f16) * x.view(i8)) -> f16. */
+void sno_dequantize_row_q8_0(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK8_0;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 34;
+        float d = sno_f16_to_f32(rd16(blk));
+        for (int i = 0; i < 32; i++) {
+            float v = d * (float)(int8_t)blk[2 + i];
+            y[b * 32 + i] = numerics ? r16(v) : v;
+        }
+    }
+}
+
+/* ggml get_scale_min_k4: sub-block j of a Q4_K super-block -> 6-bit scale and 6-bit min. */
+static void scale_min_k4(int j, const uint8_t* s, uint8_t* sc, uint8_t* mn) {
+    if (j < 4) {
+        *sc = s[j] & 63;
+        *mn = s[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4));
+        *mn = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
+    }
+}
+
+/* ggml dequantize_row_q4_K: per 64 elements, low nibbles then high nibbles of 32 bytes;
+ * y = d*sc*q - dmin*m.  Upstream: D=R(d*sc), DM=R(dmin*m), y = R(R(D*q) - DM). */
+void sno_dequantize_row_q4_K(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK_K;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 144;
+        float d = sno_f16_to_f32(rd16(blk));
+        float dmin = sno_f16_to_f32(rd16(blk + 2));
+        const uint8_t* scales = blk + 4;
+        const uint8_t* qs = blk + 16;
+        float* out = y + b * QK_K;
+        for (int c = 0; c < 4; c++) { /* 64-element chunk: sub-blocks 2c and 2c+1 */
+            uint8_t sc0, m0, sc1, m1;
+            scale_min_k4(2 * c, scales, &sc0, &m0);
+            scale_min_k4(2 * c + 1, scales, &sc1, &m1);
+            float d0 = d * (float)sc0, mm0 = dmin * (float)m0;
+            float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+            if (numerics) { d0 = r16(d0); mm0 = r16(mm0); d1 = r16(d1); mm1 = r16(mm1); }
+            for (int l = 0; l < 32; l++) {
+                float lo = (float)(qs[32 * c + l] & 0x0F);
+                float hi = (float)(qs[32 * c + l] >> 4);
+                if (numerics) {
+                    out[64 * c + l] = r16(r16(d0 * lo) - mm0);
+                    out[64 * c + 32 + l] = r16(r16(d1 * hi) - mm1);
+                } else {
+                    out[64 * c + l] = d0 * lo - mm0;
+                    out[64 * c + 32 + l] = d1 * hi - mm1;
+                }
+            }
+        }
+    }
+}
+
+/* ggml dequantize_row_q6_K: per 128-element half, 32 lanes l give elements l, l+32, l+64,
+ * l+96; y = d*scale[e/16]*(q-32).  Upstream: D=R(d*scale), y=R(D*(q-32)). */
+void sno_dequantize_row_q6_K(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK_K;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 210;
+        const uint8_t* ql = blk;
+        const uint8_t* qh = blk + 128;
+        const int8_t* sc = (const int8_t*)(blk + 192);
+        float d = sno_f16_to_f32(rd16(blk + 208));
+        float* out = y + b * QK_K;
+        for (int h = 0; h < 2; h++) {
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int q1 = (int)((ql[64 * h + l] & 0x0F) | (((qh[32 * h + l] >> 0) & 3) << 4)) - 32;
+                int q2 = (int)((ql[64 * h + l + 32] & 0x0F) | (((qh[32 * h + l] >> 2) & 3) << 4)) - 32;
+                int q3 = (int)((ql[64 * h + l] >> 4) | (((qh[32 * h + l] >> 4) & 3) << 4)) - 32;
+                int q4 = (int)((ql[64 * h + l + 32] >> 4) | (((qh[32 * h + l] >> 6) & 3) << 4)) - 32;
+                float s1 = d * (float)sc[8 * h + is + 0];
+                float s2 = d * (float)sc[8 * h + is + 2];
+                float s3 = d * (float)sc[8 * h + is + 4];
+                float s4 = d * (float)sc[8 * h + is + 6];
+                float v1, v2, v3, v4;
+                if (numerics) {
+                    v1 = r16(r16(s1) * (float)q1); v2 = r16(r16(s2) * (float)q2);
+                    v3 = r16(r16(s3) * (float)q3); v4 = r16(r16(s4) * (float)q4);
+                } else {
+                    v1 = s1 * (float)q1; v2 = s2 * (float)q2; v3 = s3 * (float)q3; v4 = s4 * (float)q4;
+                }
+                out[128 * h + l] = v1;
+                out[128 * h + l + 32] = v2;
+                out[128 * h + l + 64] = v3;
+                out[128 * h + l + 96] = v4;
+            }
+        }
+    }
+}
+
+int64_t sno_type_size(int qtype) { return qtype == 8 ? 34 : qtype == 12 ? 144 : qtype == 14 ? 210 : 0; }
+int64_t sno_block_size(int qtype) { return qtype == 8 ? 32 : (qtype == 12 || qtype == 14) ? 256 : 0; }
+
+static int dequant_row(const uint8_t* src, int qtype, float* y, int64_t k, int numerics) {
+    switch (qtype) {
+    case 8: sno_dequantize_row_q8_0(src, y, k, numerics); return 0;
+    case 12: sno_dequantize_row_q4_K(src, y, k, numerics); return 0;
+    case 14: sno_dequantize_row_q6_K(src, y, k, numerics); return 0;
+    default: return -1;
+    }
+}
+
+/*
+ * dequantize_gguf_tensor: bytes [rows][cols/bs*ts] -> [rows][cols] of out_dtype
+ * (0 = fp32, 1 = fp16 bits, 2 = bf16 bits).  `scratch` holds cols floats.
+ */
+int sno_dequantize(const uint8_t* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype,
+                   int numerics, float* scratch) {
+    int64_t bs = sno_block_size(qtype), ts = sno_type_size(qtype);
+    if (!bs || cols % bs) return -2;
+    int64_t row_bytes = cols / bs * ts;
+    for (int64_t r = 0; r < rows; r++) {
+        float* dst = out_dtype == 0 ? (float*)out + r * cols : scratch;
+        if (dequant_row(q + r * row_bytes, qtype, dst, cols, numerics)) return -1;
+        if (out_dtype == 1) {
+            uint16_t* o = (uint16_t*)out + r * cols;
+            for (int64_t i = 0; i < cols; i++) o[i] = sno_f32_to_f16(dst[i]);
+        } else if (out_dtype == 2) {
+            uint16_t* o = (uint16_t*)out + r * cols;
+            for (int64_t i = 0; i < cols; i++) o[i] = sno_f32_to_bf16(dst[i]);
+        }
+    }
+    return 0;
+}
+
+/*
+ * GGUFLinear.forward_native on bf16 bit patterns: the weight row is decoded, rounded to bf16,
+ * and dotted with each bf16 activation row.  The accumulator is a double, i.e. the exact sum
+ * up to 2^-53 - the value every fp32 summation order of F.linear scatters around - and the
+ * result (plus bias) is rounded to fp32 and then to bf16.  `scratch` holds K floats.
+ */
+int sno_linear(const uint16_t* x, int64_t M, const uint8_t* q, int qtype, int64_t N, int64_t K,
+               const uint16_t* bias, uint16_t* y, int numerics, float* scratch) {
+    int64_t bs = sno_block_size(qtype), ts = sno_type_size(qtype);
+    if (!bs || K % bs) return -2;
+    int64_t row_bytes = K / bs * ts;
+    for (int64_t n = 0; n < N; n++) {
+        if (dequant_row(q + n * row_bytes, qtype, scratch, K, numerics)) return -1;
+        for (int64_t i = 0; i < K; i++) scratch[i] = sno_bf16_to_f32(sno_f32_to_bf16(scratch[i]));
+        for (int64_t m = 0; m < M; m++) {
+            const uint16_t* xr = x + m * K;
+            double acc = 0.0;
+            for (int64_t i = 0; i < K; i++) acc += (double)sno_bf16_to_f32(xr[i]) * (double)scratch[i];
+            if (bias) acc += (double)sno_bf16_to_f32(bias[n]);
+            y[m * N + n] = sno_f32_to_bf16((float)acc);
+        }
+    }
+    return 0;
+}
+
+/* SiLU gating with the bf16 rounding after every torch op of
+ * `act_fn(gate_proj(x)) * up_proj(x)` (modeling_qwen3.py:215): inputs are the two bf16
+ * projection outputs. */
+void sno_silu_mul(const uint16_t* gate, const uint16_t* up, uint16_t* h, int64_t n) {
+    for (int64_t i = 0; i < n; i++) {
+        float g = sno_bf16_to_f32(gate[i]);
+        float s = sno_bf16_to_f32(sno_f32_to_bf16(g / (1.0f + expf(-g))));
+        h[i] = sno_f32_to_bf16(s * sno_bf16_to_f32(up[i]));
+    }
+}
+
+/*
+ * Mixed-modality routing as the unreachable branch at modeling_qwen3.py:779-783 defines it:
+ * out = zeros; out[~ind] = proj(x[~ind]); out[ind] = proj_mot_gen(x[ind]).
+ */
+int sno_grouped_linear(const uint16_t* x, int64_t M, const uint8_t* indicator, const uint8_t* q_und,
+                       int qtype_und, const uint8_t* q_gen, int qtype_gen, int64_t N, int64_t K,
+                       const uint16_t* bias_und, const uint16_t* bias_gen, uint16_t* y, int numerics,
+                       float* scratch) {
+    memset(y, 0, (size_t)(M * N) * sizeof(uint16_t));
+    for (int tower = 0; tower < 2; tower++) {
+        const uint8_t* q = tower ? q_gen : q_und;
+        const uint16_t* bias = tower ? bias_gen : bias_und;
+        int qtype = tower ? qtype_gen : qtype_und;
+        int64_t bs = sno_block_size(qtype), ts = sno_type_size(qtype);
+        if (!bs || K % bs) return -2;
+        int64_t row_bytes = K / bs * ts;
+        for (int64_t n = 0; n < N; n++) {
+            if (dequant_row(q + n * row_bytes, qtype, scratch, K, numerics)) return -1;
+            for (int64_t i = 0; i < K; i++) scratch[i] = sno_bf16_to_f32(sno_f32_to_bf16(scratch[i]));
+            for (int64_t m = 0; m < M; m++) {
+                if ((indicator[m] != 0) != tower) continue;
+                const uint16_t* xr = x + m * K;
+                double acc = 0.0;
+                for (int64_t i = 0; i < K; i++) acc += (double)sno_bf16_to_f32(xr[i]) * (double)scratch[i];
+                if (bias) acc += (double)sno_bf16_to_f32(bias[n]);
+                y[m * N + n] = sno_f32_to_bf16((float)acc);
+            }
+        }
+    }
+    return 0;
+}

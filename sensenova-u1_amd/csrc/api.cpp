@@ -1,0 +1,117 @@
+// extern "C" entry points of libsngguf: argument validation and routing to the kernel
+// launchers.  Nothing here allocates, synchronises or throws.
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+#include "../../include/sngguf.h"
+
+namespace sngguf {
+int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
+                      hipStream_t stream);
+int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
+                const void* bias, void* y, int numerics, bool gated, hipStream_t stream);
+int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                int numerics, hipStream_t stream);
+int64_t grouped_workspace_bytes(int64_t M);
+int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
+                        int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
+                        const void* bias_gen, void* y, void* workspace, int numerics, hipStream_t stream);
+}  // namespace sngguf
+
+namespace {
+
+constexpr int64_t kMaxDim = (int64_t)1 << 31;  // kernels index rows / columns with 32-bit tile counters
+
+inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline bool known_type(int t) { return t == SNGGUF_TYPE_Q8_0 || t == SNGGUF_TYPE_Q4_K || t == SNGGUF_TYPE_Q6_K; }
+inline bool known_numerics(int n) { return n == SNGGUF_NUM_GGML_FP32 || n == SNGGUF_NUM_UPSTREAM_FP16; }
+
+// Shape / pointer checks shared by the matmul entry points.
+int check_matmul(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* y, int numerics) {
+    if (!known_type(qtype) || !known_numerics(numerics)) return SNGGUF_E_BADTYPE;
+    if (M < 0 || N < 0 || K <= 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim) return SNGGUF_E_BADSHAPE;
+    if (K % sngguf_block_size(qtype) != 0) return SNGGUF_E_BADSHAPE;
+    if (M == 0 || N == 0) return SNGGUF_OK;
+    if (!x || !q || !y) return SNGGUF_E_NULLPTR;
+    if (!aligned(x, 16) || !aligned(y, 16) || !aligned(q, 16)) return SNGGUF_E_ALIGN;
+    return SNGGUF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sngguf_version(void) { return 100; }
+
+const char* sngguf_strerror(int code) {
+    switch (code) {
+    case SNGGUF_OK: return "ok";
+    case SNGGUF_E_BADTYPE: return "unsupported quant type, output dtype or numerics mode";
+    case SNGGUF_E_BADSHAPE: return "bad shape (negative, not a multiple of the block size, or too large)";
+    case SNGGUF_E_NULLPTR: return "required pointer is NULL";
+    case SNGGUF_E_ALIGN: return "pointer is not aligned as required";
+    case SNGGUF_E_LAUNCH: return "HIP kernel launch failed";
+    case SNGGUF_E_NODEVICE: return "no usable gfx950 device";
+    default: return "unknown error";
+    }
+}
+
+int64_t sngguf_type_size(int qtype) {
+    return qtype == SNGGUF_TYPE_Q8_0 ? 34 : qtype == SNGGUF_TYPE_Q4_K ? 144 : qtype == SNGGUF_TYPE_Q6_K ? 210 : 0;
+}
+
+int64_t sngguf_block_size(int qtype) {
+    return qtype == SNGGUF_TYPE_Q8_0 ? 32 : (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q6_K) ? 256 : 0;
+}
+
+int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
+                      void* stream) {
+    if (!known_type(qtype) || !known_numerics(numerics)) return SNGGUF_E_BADTYPE;
+    if (out_dtype != SNGGUF_OUT_F32 && out_dtype != SNGGUF_OUT_F16 && out_dtype != SNGGUF_OUT_BF16) return SNGGUF_E_BADTYPE;
+    if (rows < 0 || cols < 0 || rows >= kMaxDim || cols >= kMaxDim) return SNGGUF_E_BADSHAPE;
+    if (cols % sngguf_block_size(qtype) != 0) return SNGGUF_E_BADSHAPE;
+    if (rows == 0 || cols == 0) return SNGGUF_OK;
+    if (!q || !out) return SNGGUF_E_NULLPTR;
+    if (!aligned(q, 16) || !aligned(out, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_dequantize(q, qtype, rows, cols, out, out_dtype, numerics, static_cast<hipStream_t>(stream));
+}
+
+int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                  int numerics, void* stream) {
+    const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (M <= 16) return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, y, numerics, false, s);
+    return sngguf::launch_gemm(x, M, q, qtype, N, K, bias, y, numerics, s);
+}
+
+int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype, int64_t N, int64_t K,
+                        void* h, int numerics, void* stream) {
+    const int rc = check_matmul(x, M, q_gate, qtype, N, K, h, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (!q_up) return SNGGUF_E_NULLPTR;
+    if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
+    if (M > 16 || K % 64 != 0) return SNGGUF_E_BADSHAPE;
+    return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+}
+
+int64_t sngguf_grouped_workspace_bytes(int64_t M) { return sngguf::grouped_workspace_bytes(M); }
+
+int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
+                          int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
+                          const void* bias_gen, void* y, void* workspace, int numerics, void* stream) {
+    int rc = check_matmul(x, M, q_und, qtype_und, N, K, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    rc = check_matmul(x, M, q_gen, qtype_gen, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (indicator) {
+        if (!workspace) return SNGGUF_E_NULLPTR;
+        if (!aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+    } else if (n_text < 0 || n_text > M) {
+        return SNGGUF_E_BADSHAPE;
+    }
+    return sngguf::launch_grouped_gemm(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und,
+                                       bias_gen, y, workspace, numerics, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,311 @@
+// Fused dequant-GEMV for decode (M <= 16).
+//
+// One wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate matrix
+// and row n of the up matrix).  A lane takes 64 weight elements per step - 68 bytes of Q8_0,
+// one 32-byte nibble chunk of Q4_K, three 16-byte runs of Q6_K - so that one step of the wave
+// reads one contiguous 4352 / 2304 / 3360-byte span of each row.  The packed bytes go from
+// HBM to registers once, are decoded to bf16 pairs there, multiplied with the bf16
+// activations (v_dot2_f32_bf16, fp32 accumulate) and reduced across the wavefront with DPP;
+// no dequantized weight ever reaches memory.
+#include "sngguf_common.hpp"
+
+namespace sngguf {
+
+// ---- per-lane unit decoders: 64 elements -> 32 packed bf16 pairs -----------------------------
+// The pair order matches x_unit_offset(): pair i holds elements run(i / 8) + 2 * (i % 8) + {0, 1}.
+
+// element offset of 16-element run t (0..3) of unit u
+template <int QT>
+__device__ __forceinline__ int64_t unit_run_offset(int64_t u, int t) {
+    if constexpr (QT == SNGGUF_TYPE_Q6_K) {
+        // unit = (block, half h, 16-lane group j); run t is quadrant t of that half
+        const int64_t b = u >> 2;
+        const int h = (int)(u >> 1) & 1, j = (int)u & 1;
+        return b * 256 + 128 * h + 32 * t + 16 * j;
+    } else {
+        return u * 64 + 16 * t;
+    }
+}
+
+template <int NUM>
+__device__ __forceinline__ uint32_t q8_pair(float d, uint32_t two) {  // two int8 in the low half
+    const float a = rnd<NUM>(d * (float)(int8_t)(two & 0xFF));
+    const float b = rnd<NUM>(d * (float)(int8_t)((two >> 8) & 0xFF));
+    return pack_bf16(a, b);
+}
+
+template <int NUM>
+__device__ __forceinline__ void decode_unit_q8_0(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    const uint8_t* p = row + u * 68;  // two blocks; 4-byte aligned because K % 64 == 0
+    uint32_t L[17];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const u32x4_t v = ld_u128_a4(p + 16 * i);
+        L[4 * i] = v[0]; L[4 * i + 1] = v[1]; L[4 * i + 2] = v[2]; L[4 * i + 3] = v[3];
+    }
+    L[16] = ld_u32(p + 64);
+    const float d0 = f16_to_f32((uint16_t)(L[0] & 0xFFFF));
+    const float d1 = f16_to_f32((uint16_t)(L[8] >> 16));
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t q0 = __builtin_amdgcn_alignbit(L[i + 1], L[i], 16);  // block 0 quants sit 2 bytes off
+        wp[2 * i] = q8_pair<NUM>(d0, q0);
+        wp[2 * i + 1] = q8_pair<NUM>(d0, q0 >> 16);
+        const uint32_t q1 = L[9 + i];
+        wp[16 + 2 * i] = q8_pair<NUM>(d1, q1);
+        wp[16 + 2 * i + 1] = q8_pair<NUM>(d1, q1 >> 16);
+    }
+}
+
+template <int NUM>
+__device__ __forceinline__ void decode_unit_q4_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    const uint8_t* blk = row + (u >> 2) * 144;
+    const int c = (int)u & 3;
+    const u32x4_t hdr = *reinterpret_cast<const u32x4_t*>(blk);
+    const u32x4_t qa = *reinterpret_cast<const u32x4_t*>(blk + 16 + 32 * c);
+    const u32x4_t qb = *reinterpret_cast<const u32x4_t*>(blk + 32 + 32 * c);
+    const float d = f16_to_f32((uint16_t)(hdr[0] & 0xFFFF));
+    const float dmin = f16_to_f32((uint16_t)(hdr[0] >> 16));
+    uint32_t sc0, mn0, sc1, mn1;
+    q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c, sc0, mn0);
+    q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c + 1, sc1, mn1);
+    const float D0 = rnd<NUM>(d * (float)sc0), M0 = rnd<NUM>(dmin * (float)mn0);
+    const float D1 = rnd<NUM>(d * (float)sc1), M1 = rnd<NUM>(dmin * (float)mn1);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {  // dword i of the 32 quant bytes: elements 4i..4i+3 (low) and 32+4i.. (high)
+        const uint32_t q = i < 4 ? qa[i] : qb[i - 4];
+        float lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t byte = (q >> (8 * k)) & 0xFFu;
+            lo[k] = rnd<NUM>(rnd<NUM>(D0 * (float)(byte & 0x0Fu)) - M0);
+            hi[k] = rnd<NUM>(rnd<NUM>(D1 * (float)(byte >> 4)) - M1);
+        }
+        wp[2 * i] = pack_bf16(lo[0], lo[1]);
+        wp[2 * i + 1] = pack_bf16(lo[2], lo[3]);
+        wp[16 + 2 * i] = pack_bf16(hi[0], hi[1]);
+        wp[16 + 2 * i + 1] = pack_bf16(hi[2], hi[3]);
+    }
+}
+
+template <int NUM>
+__device__ __forceinline__ void decode_unit_q6_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    const uint8_t* blk = row + (u >> 2) * 210;  // 2-byte aligned
+    const int h = (int)(u >> 1) & 1, j = (int)u & 1;
+    const u32x4_t la = ld_u128_a2(blk + 64 * h + 16 * j);        // ql[l], l = 16j..16j+15
+    const u32x4_t lb = ld_u128_a2(blk + 64 * h + 32 + 16 * j);   // ql[l + 32]
+    const u32x4_t hh = ld_u128_a2(blk + 128 + 32 * h + 16 * j);  // qh[l]
+    const float d = f16_to_f32(ld_u16(blk + 208));
+    float D[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) D[t] = rnd<NUM>(d * (float)(int8_t)blk[192 + 8 * h + j + 2 * t]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {  // dword i: l = 16j + 4i .. +3
+        float v[4][4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t a = (la[i] >> (8 * k)) & 0xFFu, b = (lb[i] >> (8 * k)) & 0xFFu, c = (hh[i] >> (8 * k)) & 0xFFu;
+            const int q1 = (int)((a & 0x0Fu) | ((c & 3u) << 4)) - 32;
+            const int q2 = (int)((b & 0x0Fu) | (((c >> 2) & 3u) << 4)) - 32;
+            const int q3 = (int)((a >> 4) | (((c >> 4) & 3u) << 4)) - 32;
+            const int q4 = (int)((b >> 4) | (((c >> 6) & 3u) << 4)) - 32;
+            v[0][k] = rnd<NUM>(D[0] * (float)q1);
+            v[1][k] = rnd<NUM>(D[1] * (float)q2);
+            v[2][k] = rnd<NUM>(D[2] * (float)q3);
+            v[3][k] = rnd<NUM>(D[3] * (float)q4);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            wp[8 * t + 2 * i] = pack_bf16(v[t][0], v[t][1]);
+            wp[8 * t + 2 * i + 1] = pack_bf16(v[t][2], v[t][3]);
+        }
+    }
+}
+
+template <int QT, int NUM>
+__device__ __forceinline__ void decode_unit(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    if constexpr (QT == SNGGUF_TYPE_Q8_0) decode_unit_q8_0<NUM>(row, u, wp);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode_unit_q4_k<NUM>(row, u, wp);
+    else decode_unit_q6_k<NUM>(row, u, wp);
+}
+
+__device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, x), acc, false);
+}
+
+// ---- kernel ------------------------------------------------------------------------------------
+// GATED == false: rows (2p, 2p+1) of one matrix, y[m][n] = bf16(acc + bias[n]).
+// GATED == true : row p of qa (gate) and of qb (up), y[m][p] = bf16(bf16(silu(bf16 g)) * bf16 u).
+
+template <int QT, int NUM, int MT, bool GATED>
+__global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
+                                                   const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                   const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t n_pairs = GATED ? N : (N + 1) / 2;
+    if (pair >= n_pairs) return;
+    const int64_t row_bytes = K / Fmt<QT>::bs * Fmt<QT>::ts;
+    int64_t na, nb;
+    const uint8_t *ra, *rb;
+    if constexpr (GATED) {
+        na = nb = pair;
+        ra = qa + pair * row_bytes;
+        rb = qb + pair * row_bytes;
+    } else {
+        na = 2 * pair;
+        nb = na + 1 < N ? na + 1 : na;  // odd N: the last wave decodes its row twice, stores once
+        ra = qa + na * row_bytes;
+        rb = qa + nb * row_bytes;
+    }
+    float acc_a[MT], acc_b[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc_a[m] = acc_b[m] = 0.f;
+
+    const int64_t units = K >> 6;
+    for (int64_t u = lane; u < units; u += 64) {
+        uint32_t wa[32], wb[32];
+        decode_unit<QT, NUM>(ra, u, wa);
+        decode_unit<QT, NUM>(rb, u, wb);
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            if (m < M) {
+                const bf16_t* xr = x + (int64_t)m * K;
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const u32x4_t* xp = reinterpret_cast<const u32x4_t*>(xr + unit_run_offset<QT>(u, t));
+                    const u32x4_t x0 = xp[0], x1 = xp[1];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        acc_a[m] = dot2(wa[8 * t + i], x0[i], acc_a[m]);
+                        acc_b[m] = dot2(wb[8 * t + i], x0[i], acc_b[m]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        acc_a[m] = dot2(wa[8 * t + 4 + i], x1[i], acc_a[m]);
+                        acc_b[m] = dot2(wb[8 * t + 4 + i], x1[i], acc_b[m]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+        if (m < M) {
+            const float sa = wave_sum(acc_a[m]);
+            const float sb = wave_sum(acc_b[m]);
+            if (lane == 0) {
+                if constexpr (GATED) {
+                    const float g = bf16_to_f32(f32_to_bf16(sa));
+                    const float up = bf16_to_f32(f32_to_bf16(sb));
+                    const float s = bf16_to_f32(f32_to_bf16(g / (1.0f + expf(-g))));
+                    y[(int64_t)m * N + pair] = f32_to_bf16(s * up);
+                } else {
+                    const float ba = bias ? bf16_to_f32(bias[na]) : 0.f;
+                    y[(int64_t)m * N + na] = f32_to_bf16(sa + ba);
+                    if (nb != na) {
+                        const float bb = bias ? bf16_to_f32(bias[nb]) : 0.f;
+                        y[(int64_t)m * N + nb] = f32_to_bf16(sb + bb);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Q8_0 rows whose block count is odd are not a whole number of 64-element units (and their
+// rows are only 2-byte aligned): they take this plain path, one wavefront per row, eight
+// elements per lane and step through the shared 8-element decoder.
+template <int QT, int NUM>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q,
+                                                           int64_t N, int64_t K, const bf16_t* __restrict__ bias,
+                                                           bf16_t* __restrict__ y) {
+    const int lane = threadIdx.x & 63;
+    const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const int64_t row_bytes = K / Fmt<QT>::bs * Fmt<QT>::ts;
+    const uint8_t* row = q + n * row_bytes;
+    float acc[16];
+#pragma unroll
+    for (int m = 0; m < 16; m++) acc[m] = 0.f;
+    for (int64_t e0 = (int64_t)lane * 8; e0 < K; e0 += 64 * 8) {
+        float w[8];
+        decode8<QT, NUM>(row, e0, w);
+#pragma unroll
+        for (int i = 0; i < 8; i++) w[i] = bf16_to_f32(f32_to_bf16(w[i]));
+        for (int m = 0; m < M; m++) {
+            const bf16_t* xr = x + (int64_t)m * K + e0;
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) s = fmaf(w[i], bf16_to_f32(xr[i]), s);
+#pragma unroll
+            for (int mm = 0; mm < 16; mm++)
+                if (mm == m) acc[mm] += s;
+        }
+    }
+    for (int m = 0; m < M; m++) {
+        float v = 0.f;
+#pragma unroll
+        for (int mm = 0; mm < 16; mm++)
+            if (mm == m) v = acc[mm];
+        v = wave_sum(v);
+        if (lane == 0) y[(int64_t)m * N + n] = f32_to_bf16(v + (bias ? bf16_to_f32(bias[n]) : 0.f));
+    }
+}
+
+// ---- host-side dispatch ------------------------------------------------------------------------
+
+template <int QT, int NUM, bool GATED>
+static int launch_mt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                     const bf16_t* bias, bf16_t* y, hipStream_t stream) {
+    const int64_t n_pairs = GATED ? N : (N + 1) / 2;
+    dim3 grid((unsigned)((n_pairs + 3) / 4)), block(256);
+#define SNGGUF_GEMV_CASE(MT) \
+    gemv_kernel<QT, NUM, MT, GATED><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y)
+    if (M == 1) SNGGUF_GEMV_CASE(1);
+    else if (M == 2) SNGGUF_GEMV_CASE(2);
+    else if (M <= 4) SNGGUF_GEMV_CASE(4);
+    else if (M <= 8) SNGGUF_GEMV_CASE(8);
+    else SNGGUF_GEMV_CASE(16);
+#undef SNGGUF_GEMV_CASE
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
+template <int QT, int NUM>
+static int launch_gated(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                        const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+    if (K % 64 != 0) {  // only Q8_0 with an odd block count
+        if (gated) return SNGGUF_E_BADSHAPE;
+        dim3 grid((unsigned)((N + 3) / 4)), block(256);
+        gemv_generic_kernel<QT, NUM><<<grid, block, 0, stream>>>(x, M, qa, N, K, bias, y);
+        return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+    }
+    if (gated) return launch_mt<QT, NUM, true>(x, M, qa, qb, N, K, bias, y, stream);
+    return launch_mt<QT, NUM, false>(x, M, qa, qb, N, K, bias, y, stream);
+}
+
+template <int QT>
+static int launch_num(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                      const bf16_t* bias, bf16_t* y, int numerics, bool gated, hipStream_t stream) {
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_gated<QT, SNGGUF_NUM_GGML_FP32>(x, M, qa, qb, N, K, bias, y, gated, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_gated<QT, SNGGUF_NUM_UPSTREAM_FP16>(x, M, qa, qb, N, K, bias, y, gated, stream);
+    return SNGGUF_E_BADTYPE;
+}
+
+// M in 1..16, N >= 1, K a positive multiple of the block size (checked by the caller).
+int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
+                const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
+    const bf16_t* xp = static_cast<const bf16_t*>(x);
+    const uint8_t* a = static_cast<const uint8_t*>(qa);
+    const uint8_t* b = static_cast<const uint8_t*>(qb);
+    const bf16_t* bp = static_cast<const bf16_t*>(bias);
+    bf16_t* yp = static_cast<bf16_t*>(y);
+    switch (qtype) {
+    case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
+    case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
+    case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
+    default: return SNGGUF_E_BADTYPE;
+    }
+}
+
+}  // namespace sngguf

@@ -1,0 +1,193 @@
+// Shared device helpers of the gfx950 GGUF quantized-linear kernels: scalar format
+// conversions, the three block decoders and wavefront reductions.  Included by every .hip
+// file of the library; nothing here touches the host runtime.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/sngguf.h"
+
+namespace sngguf {
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---- scalar formats ---------------------------------------------------------------------
+
+__device__ __forceinline__ float f16_to_f32(uint16_t bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+__device__ __forceinline__ uint16_t f32_to_f16(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+// One fp16 tensor-op rounding (v_cvt_f16_f32 is round-to-nearest-even with subnormals), widened again.
+__device__ __forceinline__ float round_f16(float v) { return (float)(_Float16)v; }
+__device__ __forceinline__ bf16_t f32_to_bf16(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t p) { return __builtin_bit_cast(float, p << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t p) { return __builtin_bit_cast(float, p & 0xFFFF0000u); }
+// two floats -> packed bf16 pair (low half = a), one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    f2 f = {a, b};
+    v2 r = __builtin_convertvector(f, v2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// NUM == SNGGUF_NUM_UPSTREAM_FP16: the value is an fp16 tensor element; else exact fp32.
+template <int NUM>
+__device__ __forceinline__ float rnd(float v) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) return round_f16(v);
+    return v;
+}
+
+// ---- unaligned loads ----------------------------------------------------------------------
+// GGUF blocks are only 2-byte aligned (34- and 210-byte blocks).  memcpy from a pointer of
+// declared alignment lets the compiler pick the widest legal access.
+
+__device__ __forceinline__ uint16_t ld_u16(const uint8_t* p) {
+    return *reinterpret_cast<const uint16_t*>(p);
+}
+// 4 / 16 bytes from an address that is only 2-byte aligned (gfx950 runs global and LDS
+// accesses in unaligned mode, so these become one dword / dwordx4 access)
+__device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
+    return v;
+}
+__device__ __forceinline__ u32x4_t ld_u128_a2(const uint8_t* p) {
+    u32x4_t v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
+    return v;
+}
+__device__ __forceinline__ u32x4_t ld_u128_a4(const uint8_t* p) {
+    u32x4_t v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
+    return v;
+}
+__device__ __forceinline__ uint32_t ld_u32(const uint8_t* p) { return *reinterpret_cast<const uint32_t*>(p); }
+
+// ---- format constants -----------------------------------------------------------------------
+
+template <int QT> struct Fmt;
+template <> struct Fmt<SNGGUF_TYPE_Q8_0> { static constexpr int bs = 32, ts = 34; };
+template <> struct Fmt<SNGGUF_TYPE_Q4_K> { static constexpr int bs = 256, ts = 144; };
+template <> struct Fmt<SNGGUF_TYPE_Q6_K> { static constexpr int bs = 256, ts = 210; };
+
+// Q4_K: 6-bit (scale, min) of sub-block j from the 12 packed bytes held as three dwords
+// s0 = bytes 0..3, s1 = bytes 4..7, s2 = bytes 8..11.
+__device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j, uint32_t& sc, uint32_t& mn) {
+    if (j < 4) {
+        sc = (s0 >> (8 * j)) & 63u;
+        mn = (s1 >> (8 * j)) & 63u;
+    } else {
+        const int i = j - 4;
+        const uint32_t b = (s2 >> (8 * i)) & 0xFFu;
+        sc = (b & 0x0Fu) | (((s0 >> (8 * i + 6)) & 3u) << 4);
+        mn = (b >> 4) | (((s1 >> (8 * i + 6)) & 3u) << 4);
+    }
+}
+
+// ---- 8-element decoders (standalone dequantize, GEMM tile fill) -------------------------------
+// decode8<QT,NUM>(row, e0, w): eight consecutive elements e0..e0+7 (e0 % 8 == 0) of a packed
+// row, as the fp32 value of the ggml decode (NUM 0) or of the upstream fp16 tensor (NUM 1).
+
+template <int QT, int NUM>
+__device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]);
+
+template <int NUM>
+__device__ __forceinline__ void decode8_q8_0(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    const uint8_t* blk = row + (e0 >> 5) * 34;
+    const float d = f16_to_f32(ld_u16(blk));
+    const uint8_t* qs = blk + 2 + (e0 & 31);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t h = ld_u16(qs + 2 * i);
+        w[2 * i] = rnd<NUM>(d * (float)(int8_t)(h & 0xFF));
+        w[2 * i + 1] = rnd<NUM>(d * (float)(int8_t)(h >> 8));
+    }
+}
+
+template <int NUM>
+__device__ __forceinline__ void decode8_q4_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    const uint8_t* blk = row + (e0 >> 8) * 144;  // 144 = 16 * 9: blocks stay 4-byte aligned when the row is
+    const int r = (int)(e0 & 255);
+    const int c = r >> 6;          // 64-element chunk
+    const int hi = (r >> 5) & 1;   // 0: low nibbles (sub-block 2c), 1: high nibbles (sub-block 2c+1)
+    const int l0 = r & 31;
+    const uint32_t dd = ld_u32(blk);
+    const float d = f16_to_f32((uint16_t)(dd & 0xFFFF));
+    const float dmin = f16_to_f32((uint16_t)(dd >> 16));
+    uint32_t sc, mn;
+    q4k_scale_min(ld_u32(blk + 4), ld_u32(blk + 8), ld_u32(blk + 12), 2 * c + hi, sc, mn);
+    const float D = rnd<NUM>(d * (float)sc);
+    const float DM = rnd<NUM>(dmin * (float)mn);
+    const uint8_t* qs = blk + 16 + 32 * c + l0;
+    const uint32_t q0 = ld_u32(qs), q1 = ld_u32(qs + 4);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t byte = ((i < 4 ? q0 : q1) >> (8 * (i & 3))) & 0xFFu;
+        const float q = (float)(hi ? (byte >> 4) : (byte & 0x0Fu));
+        // fp32: the product is exact, one rounding in the subtraction; fp16 chain: R(R(D*q) - DM)
+        w[i] = rnd<NUM>(rnd<NUM>(D * q) - DM);
+    }
+}
+
+template <int NUM>
+__device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    const uint8_t* blk = row + (e0 >> 8) * 210;
+    const int r = (int)(e0 & 255);
+    const int h = r >> 7;           // 128-element half
+    const int quad = (r >> 5) & 3;  // which of q1..q4
+    const int l0 = r & 31;
+    const uint8_t* ql = blk + 64 * h + 32 * (quad & 1) + l0;
+    const uint8_t* qh = blk + 128 + 32 * h + l0;
+    const int sh_l = 4 * (quad >> 1);
+    const int sh_h = 2 * quad;
+    const float d = f16_to_f32(ld_u16(blk + 208));
+    const int8_t scale = (int8_t)blk[192 + (r >> 4)];
+    const float D = rnd<NUM>(d * (float)scale);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t lo2 = ld_u16(ql + 2 * i), hi2 = ld_u16(qh + 2 * i);
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const uint32_t lb = (lo2 >> (8 * k)) & 0xFFu, hb = (hi2 >> (8 * k)) & 0xFFu;
+            const int q = (int)(((lb >> sh_l) & 0x0Fu) | (((hb >> sh_h) & 3u) << 4)) - 32;
+            w[2 * i + k] = rnd<NUM>(D * (float)q);
+        }
+    }
+}
+
+template <int QT, int NUM>
+__device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    if constexpr (QT == SNGGUF_TYPE_Q8_0) decode8_q8_0<NUM>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode8_q4_k<NUM>(row, e0, w);
+    else decode8_q6_k<NUM>(row, e0, w);
+}
+
+// ---- wavefront sum ---------------------------------------------------------------------------
+// Butterfly over the 64 lanes: four DPP steps inside each row of 16 lanes, then two
+// ds_swizzle/bpermute steps across rows.  Every lane ends with the full sum.
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+}  // namespace sngguf

@@ -1,0 +1,147 @@
+"""GGUF checkpoint loader: the loader half of the drop-in boundary.
+
+Same three functions, signatures, tensor-name mapping (identity) and error behaviour as
+``src/sensenova_u1/utils/gguf_loader.py`` of the reference, with the third-party ``gguf`` /
+``diffusers`` machinery replaced by this package's own reader and ``GGUFLinear``:
+
+    load_gguf_checkpoint(path) -> dict[str, Tensor | GGUFParameter]        (reference :17-47)
+    set_gguf2meta_model(meta_model, state_dict, dtype, device) -> nn.Module (reference :50-85)
+    match_state_dict(meta_model, state_dict, show_num=10) -> dict           (reference :88-114)
+"""
+from __future__ import annotations
+
+import gc
+
+import torch
+from torch import nn
+
+from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader
+from .quantized_linear import (
+    SUPPORTED_GGUF_QUANT_TYPES,
+    GGUFLinear,
+    GGUFParameter,
+    _quant_shape_from_byte_shape,
+    _replace_with_gguf_linear,
+)
+
+
+def load_gguf_checkpoint(gguf_checkpoint_path: str) -> dict:
+    """Parse a .gguf file into a state-dict-compatible mapping.
+
+    F32 / F16 tensors come back as plain torch tensors; every other type must be one the HIP
+    kernels decode and is wrapped in ``GGUFParameter`` (packed bytes, copied out of the file
+    mapping).  Tensor names are used verbatim: GGUF names are the model's state-dict keys.
+    """
+    reader = GGUFReader(gguf_checkpoint_path)
+    parsed: dict = {}
+    try:
+        for tensor in reader.tensors:
+            name = tensor.name
+            quant_type = tensor.tensor_type
+            is_quant = quant_type not in (GGMLQuantizationType.F32, GGMLQuantizationType.F16)
+            if is_quant and quant_type not in SUPPORTED_GGUF_QUANT_TYPES:
+                supported = "\n".join(str(t) for t in SUPPORTED_GGUF_QUANT_TYPES)
+                raise ValueError(f"{name} has unsupported quant type {quant_type!s}.\nSupported:\n{supported}")
+            weights = torch.from_numpy(tensor.data.copy())
+            parsed[name] = GGUFParameter(weights, quant_type=quant_type) if is_quant else weights
+            del tensor, weights
+    finally:
+        reader.close()
+        del reader
+        gc.collect()
+    return parsed
+
+
+def _split_param_name(model: nn.Module, full_name: str):
+    module_path, _, leaf = full_name.rpartition(".")
+    module = model.get_submodule(module_path) if module_path else model
+    return module, leaf
+
+
+def _load_state_dict_into_meta(model: nn.Module, state_dict: dict, dtype: torch.dtype | None, device) -> list[str]:
+    """Place every tensor of ``state_dict`` that the model has a slot for.  Quantized entries
+    keep their bytes and tag (after a shape check against the slot); plain entries are cast to
+    ``dtype`` when they are floating point.  Returns the keys the model had no slot for."""
+    expected = set(model.state_dict().keys())
+    unexpected = []
+    target = torch.device(device) if device is not None else torch.device("cpu")
+    for name, value in state_dict.items():
+        if name not in expected:
+            unexpected.append(name)
+            continue
+        module, leaf = _split_param_name(model, name)
+        is_buffer = leaf in module._buffers
+        slot = module._buffers[leaf] if is_buffer else module._parameters[leaf]
+        if isinstance(value, GGUFParameter):
+            block_size, type_size = GGML_QUANT_SIZES[value.quant_type]
+            inferred = _quant_shape_from_byte_shape(value.shape, type_size, block_size)
+            if slot is not None and tuple(inferred) != tuple(slot.shape):
+                raise ValueError(
+                    f"{name} has an expected quantized shape of: {tuple(inferred)}, but received shape: {tuple(slot.shape)}")
+            placed = value.to(target)
+            if not isinstance(placed, GGUFParameter) or not hasattr(placed, "quant_type"):
+                placed = GGUFParameter(placed, quant_type=value.quant_type)
+            placed.requires_grad_(False)
+            module._parameters[leaf] = placed
+            continue
+        if slot is not None and tuple(value.shape) != tuple(slot.shape):
+            raise ValueError(
+                f"Cannot load {name} because its shape {tuple(value.shape)} does not match the model's "
+                f"{tuple(slot.shape)}")
+        tensor = value.to(device=target, dtype=dtype if (dtype is not None and value.is_floating_point()) else None)
+        if is_buffer:
+            module._buffers[leaf] = tensor
+        else:
+            module._parameters[leaf] = nn.Parameter(tensor, requires_grad=False)
+    return unexpected
+
+
+def set_gguf2meta_model(
+    meta_model: nn.Module,
+    model_state_dict: dict,
+    dtype: torch.dtype,
+    device: torch.device | None,
+) -> nn.Module:
+    """Inject GGUF weights into a meta-initialized model.
+
+    The model must have been built on the meta device (``accelerate.init_empty_weights()`` or
+    ``torch.device("meta")``).  This function:
+      1. replaces every ``nn.Linear`` whose ``<prefix>weight`` is quantized in the dict with
+         ``GGUFLinear(in, out, bias is not None, compute_dtype=dtype or bf16)``;
+      2. loads the parsed state dict into the model on ``device``;
+      3. returns the model cast to ``dtype`` (floating-point, i.e. non-quantized, params only).
+    """
+    compute_dtype = dtype or torch.bfloat16
+    _replace_with_gguf_linear(meta_model, compute_dtype, model_state_dict)
+    _load_state_dict_into_meta(meta_model, model_state_dict, dtype, device)
+    del model_state_dict
+    gc.collect()
+    return meta_model.to(dtype=dtype)
+
+
+def match_state_dict(meta_model: nn.Module, sd: dict, show_num: int = 10) -> dict:
+    """Debug helper: compare the keys of a parsed state dict with the model's.
+
+    Prints a short report and returns ``{"matching": int, "extra": set, "missing": set}``
+    (``extra``: in the file only, ``missing``: in the model only)."""
+    wanted = set(meta_model.state_dict())
+    given = set(sd)
+    report = {"matching": len(wanted & given), "extra": given - wanted, "missing": wanted - given}
+
+    def show(title: str, keys: set, mark: str) -> None:
+        if keys:
+            print(f"[gguf] {title}: {len(keys)}")
+            for key in sorted(keys)[:show_num]:
+                print(f"  {mark} {key}")
+
+    print(f"[gguf] matching keys: {report['matching']}")
+    show("extra in state_dict (not in model)", report["extra"], "+")
+    show("missing in state_dict (in model only)", report["missing"], "-")
+    print(f"[gguf] sample matches: {sorted(wanted & given)[:5]}")
+    return report
+
+
+def count_gguf_linear(model: nn.Module) -> int:
+    """Number of active ``GGUFLinear`` modules, found by type name as the reference's sanity
+    check does (``src/sensenova_u1/utils/checkpoint_loading.py:315``)."""
+    return sum(1 for m in model.modules() if type(m).__name__ == GGUFLinear.__name__)

@@ -1,0 +1,77 @@
+"""Modality-grouped launcher: text rows through the understanding weights, image rows through
+the generation (``_mot_gen``) weights, in one pass over the hidden states.
+
+The reference routes a whole forward to one tower (``Qwen3DecoderLayer.forward``,
+``src/sensenova_u1/models/neo_unify/modeling_qwen3.py:983-1006``) and spells out the mixed
+case only in code below a ``raise`` (``:779-783,802-806,825-829,879-883,1036-1041``):
+
+    out = hidden.new_zeros(...); out[~ind] = proj(hidden[~ind]); out[ind] = proj_mot_gen(hidden[ind])
+
+``grouped_linear`` computes exactly that for a pair of ``GGUFLinear`` modules.  Pairing follows
+the naming rule the offloader uses (``src/sensenova_u1/utils/layer_offload.py:195-222``): the
+generation twin of ``X`` is ``X_mot_gen`` in the same parent module.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .quantized_linear import GGUFLinear
+
+MOT_GEN_SUFFIX = "_mot_gen"
+
+
+def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[torch.Tensor], proj: GGUFLinear,
+                   proj_mot_gen: GGUFLinear, n_text: Optional[int] = None) -> torch.Tensor:
+    """Route rows of ``hidden_states[..., K]`` to ``proj`` (indicator False) or ``proj_mot_gen``
+    (indicator True) in one launch.
+
+    ``image_gen_indicators`` is a bool tensor over the leading dims.  When the layout is known
+    to be ``[text rows | image rows]`` pass ``image_gen_indicators=None`` and ``n_text`` instead:
+    no row map is built and both groups stream contiguous rows.
+    """
+    for mod in (proj, proj_mot_gen):
+        if type(mod).__name__ != "GGUFLinear":
+            raise TypeError(f"grouped_linear needs GGUFLinear modules, got {type(mod).__name__}")
+    if (proj.in_features, proj.out_features) != (proj_mot_gen.in_features, proj_mot_gen.out_features):
+        raise ValueError("understanding and generation projections differ in shape")
+    if image_gen_indicators is None:
+        if n_text is None:
+            raise ValueError("give either image_gen_indicators or n_text")
+        ind, split = None, int(n_text)
+    else:
+        if tuple(image_gen_indicators.shape) != tuple(hidden_states.shape[:-1]):
+            raise ValueError("image_gen_indicators must cover the leading dims of hidden_states")
+        ind, split = image_gen_indicators, 0
+    return ops.grouped_linear(hidden_states, ind, split, proj.weight, int(proj.weight.quant_type),
+                              proj_mot_gen.weight, int(proj_mot_gen.weight.quant_type), proj.bias, proj_mot_gen.bias,
+                              proj.numerics)
+
+
+def find_mot_pairs(module: nn.Module) -> dict[str, tuple[GGUFLinear, GGUFLinear]]:
+    """``{qualified name of X: (X, X_mot_gen)}`` for every GGUFLinear with a generation twin."""
+    pairs = {}
+    for parent_name, parent in module.named_modules():
+        for name, child in parent.named_children():
+            twin = getattr(parent, name + MOT_GEN_SUFFIX, None)
+            if isinstance(child, GGUFLinear) and isinstance(twin, GGUFLinear):
+                pairs[f"{parent_name}.{name}" if parent_name else name] = (child, twin)
+    return pairs
+
+
+def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_proj: GGUFLinear) -> torch.Tensor:
+    """``down_proj(silu(gate_proj(x)) * up_proj(x))`` (``Qwen3MLP.forward``, modeling_qwen3.py:214-216).
+
+    For decode (at most 16 rows, same quant type on gate and up, no bias) the gate and up
+    projections and the SiLU product run as one fused GEMV launch."""
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    same = int(gate_proj.weight.quant_type) == int(up_proj.weight.quant_type)
+    if 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16 \
+            and gate_proj.in_features % 64 == 0:
+        h = ops.gate_up_silu(x, gate_proj.weight, up_proj.weight, int(gate_proj.weight.quant_type), gate_proj.numerics)
+    else:
+        h = torch.nn.functional.silu(gate_proj(x)) * up_proj(x)
+    return down_proj(h)

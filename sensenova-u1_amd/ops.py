@@ -1,0 +1,321 @@
+"""ctypes binding of libsngguf.so and its registration as torch custom ops ``sn_gguf::*``.
+
+The library is the product: there is no CPU implementation behind these ops.  If the shared
+object is missing or a tensor is not on a HIP device the call raises; nothing falls back to
+eager PyTorch arithmetic.
+
+Ops (all launch on the current torch stream of the input's device, never synchronise):
+
+* ``sn_gguf::dequantize(packed, quant_type, out_dtype, numerics) -> Tensor``
+* ``sn_gguf::linear(x, packed, quant_type, bias, numerics) -> Tensor``
+* ``sn_gguf::gate_up_silu(x, gate, up, quant_type, numerics) -> Tensor``
+* ``sn_gguf::grouped_linear(x, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen,
+  bias_und, bias_gen, numerics) -> Tensor``
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libsngguf.so")
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+NUM_GGML_FP32, NUM_UPSTREAM_FP16 = 0, 1
+GGML_QUANT_SIZES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}  # type -> (block elements, block bytes)
+_OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+EXPORTED_SYMBOLS = (
+    "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
+    "sngguf_linear", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+)
+
+_lib = None
+
+
+class SnGgufError(RuntimeError):
+    """A libsngguf entry point returned a negative status."""
+
+
+def load_library() -> ctypes.CDLL:
+    """Load libsngguf.so (once).  Raises if it has not been built: build it with
+    ``python -m sensenova_u1_amd.build`` on a host with hipcc."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise SnGgufError(
+            f"{LIB_PATH} is missing: the HIP library has not been built "
+            "(run `python -m sensenova_u1_amd.build`); there is no CPU fallback for sn_gguf ops")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.sngguf_version.argtypes = []
+    lib.sngguf_version.restype = ci
+    lib.sngguf_strerror.argtypes = [ci]
+    lib.sngguf_strerror.restype = ctypes.c_char_p
+    lib.sngguf_type_size.argtypes = [ci]
+    lib.sngguf_type_size.restype = i64
+    lib.sngguf_block_size.argtypes = [ci]
+    lib.sngguf_block_size.restype = i64
+    lib.sngguf_dequantize.argtypes = [vp, ci, i64, i64, vp, ci, ci, vp]
+    lib.sngguf_dequantize.restype = ci
+    lib.sngguf_linear.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, ci, vp]
+    lib.sngguf_linear.restype = ci
+    lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
+    lib.sngguf_gate_up_silu.restype = ci
+    lib.sngguf_grouped_workspace_bytes.argtypes = [i64]
+    lib.sngguf_grouped_workspace_bytes.restype = i64
+    lib.sngguf_grouped_linear.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, ci, vp]
+    lib.sngguf_grouped_linear.restype = ci
+    _lib = lib
+    return lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load_library().sngguf_strerror(rc).decode()
+        raise SnGgufError(f"{what} failed: {msg} (code {rc})")
+
+
+def _require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise SnGgufError(
+                f"sn_gguf ops run on a HIP device only, got a tensor on '{t.device}'; "
+                "there is no CPU implementation")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise SnGgufError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _packed_2d(packed: torch.Tensor, quant_type: int):
+    """View the packed weight as uint8 [N, row_bytes]; returns (tensor, N, K)."""
+    if quant_type not in GGML_QUANT_SIZES:
+        raise SnGgufError(f"quant type {quant_type} is not implemented (have Q8_0=8, Q4_K=12, Q6_K=14)")
+    bs, ts = GGML_QUANT_SIZES[quant_type]
+    p = packed.detach()
+    if p.dtype != torch.uint8:
+        p = p.view(torch.uint8)
+    if p.dim() != 2:
+        p = p.reshape(-1, p.shape[-1])
+    if not p.is_contiguous():
+        p = p.contiguous()
+    if p.shape[1] % ts != 0:
+        raise SnGgufError(f"packed row of {p.shape[1]} bytes is not a whole number of {ts}-byte blocks")
+    return p, p.shape[0], p.shape[1] // ts * bs
+
+
+# ---- raw entry points (tensor in, tensor out; used by the custom ops and by the bench) --------------
+
+def dequantize_into(packed: torch.Tensor, quant_type: int, out: torch.Tensor, numerics: int) -> None:
+    dev = _require_device(packed, out)
+    p, n, k = _packed_2d(packed, quant_type)
+    if out.numel() != n * k or not out.is_contiguous() or out.dtype not in _OUT_CODE:
+        raise SnGgufError("dequantize: out must be a contiguous fp32/fp16/bf16 tensor of N*K elements")
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_dequantize(_ptr(p), quant_type, n, k, _ptr(out), _OUT_CODE[out.dtype], numerics,
+                                              ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_dequantize")
+
+
+def linear_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],
+                y2d: torch.Tensor, numerics: int) -> None:
+    """y2d[M, N] = x2d[M, K] @ W^T (+ bias); x2d / y2d contiguous bf16, no checks beyond the library's."""
+    dev = x2d.device
+    n, k = y2d.shape[1], x2d.shape[1]
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_linear(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
+                                          _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_linear")
+
+
+def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int, h2d: torch.Tensor,
+                      numerics: int) -> None:
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_gate_up_silu(_ptr(x2d), x2d.shape[0], _ptr(gate), _ptr(up), quant_type,
+                                                h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
+                                                ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_gate_up_silu")
+
+
+def grouped_linear_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, y2d,
+                        workspace, numerics) -> None:
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_grouped_linear(
+            _ptr(x2d), x2d.shape[0], _ptr(indicator), n_text, _ptr(packed_und), qt_und, _ptr(packed_gen), qt_gen,
+            y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), numerics,
+            ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_grouped_linear")
+
+
+def _as_bf16_rows(x: torch.Tensor, k: int, what: str) -> torch.Tensor:
+    if x.dtype != torch.bfloat16:
+        raise SnGgufError(f"{what}: activations must be torch.bfloat16, got {x.dtype}")
+    if x.shape[-1] != k:
+        raise SnGgufError(f"{what}: last dim of the input is {x.shape[-1]}, the weight has in_features={k}")
+    x2d = x.reshape(-1, k)
+    return x2d if x2d.is_contiguous() else x2d.contiguous()
+
+
+def _bias_bf16(bias: Optional[torch.Tensor], n: int, what: str) -> Optional[torch.Tensor]:
+    if bias is None:
+        return None
+    if bias.numel() != n:
+        raise SnGgufError(f"{what}: bias has {bias.numel()} elements, expected {n}")
+    b = bias.detach()
+    if b.dtype != torch.bfloat16:
+        b = b.to(torch.bfloat16)
+    return b.contiguous()
+
+
+# ---- torch custom ops ----------------------------------------------------------------------------------
+
+_torch_lib = torch.library.Library("sn_gguf", "DEF")
+_torch_lib.define("dequantize(Tensor packed, int quant_type, ScalarType out_dtype, int numerics) -> Tensor")
+_torch_lib.define("linear(Tensor x, Tensor packed, int quant_type, Tensor? bias, int numerics) -> Tensor")
+_torch_lib.define("gate_up_silu(Tensor x, Tensor gate, Tensor up, int quant_type, int numerics) -> Tensor")
+_torch_lib.define(
+    "grouped_linear(Tensor x, Tensor? indicator, int n_text, Tensor packed_und, int quant_type_und, "
+    "Tensor packed_gen, int quant_type_gen, Tensor? bias_und, Tensor? bias_gen, int numerics) -> Tensor")
+
+
+def _dequantize_hip(packed, quant_type, out_dtype, numerics):
+    _require_device(packed)
+    p, n, k = _packed_2d(packed, quant_type)
+    out = torch.empty((*packed.shape[:-1], k), dtype=out_dtype, device=packed.device)
+    dequantize_into(p, quant_type, out, numerics)
+    return out
+
+
+def _linear_hip(x, packed, quant_type, bias, numerics):
+    _require_device(x, packed, bias)
+    p, n, k = _packed_2d(packed, quant_type)
+    x2d = _as_bf16_rows(x, k, "linear")
+    y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
+    if y.numel():
+        linear_into(x2d, p, quant_type, _bias_bf16(bias, n, "linear"), y.view(-1, n), numerics)
+    return y
+
+
+def _gate_up_silu_hip(x, gate, up, quant_type, numerics):
+    _require_device(x, gate, up)
+    pg, n, k = _packed_2d(gate, quant_type)
+    pu, n2, k2 = _packed_2d(up, quant_type)
+    if (n, k) != (n2, k2):
+        raise SnGgufError("gate_up_silu: gate and up weights differ in shape")
+    x2d = _as_bf16_rows(x, k, "gate_up_silu")
+    h = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
+    if h.numel():
+        gate_up_silu_into(x2d, pg, pu, quant_type, h.view(-1, n), numerics)
+    return h
+
+
+def _grouped_linear_hip(x, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, numerics):
+    _require_device(x, indicator, packed_und, packed_gen, bias_und, bias_gen)
+    pu, n, k = _packed_2d(packed_und, qt_und)
+    pg, n2, k2 = _packed_2d(packed_gen, qt_gen)
+    if (n, k) != (n2, k2):
+        raise SnGgufError("grouped_linear: the two weight sets differ in shape")
+    x2d = _as_bf16_rows(x, k, "grouped_linear")
+    m = x2d.shape[0]
+    y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
+    if not y.numel():
+        return y
+    ind = ws = None
+    if indicator is not None:
+        if indicator.numel() != m:
+            raise SnGgufError(f"grouped_linear: indicator has {indicator.numel()} entries for {m} rows")
+        ind = indicator.detach().reshape(-1)
+        ind = (ind != 0).to(torch.uint8) if ind.dtype != torch.uint8 else ind.contiguous()
+        ws = torch.empty(load_library().sngguf_grouped_workspace_bytes(m), dtype=torch.uint8, device=x.device)
+    grouped_linear_into(x2d, ind, n_text, pu, qt_und, pg, qt_gen, _bias_bf16(bias_und, n, "grouped_linear"),
+                        _bias_bf16(bias_gen, n, "grouped_linear"), y.view(-1, n), ws, numerics)
+    return y
+
+
+def _no_cpu(*args, **kwargs):
+    raise SnGgufError("sn_gguf ops have no CPU implementation: move the tensors to the MI355X (HIP) device")
+
+
+for _name, _fn in (("dequantize", _dequantize_hip), ("linear", _linear_hip), ("gate_up_silu", _gate_up_silu_hip),
+                   ("grouped_linear", _grouped_linear_hip)):
+    _torch_lib.impl(_name, _fn, "CUDA")  # torch's dispatch key for HIP devices
+    _torch_lib.impl(_name, _no_cpu, "CPU")
+
+
+def _packed_shape(packed, quant_type):
+    bs, ts = GGML_QUANT_SIZES[quant_type]
+    return packed.shape[-1] // ts * bs
+
+
+def _dequantize_meta(packed, quant_type, out_dtype, numerics):
+    return packed.new_empty((*packed.shape[:-1], _packed_shape(packed, quant_type)), dtype=out_dtype)
+
+
+def _linear_meta(x, packed, quant_type, bias, numerics):
+    return x.new_empty((*x.shape[:-1], packed.shape[0]), dtype=torch.bfloat16)
+
+
+def _gate_up_silu_meta(x, gate, up, quant_type, numerics):
+    return x.new_empty((*x.shape[:-1], gate.shape[0]), dtype=torch.bfloat16)
+
+
+def _grouped_linear_meta(x, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, numerics):
+    return x.new_empty((*x.shape[:-1], packed_und.shape[0]), dtype=torch.bfloat16)
+
+
+_torch_lib.impl("dequantize", _dequantize_meta, "Meta")
+_torch_lib.impl("linear", _linear_meta, "Meta")
+_torch_lib.impl("gate_up_silu", _gate_up_silu_meta, "Meta")
+_torch_lib.impl("grouped_linear", _grouped_linear_meta, "Meta")
+
+
+# ---- Python-facing wrappers ----------------------------------------------------------------------------------
+
+def _plain(t):
+    """Strip Parameter subclasses so the dispatcher sees an ordinary tensor."""
+    if t is None:
+        return None
+    return t.as_tensor() if hasattr(t, "as_tensor") else t.detach()
+
+
+def dequantize(packed: torch.Tensor, quant_type: int, out_dtype: torch.dtype = torch.float32,
+               numerics: int = NUM_GGML_FP32) -> torch.Tensor:
+    return torch.ops.sn_gguf.dequantize(_plain(packed), int(quant_type), out_dtype, int(numerics))
+
+
+def linear(x: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor] = None,
+           numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    return torch.ops.sn_gguf.linear(x, _plain(packed), int(quant_type), _plain(bias), int(numerics))
+
+
+def gate_up_silu(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int,
+                 numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    return torch.ops.sn_gguf.gate_up_silu(x, _plain(gate), _plain(up), int(quant_type), int(numerics))
+
+
+def grouped_linear(x: torch.Tensor, indicator: Optional[torch.Tensor], n_text: int, packed_und: torch.Tensor,
+                   quant_type_und: int, packed_gen: torch.Tensor, quant_type_gen: int,
+                   bias_und: Optional[torch.Tensor] = None, bias_gen: Optional[torch.Tensor] = None,
+                   numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    return torch.ops.sn_gguf.grouped_linear(x, _plain(indicator), int(n_text), _plain(packed_und), int(quant_type_und),
+                                            _plain(packed_gen), int(quant_type_gen), _plain(bias_und),
+                                            _plain(bias_gen), int(numerics))

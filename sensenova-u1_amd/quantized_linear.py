@@ -1,0 +1,166 @@
+"""``GGUFParameter`` and ``GGUFLinear``: the module half of the drop-in boundary.
+
+The reference gets both from ``diffusers.quantizers.gguf.utils``
+(``src/sensenova_u1/utils/gguf_loader.py:30,43,64-81``) and recognises the module by its type
+name (``src/sensenova_u1/utils/checkpoint_loading.py:315``).  Same constructor, same
+``forward(inputs)``; the arithmetic behind it is the HIP library, not torch elementwise ops.
+
+``weight`` keeps the GGUF-native bytes ``uint8 [out_features, in_features / block * type_size]``
+and carries ``quant_type`` / ``quant_shape`` on the Parameter object itself, so they survive
+``weight.data = <other storage>`` - which the layer offloader does around every forward
+(``src/sensenova_u1/utils/layer_offload.py:349-356,373-375``).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType
+
+# quant types the HIP kernels decode
+SUPPORTED_GGUF_QUANT_TYPES = (
+    GGMLQuantizationType.Q8_0,
+    GGMLQuantizationType.Q4_K,
+    GGMLQuantizationType.Q6_K,
+)
+
+
+def _quant_shape_from_byte_shape(shape, type_size: int, block_size: int):
+    return (*shape[:-1], shape[-1] // type_size * block_size)
+
+
+class GGUFParameter(torch.nn.Parameter):
+    """uint8 parameter holding packed GGUF blocks, tagged with its ggml type."""
+
+    def __new__(cls, data, requires_grad: bool = False, quant_type=None):
+        if quant_type is None:
+            raise ValueError("GGUFParameter needs a quant_type")
+        data = data if data is not None else torch.empty(0, dtype=torch.uint8)
+        self = torch.Tensor._make_subclass(cls, data, requires_grad)
+        self.quant_type = GGMLQuantizationType(int(quant_type))
+        block_size, type_size = GGML_QUANT_SIZES[self.quant_type]
+        self.quant_shape = _quant_shape_from_byte_shape(self.shape, type_size, block_size)
+        return self
+
+    def as_tensor(self) -> torch.Tensor:
+        """The same storage as a plain tensor (no subclass, no tag)."""
+        return torch.Tensor._make_subclass(torch.Tensor, self, self.requires_grad)
+
+    @staticmethod
+    def _tag_source(args):
+        for a in args:
+            if isinstance(a, GGUFParameter):
+                return a
+            if isinstance(a, (list, tuple)):
+                for b in a:
+                    if isinstance(b, GGUFParameter):
+                        return b
+        return None
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        result = super().__torch_function__(func, types, args, kwargs)
+        # .to() / .cuda() / .pin_memory() / views hand back the subclass without Python attributes
+        src = cls._tag_source(args)
+        if src is None:
+            return result
+
+        def retag(t):
+            if isinstance(t, torch.Tensor) and t.dtype == torch.uint8 and t.dim() >= 1 and not hasattr(t, "quant_type"):
+                _, ts = GGML_QUANT_SIZES[src.quant_type]
+                if t.shape[-1] % ts == 0:
+                    if not isinstance(t, GGUFParameter):
+                        t = torch.Tensor._make_subclass(cls, t, False)
+                    t.quant_type = src.quant_type
+                    t.quant_shape = _quant_shape_from_byte_shape(t.shape, ts, GGML_QUANT_SIZES[src.quant_type][0])
+            return t
+
+        if isinstance(result, torch.Tensor):
+            return retag(result)
+        if isinstance(result, (tuple, list)):
+            return type(result)(retag(r) for r in result)
+        return result
+
+    def __reduce_ex__(self, proto):
+        return (_rebuild_gguf_parameter, (self.as_tensor().detach(), int(self.quant_type)))
+
+
+def _rebuild_gguf_parameter(data, quant_type):
+    return GGUFParameter(data, quant_type=quant_type)
+
+
+def dequantize_gguf_tensor(tensor: torch.Tensor, dtype: Optional[torch.dtype] = None,
+                           numerics: int = ops.NUM_UPSTREAM_FP16) -> torch.Tensor:
+    """Packed parameter -> dense ``quant_shape`` tensor on the same (HIP) device.
+
+    With the default numerics the result is the fp16 tensor the reference's
+    ``dequantize_gguf_tensor`` returns; ``numerics=ops.NUM_GGML_FP32`` gives ggml's exact fp32
+    values.  Tensors without a ``quant_type`` pass through unchanged, as upstream does.
+    """
+    if not hasattr(tensor, "quant_type"):
+        return tensor
+    if dtype is None:
+        dtype = torch.float16 if numerics == ops.NUM_UPSTREAM_FP16 else torch.float32
+    return ops.dequantize(tensor, int(tensor.quant_type), dtype, numerics)
+
+
+class GGUFLinear(nn.Linear):
+    """``nn.Linear`` whose weight is a :class:`GGUFParameter`.
+
+    ``forward`` computes ``F.linear(x, dequantize(weight).to(compute_dtype), bias)`` with the
+    reference's rounding chain, through the fused HIP kernels when ``compute_dtype`` is bf16
+    (GEMV for up to 16 rows, MFMA GEMM above), or through the HIP dequantize op followed by the
+    device matmul for other compute dtypes.
+    """
+
+    numerics: int = ops.NUM_UPSTREAM_FP16
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = False,
+                 compute_dtype: Optional[torch.dtype] = None, device=None) -> None:
+        super().__init__(in_features, out_features, bias, device)
+        self.compute_dtype = compute_dtype
+
+    def _weight_type(self) -> int:
+        w = self.weight
+        if not hasattr(w, "quant_type"):
+            raise RuntimeError("GGUFLinear.weight is not a GGUFParameter (no quant_type); was the checkpoint loaded?")
+        return int(w.quant_type)
+
+    def forward(self, inputs: torch.Tensor) -> torch.Tensor:
+        qtype = self._weight_type()
+        compute_dtype = self.compute_dtype or inputs.dtype
+        if inputs.dtype != compute_dtype:
+            raise RuntimeError(f"GGUFLinear: input dtype {inputs.dtype} does not match compute dtype {compute_dtype}")
+        if compute_dtype == torch.bfloat16:
+            return ops.linear(inputs, self.weight, qtype, self.bias, self.numerics)
+        weight = ops.dequantize(self.weight, qtype, torch.float16 if self.numerics == ops.NUM_UPSTREAM_FP16
+                                else torch.float32, self.numerics).to(compute_dtype)
+        bias = self.bias.to(compute_dtype) if self.bias is not None else None
+        return torch.nn.functional.linear(inputs, weight, bias)
+
+    def extra_repr(self) -> str:
+        qt = getattr(self.weight, "quant_type", None)
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"quant_type={qt.name if qt is not None else None}, compute_dtype={self.compute_dtype}")
+
+
+def _replace_with_gguf_linear(model: nn.Module, compute_dtype, state_dict: dict, prefix: str = "",
+                              modules_to_not_convert=()) -> nn.Module:
+    """Swap every ``nn.Linear`` whose ``<prefix>weight`` entry of ``state_dict`` is a
+    :class:`GGUFParameter` for a :class:`GGUFLinear` built on the meta device."""
+    for name, module in list(model.named_children()):
+        module_prefix = f"{prefix}{name}."
+        _replace_with_gguf_linear(module, compute_dtype, state_dict, module_prefix, modules_to_not_convert)
+        if isinstance(module, nn.Linear) and not isinstance(module, GGUFLinear) and name not in modules_to_not_convert:
+            if isinstance(state_dict.get(module_prefix + "weight"), GGUFParameter):
+                with torch.device("meta"):
+                    new = GGUFLinear(module.in_features, module.out_features, module.bias is not None,
+                                     compute_dtype=compute_dtype)
+                new.source_cls = type(module)
+                new.requires_grad_(False)
+                model._modules[name] = new
+    return model
