@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-linear hot path on one MI355X.
+
+Headline leg (``value``): the Q8_0 SiLU-gated MLP of one decoder layer at decode, M = 1
+(gate / up 4096 -> 12288, down 12288 -> 4096).  One *step* is one pass of that MLP over one
+layer's packed weights; consecutive steps walk over ``--layers`` distinct weight sets (default
+16 x 160 MB = 2.6 GB, far beyond the 256 MB last-level cache), so every step streams its
+weights from HBM.  ``value`` is algorithmic bytes per step / wall time per step.
+
+Further legs in the same JSON line: the same MLP at M = 4 and 16, and the M = 4096 Q8_0
+generation-tower projections (q, k, v, o, gate, up, down of one tower-layer) on the MFMA GEMM,
+reported in TFLOP/s.  ``roofline`` belongs to the dominant kernel of the headline leg (the fused
+gate/up GEMV), timed alone with HIP events; ``gemm.roofline`` to the largest GEMM (gate shape).
+``cpu_baseline`` times the CPU oracle's port of the reference forward on the host cores.
+
+All inputs are synthetic, seeded, resident in HBM before the timed region starts.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HIDDEN, INTER, KV = 4096, 12288, 1024
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+Q8_0 = 8
+
+
+def q8_bytes(n: int, k: int) -> int:
+    return n * (k // 32) * 34
+
+
+def linear_bytes(m: int, n: int, k: int) -> int:
+    """Algorithmic bytes of one quantized linear: packed weight once, bf16 x once, bf16 y once."""
+    return q8_bytes(n, k) + 2 * m * k + 2 * m * n
+
+
+def mlp_bytes(m: int) -> int:
+    return 2 * linear_bytes(m, INTER, HIDDEN) + linear_bytes(m, HIDDEN, INTER)
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=512)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--layers", type=int, default=16, help="distinct MLP weight sets the steps rotate over")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--gemm-steps", type=int, default=3)
+    ap.add_argument("--numerics", type=int, default=1, help="1 = upstream fp16 chain (drop-in), 0 = ggml fp32")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(the path shards by output rows, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from sensenova_u1_amd import ops, synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device", file=sys.stderr)
+        sys.exit(1)
+    ops.load_library()
+    dev = torch.device("cuda:0")
+    num = args.numerics
+    K, W, L = args.steps, args.warmup, args.layers
+
+    # ---- synthetic weights, resident in HBM --------------------------------------------------
+    layers = []
+    for i in range(L):
+        layers.append((synthetic.make_packed(Q8_0, INTER, HIDDEN, seed=1000 + 3 * i, device=dev),
+                       synthetic.make_packed(Q8_0, INTER, HIDDEN, seed=1001 + 3 * i, device=dev),
+                       synthetic.make_packed(Q8_0, HIDDEN, INTER, seed=1002 + 3 * i, device=dev)))
+    torch.cuda.synchronize()
+
+    def run_region(fn, n_steps: int, warmup: int):
+        """W warm-up steps, then exactly n_steps steps timed (wall clock around a synchronised
+        region, and HIP events on the launch stream).  Returns (wall_ms, event_ms)."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        graph = None
+        if not args.no_graph:
+            try:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for i in range(n_steps):
+                        fn(warmup + i)
+            except Exception as exc:  # capture unsupported: time eager launches instead
+                print(f"bench.py: graph capture failed ({exc}); timing eager launches", file=sys.stderr)
+                graph = None
+                torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(n_steps):
+                fn(warmup + i)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) * 1e3, e0.elapsed_time(e1)
+
+    def mlp_leg(m: int, n_steps: int, warmup: int):
+        x = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
+        h = torch.empty((m, INTER), dtype=torch.bfloat16, device=dev)
+        y = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
+
+        def step(i):
+            gate, up, down = layers[i % L]
+            ops.gate_up_silu_into(x, gate, up, Q8_0, h, num)
+            ops.linear_into(h, down, Q8_0, None, y, num)
+
+        def gate_up_only(i):
+            gate, up, _ = layers[i % L]
+            ops.gate_up_silu_into(x, gate, up, Q8_0, h, num)
+
+        def down_only(i):
+            ops.linear_into(h, layers[i % L][2], Q8_0, None, y, num)
+
+        wall, ev = run_region(step, n_steps, warmup)
+        _, ev_gu = run_region(gate_up_only, n_steps, warmup)
+        _, ev_dn = run_region(down_only, n_steps, warmup)
+        return wall, ev, ev_gu / n_steps, ev_dn / n_steps
+
+    wall1, ev1, gu_ms, dn_ms = mlp_leg(1, K, W)
+    step_bytes = mlp_bytes(1)
+    ms_per_step = wall1 / K
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    gu_bytes = 2 * linear_bytes(1, INTER, HIDDEN)
+    gu_gbps = gu_bytes / (gu_ms * 1e-3) / 1e9
+    dn_bytes = linear_bytes(1, HIDDEN, INTER)
+
+    result = {
+        "metric": "Q8_0 dequant-GEMV HBM GB/s (% of peak); M=4096 dequant-GEMM TFLOP/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: Q8_0 MLP of one decoder layer, text decode M=1 "
+                        "(gate/up 4096->12288 fused with SiLU, down 12288->4096)",
+            "layers_rotated": L,
+            "bytes_per_step": step_bytes,
+            "graph": not args.no_graph,
+            "numerics": "upstream_fp16" if num == 1 else "ggml_fp32",
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "device_ms_per_step": round(ev1 / K, 6),
+        "roofline": {
+            "kernel": "gemv_kernel<Q8_0, gated> (fused gate/up + SiLU, M=1)",
+            "bound": "hbm",
+            "achieved": round(gu_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gu_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": gu_bytes,
+            "avg_launch_us": round(gu_ms * 1e3, 3),
+        },
+        "down_proj": {
+            "kernel": "gemv_kernel<Q8_0> (down 12288->4096, M=1)",
+            "achieved": round(dn_bytes / (dn_ms * 1e-3) / 1e9, 1),
+            "unit": "GB/s",
+            "avg_launch_us": round(dn_ms * 1e3, 3),
+        },
+    }
+
+    # ---- same MLP at M = 4 and 16 --------------------------------------------------------------
+    decode = {}
+    for m in (4, 16):
+        k2 = max(64, K // 4)
+        wall, ev, gu, dn = mlp_leg(m, k2, min(W, 16))
+        gbps = mlp_bytes(m) / (wall / k2 * 1e-3) / 1e9
+        decode[f"M{m}"] = {"value": round(gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
+                           "ms_per_step": round(wall / k2, 6), "gate_up_us": round(gu * 1e3, 3),
+                           "down_us": round(dn * 1e3, 3)}
+    result["decode_other_M"] = decode
+
+    # ---- M = 4096 generation-tower projections on the MFMA GEMM ----------------------------------
+    if not args.no_gemm:
+        m = 4096
+        shapes = [("q", HIDDEN, HIDDEN), ("k", KV, HIDDEN), ("v", KV, HIDDEN), ("o", HIDDEN, HIDDEN),
+                  ("gate", INTER, HIDDEN), ("up", INTER, HIDDEN), ("down", HIDDEN, INTER)]
+        tower = [[synthetic.make_packed(Q8_0, n, k, seed=5000 + 10 * r + j, device=dev) for j, (_, n, k) in enumerate(shapes)]
+                 for r in range(2)]
+        xs = {k: synthetic.make_activations(m, k, seed=k, device=dev) for k in (HIDDEN, INTER)}
+        ys = {n: torch.empty((m, n), dtype=torch.bfloat16, device=dev) for n in (HIDDEN, KV, INTER)}
+
+        def tower_step(i):
+            ws = tower[i % 2]
+            for j, (_, n, k) in enumerate(shapes):
+                ops.linear_into(xs[k], ws[j], Q8_0, None, ys[n], num)
+
+        def gate_only(i):
+            ops.linear_into(xs[HIDDEN], tower[i % 2][4], Q8_0, None, ys[INTER], num)
+
+        gs = args.gemm_steps
+        wall, ev = run_region(tower_step, gs, 1)
+        flops = sum(2.0 * m * n * k for _, n, k in shapes)
+        tflops = flops / (wall / gs * 1e-3) / 1e12
+        _, ev_gate = run_region(gate_only, gs * 2, 1)
+        gate_ms = ev_gate / (gs * 2)
+        gate_tflops = 2.0 * m * INTER * HIDDEN / (gate_ms * 1e-3) / 1e12
+        result["gemm"] = {
+            "workload": "configs[2]: Q8_0 generation-tower projections over M=4096 image tokens "
+                        "(q,o 4096^2; k,v 4096->1024; gate/up 4096->12288; down 12288->4096)",
+            "value": round(tflops, 2),
+            "unit": "TFLOP/s",
+            "steps": gs,
+            "ms_per_step": round(wall / gs, 4),
+            "flop_per_step": flops,
+            "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+            "roofline": {
+                "kernel": "gemm_kernel<Q8_0> (gate 4096->12288, M=4096)",
+                "bound": "mfma",
+                "achieved": round(gate_tflops, 2),
+                "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s",
+                "frac": round(gate_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                "traffic": None,
+                "avg_launch_us": round(gate_ms * 1e3, 2),
+            },
+        }
+        del tower, xs, ys
+
+    # ---- CPU baseline: the oracle's port of GGUFLinear.forward_native on the host cores -----------
+    if not args.no_cpu_baseline:
+        from oracle import gguf_oracle as go
+
+        gate, up, down = (t.cpu() for t in layers[0])
+        x = synthetic.make_activations(1, HIDDEN, seed=7)
+        reps, times = 3, []
+        go.mlp_forward(x, gate[:256], up[:256], down[:, :256 // 32 * 34], (Q8_0, Q8_0, Q8_0))  # warm torch's thread pool
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            go.mlp_forward(x, gate, up, down, (Q8_0, Q8_0, Q8_0))
+            times.append(time.perf_counter() - t0)
+        med = sorted(times)[len(times) // 2]
+        result["cpu_baseline"] = {
+            "value": round(step_bytes / med / 1e9, 3),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"median of {reps} full M=1 MLP steps (one layer, {step_bytes} algorithmic bytes each): torch-CPU "
+                      "block decode -> bf16 cast -> F.linear, as GGUFLinear.forward_native does",
+            "ms_per_step": round(med * 1e3, 2),
+            "host_cpus": os.cpu_count(),
+        }
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

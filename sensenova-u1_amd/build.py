@@ -20,6 +20,8 @@ SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemm.hip"]
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIP_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall",
+    # no fused multiply-add unless written as one: the fp16 decode chain rounds after every op
+    "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 

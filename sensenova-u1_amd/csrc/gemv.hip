@@ -27,11 +27,26 @@ __device__ __forceinline__ int64_t unit_run_offset(int64_t u, int t) {
     }
 }
 
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
 template <int NUM>
-__device__ __forceinline__ uint32_t q8_pair(float d, uint32_t two) {  // two int8 in the low half
-    const float a = rnd<NUM>(d * (float)(int8_t)(two & 0xFF));
-    const float b = rnd<NUM>(d * (float)(int8_t)((two >> 8) & 0xFF));
-    return pack_bf16(a, b);
+__device__ __forceinline__ void q8_dword(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
+        const uint32_t u = dw ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
+        const half2_t d2 = {d, d};
+        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
+        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        const float d = f16_to_f32(d_bits);
+        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
+        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
+    }
 }
 
 template <int NUM>
@@ -44,33 +59,29 @@ __device__ __forceinline__ void decode_unit_q8_0(const uint8_t* __restrict__ row
         L[4 * i] = v[0]; L[4 * i + 1] = v[1]; L[4 * i + 2] = v[2]; L[4 * i + 3] = v[3];
     }
     L[16] = ld_u32(p + 64);
-    const float d0 = f16_to_f32((uint16_t)(L[0] & 0xFFFF));
-    const float d1 = f16_to_f32((uint16_t)(L[8] >> 16));
+    const uint16_t d0 = (uint16_t)(L[0] & 0xFFFF), d1 = (uint16_t)(L[8] >> 16);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const uint32_t q0 = __builtin_amdgcn_alignbit(L[i + 1], L[i], 16);  // block 0 quants sit 2 bytes off
-        wp[2 * i] = q8_pair<NUM>(d0, q0);
-        wp[2 * i + 1] = q8_pair<NUM>(d0, q0 >> 16);
-        const uint32_t q1 = L[9 + i];
-        wp[16 + 2 * i] = q8_pair<NUM>(d1, q1);
-        wp[16 + 2 * i + 1] = q8_pair<NUM>(d1, q1 >> 16);
+        q8_dword<NUM>(d0, q0, wp[2 * i], wp[2 * i + 1]);
+        q8_dword<NUM>(d1, L[9 + i], wp[16 + 2 * i], wp[16 + 2 * i + 1]);
     }
 }
 
 template <int NUM>
 __device__ __forceinline__ void decode_unit_q4_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    typedef Num<NUM> A;
     const uint8_t* blk = row + (u >> 2) * 144;
     const int c = (int)u & 3;
     const u32x4_t hdr = *reinterpret_cast<const u32x4_t*>(blk);
     const u32x4_t qa = *reinterpret_cast<const u32x4_t*>(blk + 16 + 32 * c);
     const u32x4_t qb = *reinterpret_cast<const u32x4_t*>(blk + 32 + 32 * c);
-    const float d = f16_to_f32((uint16_t)(hdr[0] & 0xFFFF));
-    const float dmin = f16_to_f32((uint16_t)(hdr[0] >> 16));
+    const typename A::T d = A::scale((uint16_t)(hdr[0] & 0xFFFF)), dmin = A::scale((uint16_t)(hdr[0] >> 16));
     uint32_t sc0, mn0, sc1, mn1;
     q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c, sc0, mn0);
     q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c + 1, sc1, mn1);
-    const float D0 = rnd<NUM>(d * (float)sc0), M0 = rnd<NUM>(dmin * (float)mn0);
-    const float D1 = rnd<NUM>(d * (float)sc1), M1 = rnd<NUM>(dmin * (float)mn1);
+    const typename A::T D0 = d * A::integer((int)sc0), M0 = dmin * A::integer((int)mn0);
+    const typename A::T D1 = d * A::integer((int)sc1), M1 = dmin * A::integer((int)mn1);
 #pragma unroll
     for (int i = 0; i < 8; i++) {  // dword i of the 32 quant bytes: elements 4i..4i+3 (low) and 32+4i.. (high)
         const uint32_t q = i < 4 ? qa[i] : qb[i - 4];
@@ -78,8 +89,8 @@ __device__ __forceinline__ void decode_unit_q4_k(const uint8_t* __restrict__ row
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const uint32_t byte = (q >> (8 * k)) & 0xFFu;
-            lo[k] = rnd<NUM>(rnd<NUM>(D0 * (float)(byte & 0x0Fu)) - M0);
-            hi[k] = rnd<NUM>(rnd<NUM>(D1 * (float)(byte >> 4)) - M1);
+            lo[k] = A::widen(D0 * A::integer((int)(byte & 0x0Fu)) - M0);
+            hi[k] = A::widen(D1 * A::integer((int)(byte >> 4)) - M1);
         }
         wp[2 * i] = pack_bf16(lo[0], lo[1]);
         wp[2 * i + 1] = pack_bf16(lo[2], lo[3]);
@@ -90,15 +101,16 @@ __device__ __forceinline__ void decode_unit_q4_k(const uint8_t* __restrict__ row
 
 template <int NUM>
 __device__ __forceinline__ void decode_unit_q6_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
+    typedef Num<NUM> A;
     const uint8_t* blk = row + (u >> 2) * 210;  // 2-byte aligned
     const int h = (int)(u >> 1) & 1, j = (int)u & 1;
     const u32x4_t la = ld_u128_a2(blk + 64 * h + 16 * j);        // ql[l], l = 16j..16j+15
     const u32x4_t lb = ld_u128_a2(blk + 64 * h + 32 + 16 * j);   // ql[l + 32]
     const u32x4_t hh = ld_u128_a2(blk + 128 + 32 * h + 16 * j);  // qh[l]
-    const float d = f16_to_f32(ld_u16(blk + 208));
-    float D[4];
+    const typename A::T d = A::scale(ld_u16(blk + 208));
+    typename A::T D[4];
 #pragma unroll
-    for (int t = 0; t < 4; t++) D[t] = rnd<NUM>(d * (float)(int8_t)blk[192 + 8 * h + j + 2 * t]);
+    for (int t = 0; t < 4; t++) D[t] = d * A::integer((int8_t)blk[192 + 8 * h + j + 2 * t]);
 #pragma unroll
     for (int i = 0; i < 4; i++) {  // dword i: l = 16j + 4i .. +3
         float v[4][4];
@@ -109,10 +121,10 @@ __device__ __forceinline__ void decode_unit_q6_k(const uint8_t* __restrict__ row
             const int q2 = (int)((b & 0x0Fu) | (((c >> 2) & 3u) << 4)) - 32;
             const int q3 = (int)((a >> 4) | (((c >> 4) & 3u) << 4)) - 32;
             const int q4 = (int)((b >> 4) | (((c >> 6) & 3u) << 4)) - 32;
-            v[0][k] = rnd<NUM>(D[0] * (float)q1);
-            v[1][k] = rnd<NUM>(D[1] * (float)q2);
-            v[2][k] = rnd<NUM>(D[2] * (float)q3);
-            v[3][k] = rnd<NUM>(D[3] * (float)q4);
+            v[0][k] = A::widen(D[0] * A::integer(q1));
+            v[1][k] = A::widen(D[1] * A::integer(q2));
+            v[2][k] = A::widen(D[2] * A::integer(q3));
+            v[3][k] = A::widen(D[3] * A::integer(q4));
         }
 #pragma unroll
         for (int t = 0; t < 4; t++) {

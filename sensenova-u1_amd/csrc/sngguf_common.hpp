@@ -39,12 +39,26 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// NUM == SNGGUF_NUM_UPSTREAM_FP16: the value is an fp16 tensor element; else exact fp32.
-template <int NUM>
-__device__ __forceinline__ float rnd(float v) {
-    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) return round_f16(v);
-    return v;
-}
+// Arithmetic of the block decode.  Num<SNGGUF_NUM_GGML_FP32> works in fp32, where every product
+// of the three formats is exact.  Num<SNGGUF_NUM_UPSTREAM_FP16> works in native fp16
+// (v_mul_f16 / v_sub_f16, round-to-nearest-even, subnormals and signed zeros kept): each
+// upstream tensor op is "compute in fp32, round to fp16", and because the operands are fp16
+// values or small integers the exact result fits fp32, so the single fp16 rounding of the
+// native instruction gives the same bits.  The library is compiled with -ffp-contract=off so
+// that no two of these roundings are fused.
+template <int NUM> struct Num;
+template <> struct Num<SNGGUF_NUM_GGML_FP32> {
+    typedef float T;
+    static __device__ __forceinline__ T scale(uint16_t f16_bits) { return f16_to_f32(f16_bits); }
+    static __device__ __forceinline__ T integer(int q) { return (float)q; }
+    static __device__ __forceinline__ float widen(T v) { return v; }
+};
+template <> struct Num<SNGGUF_NUM_UPSTREAM_FP16> {
+    typedef _Float16 T;
+    static __device__ __forceinline__ T scale(uint16_t f16_bits) { return __builtin_bit_cast(_Float16, f16_bits); }
+    static __device__ __forceinline__ T integer(int q) { return (_Float16)(short)q; }  // |q| <= 2048: exact
+    static __device__ __forceinline__ float widen(T v) { return (float)v; }
+};
 
 // ---- unaligned loads ----------------------------------------------------------------------
 // GGUF blocks are only 2-byte aligned (34- and 210-byte blocks).  memcpy from a pointer of
@@ -102,44 +116,45 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t
 
 template <int NUM>
 __device__ __forceinline__ void decode8_q8_0(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
     const uint8_t* blk = row + (e0 >> 5) * 34;
-    const float d = f16_to_f32(ld_u16(blk));
+    const typename A::T d = A::scale(ld_u16(blk));
     const uint8_t* qs = blk + 2 + (e0 & 31);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t h = ld_u16(qs + 2 * i);
-        w[2 * i] = rnd<NUM>(d * (float)(int8_t)(h & 0xFF));
-        w[2 * i + 1] = rnd<NUM>(d * (float)(int8_t)(h >> 8));
+        w[2 * i] = A::widen(d * A::integer((int8_t)(h & 0xFF)));
+        w[2 * i + 1] = A::widen(d * A::integer((int8_t)(h >> 8)));
     }
 }
 
 template <int NUM>
 __device__ __forceinline__ void decode8_q4_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
     const uint8_t* blk = row + (e0 >> 8) * 144;  // 144 = 16 * 9: blocks stay 4-byte aligned when the row is
     const int r = (int)(e0 & 255);
     const int c = r >> 6;          // 64-element chunk
     const int hi = (r >> 5) & 1;   // 0: low nibbles (sub-block 2c), 1: high nibbles (sub-block 2c+1)
     const int l0 = r & 31;
     const uint32_t dd = ld_u32(blk);
-    const float d = f16_to_f32((uint16_t)(dd & 0xFFFF));
-    const float dmin = f16_to_f32((uint16_t)(dd >> 16));
     uint32_t sc, mn;
     q4k_scale_min(ld_u32(blk + 4), ld_u32(blk + 8), ld_u32(blk + 12), 2 * c + hi, sc, mn);
-    const float D = rnd<NUM>(d * (float)sc);
-    const float DM = rnd<NUM>(dmin * (float)mn);
+    const typename A::T D = A::scale((uint16_t)(dd & 0xFFFF)) * A::integer((int)sc);
+    const typename A::T DM = A::scale((uint16_t)(dd >> 16)) * A::integer((int)mn);
     const uint8_t* qs = blk + 16 + 32 * c + l0;
     const uint32_t q0 = ld_u32(qs), q1 = ld_u32(qs + 4);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const uint32_t byte = ((i < 4 ? q0 : q1) >> (8 * (i & 3))) & 0xFFu;
-        const float q = (float)(hi ? (byte >> 4) : (byte & 0x0Fu));
-        // fp32: the product is exact, one rounding in the subtraction; fp16 chain: R(R(D*q) - DM)
-        w[i] = rnd<NUM>(rnd<NUM>(D * q) - DM);
+        const int q = (int)(hi ? (byte >> 4) : (byte & 0x0Fu));
+        // fp32: both products exact, one rounding in the subtraction; fp16: R(R(D*q) - DM)
+        w[i] = A::widen(D * A::integer(q) - DM);
     }
 }
 
 template <int NUM>
 __device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
     const uint8_t* blk = row + (e0 >> 8) * 210;
     const int r = (int)(e0 & 255);
     const int h = r >> 7;           // 128-element half
@@ -149,9 +164,7 @@ __device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, in
     const uint8_t* qh = blk + 128 + 32 * h + l0;
     const int sh_l = 4 * (quad >> 1);
     const int sh_h = 2 * quad;
-    const float d = f16_to_f32(ld_u16(blk + 208));
-    const int8_t scale = (int8_t)blk[192 + (r >> 4)];
-    const float D = rnd<NUM>(d * (float)scale);
+    const typename A::T D = A::scale(ld_u16(blk + 208)) * A::integer((int8_t)blk[192 + (r >> 4)]);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t lo2 = ld_u16(ql + 2 * i), hi2 = ld_u16(qh + 2 * i);
@@ -159,7 +172,7 @@ __device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, in
         for (int k = 0; k < 2; k++) {
             const uint32_t lb = (lo2 >> (8 * k)) & 0xFFu, hb = (hi2 >> (8 * k)) & 0xFFu;
             const int q = (int)(((lb >> sh_l) & 0x0Fu) | (((hb >> sh_h) & 3u) << 4)) - 32;
-            w[2 * i + k] = rnd<NUM>(D * (float)q);
+            w[2 * i + k] = A::widen(D * A::integer(q));
         }
     }
 }

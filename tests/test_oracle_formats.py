@@ -1,0 +1,286 @@
+"""Pins the CPU oracle without the (absent) upstream packages.
+
+Each check is chosen so that one plausible decoder mistake fails it: a wrong element order
+(one-hot blocks), a wrong nibble / high-bit shift (one-hot + packer round trip), a wrong
+scale index or a dropped high scale bit (scale-packing cases), a dropped min term or wrong
+sign (closed form), a sloppy fp16 / bf16 rounding (exhaustive conversion tables).
+The packers in oracle.gguf_oracle are written from the *quantize* side of the format and
+share no code with either decoder.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as go
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+TYPES = [go.Q8_0, go.Q4_K, go.Q6_K]
+
+
+def _blocks(raw: bytes) -> torch.Tensor:
+    return torch.frombuffer(bytearray(raw), dtype=torch.uint8).reshape(1, -1)
+
+
+def _both(c_oracle, packed, qt, numerics=0):
+    a = c_oracle.dequantize(packed, qt, torch.float32, numerics)
+    b = go.dequantize_gguf_tensor(packed, qt, numerics).float()
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), "C and torch restatements disagree"
+    return a.flatten()
+
+
+# ---- scalar conversions -------------------------------------------------------------------
+
+def test_f16_to_f32_exhaustive(c_oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([c_oracle.lib.sno_f16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_f32_to_f16_rne_against_numpy(c_oracle):
+    rng = np.random.default_rng(0)
+    # every half value, every midpoint between neighbouring halves, and just off the midpoints
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = (h[:-1] + h[1:]) / 2
+    cases = np.concatenate([h, mids, np.nextafter(mids.astype(np.float32), np.float32(np.inf)).astype(np.float64),
+                            np.nextafter(mids.astype(np.float32), np.float32(-np.inf)).astype(np.float64),
+                            [65504.0, 65519.99, 65520.0, 65536.0, 1e-8, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 0.0],
+                            rng.standard_normal(20000) * 10.0 ** rng.integers(-9, 5, 20000)]).astype(np.float32)
+    cases = np.concatenate([cases, -cases])
+    with np.errstate(over="ignore"):
+        want = cases.astype(np.float16).view(np.uint16)
+    got = np.array([c_oracle.lib.sno_f32_to_f16(float(v)) for v in cases], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_f32_to_bf16_rne_against_torch(c_oracle):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(50000, generator=g) * torch.pow(10.0, torch.randint(-8, 8, (50000,), generator=g).float())
+    ties = (torch.arange(1, 2000, dtype=torch.int32) << 16 | 0x8000).view(torch.float32)  # exact midpoints
+    x = torch.cat([x, ties, -ties, torch.tensor([0.0, -0.0, 3.3895e38])])
+    want = x.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([c_oracle.lib.sno_f32_to_bf16(float(v)) for v in x.tolist()], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---- Q8_0 ------------------------------------------------------------------------------------
+
+def test_q8_0_one_hot_positions(c_oracle):
+    for pos in range(32):
+        qs = np.zeros(32, dtype=np.int8)
+        qs[pos] = -3
+        out = _both(c_oracle, _blocks(go.pack_q8_0(0.5, qs)), go.Q8_0)
+        want = torch.zeros(32)
+        want[pos] = -1.5
+        assert torch.equal(out, want)
+
+
+def test_q8_0_closed_form_and_extremes(c_oracle):
+    rng = np.random.default_rng(2)
+    for d in (1.0, 6.1035e-05, 5.96e-08, 65504.0, 0.0, -2.5, 0.00015):
+        qs = rng.integers(-128, 128, 32).astype(np.int8)
+        qs[0], qs[1] = -128, 127
+        out = _both(c_oracle, _blocks(go.pack_q8_0(d, qs)), go.Q8_0)
+        want = np.float32(np.float16(d)) * qs.astype(np.float32)   # exact in fp32 (<= 19 significant bits)
+        assert np.array_equal(out.numpy(), want)
+        assert np.array_equal(want.astype(np.float64), np.float64(np.float16(d)) * qs.astype(np.float64))
+
+
+def test_q8_0_quantizer_round_trip(c_oracle):
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((8, 256)) * 0.02).astype(np.float32)
+    packed = torch.from_numpy(go.quantize_q8_0(w))
+    deq = c_oracle.dequantize(packed, go.Q8_0, torch.float32, 0).numpy()
+    d = packed.view(8, -1, 34)[..., :2].contiguous().view(torch.float16).float().numpy().repeat(32, axis=-1).reshape(8, 256)
+    # |x - d*round(x/d)| <= d/2, plus the fp16 rounding of d itself (relative 2^-11 on |x| <= 127 d)
+    assert np.all(np.abs(deq - w) <= d * (0.5 + 127 * 2.0 ** -11) + 1e-12)
+    assert np.abs(deq - w).max() > 0
+
+
+# ---- Q4_K ------------------------------------------------------------------------------------
+
+def test_q4_k_one_hot_positions(c_oracle):
+    sc, mn = [1] * 8, [0] * 8
+    for pos in list(range(0, 256, 7)) + [31, 32, 63, 64, 255]:
+        q = [0] * 256
+        q[pos] = 9
+        out = _both(c_oracle, _blocks(go.pack_q4_k(1.0, 0.0, sc, mn, q)), go.Q4_K)
+        want = torch.zeros(256)
+        want[pos] = 9.0
+        assert torch.equal(out, want), pos
+
+
+def test_q4_k_scale_packing(c_oracle):
+    """Eight distinct scales and mins, including values > 15 and > 31 (the split high bits)."""
+    sc = [1, 17, 33, 63, 2, 18, 47, 62]
+    mn = [63, 5, 21, 40, 59, 3, 16, 32]
+    q = [(7 * i + 3) % 16 for i in range(256)]
+    out = _both(c_oracle, _blocks(go.pack_q4_k(2.0, 0.5, sc, mn, q)), go.Q4_K).numpy()
+    want = np.array([2.0 * sc[i // 32] * q[i] - 0.5 * mn[i // 32] for i in range(256)], dtype=np.float32)
+    assert np.array_equal(out, want)
+
+
+def test_q4_k_random_round_trip_closed_form(c_oracle):
+    rng = np.random.default_rng(4)
+    for _ in range(50):
+        sc, mn = rng.integers(0, 64, 8), rng.integers(0, 64, 8)
+        q = rng.integers(0, 16, 256)
+        d, dmin = np.float16(abs(rng.standard_normal()) * 0.01), np.float16(abs(rng.standard_normal()) * 0.01)
+        out = _both(c_oracle, _blocks(go.pack_q4_k(d, dmin, sc, mn, q)), go.Q4_K).numpy()
+        # both products are exact in fp64 and in fp32; one rounding in the subtraction
+        exact = np.float64(d) * sc.repeat(32) * q - np.float64(dmin) * mn.repeat(32)
+        assert np.array_equal(out, exact.astype(np.float32))
+
+
+# ---- Q6_K ------------------------------------------------------------------------------------
+
+def test_q6_k_one_hot_positions(c_oracle):
+    scales = np.ones(16, dtype=np.int8)
+    for pos in list(range(0, 256, 5)) + [31, 32, 95, 96, 127, 128, 255]:
+        q = [32] * 256          # 32 decodes to 0
+        q[pos] = 32 + 21        # uses low nibble and both high bits
+        out = _both(c_oracle, _blocks(go.pack_q6_k(1.0, scales, q)), go.Q6_K)
+        want = torch.zeros(256)
+        want[pos] = 21.0
+        assert torch.equal(out, want), pos
+
+
+def test_q6_k_scale_index_and_sign(c_oracle):
+    scales = np.array([-128, 127, 3, -5, 7, -11, 13, -17, 19, -23, 29, -31, 37, -41, 43, -47], dtype=np.int8)
+    q = [(11 * i + 5) % 64 for i in range(256)]
+    out = _both(c_oracle, _blocks(go.pack_q6_k(0.25, scales, q)), go.Q6_K).numpy()
+    want = np.array([0.25 * int(scales[i // 16]) * (q[i] - 32) for i in range(256)], dtype=np.float32)
+    assert np.array_equal(out, want)
+
+
+def test_q6_k_random_round_trip_closed_form(c_oracle):
+    rng = np.random.default_rng(5)
+    for _ in range(50):
+        scales = rng.integers(-128, 128, 16).astype(np.int8)
+        q = rng.integers(0, 64, 256)
+        d = np.float16(abs(rng.standard_normal()) * 0.01)
+        out = _both(c_oracle, _blocks(go.pack_q6_k(d, scales, q)), go.Q6_K).numpy()
+        exact = np.float64(d) * scales.astype(np.float64).repeat(16) * (q - 32)   # <= 24 significant bits
+        assert np.array_equal(out.astype(np.float64), exact)
+
+
+# ---- hand-written known-answer blocks ---------------------------------------------------------
+
+def test_known_answer_blocks(c_oracle):
+    """tests/golden/kat_blocks.json holds blocks typed in by hand from the format definition
+    (hex bytes) with expected values worked out on paper; see the file's "how" fields."""
+    with open(os.path.join(HERE, "golden", "kat_blocks.json")) as f:
+        kats = json.load(f)
+    assert len(kats) >= 6
+    for kat in kats:
+        packed = _blocks(bytes.fromhex(kat["hex"]))
+        qt = kat["type"]
+        assert packed.shape[1] == go.GGML_QUANT_SIZES[qt][1], kat["name"]
+        out = _both(c_oracle, packed, qt, kat.get("numerics", 0)).numpy().astype(np.float64)
+        want = np.zeros(go.GGML_QUANT_SIZES[qt][0]) + kat.get("fill", 0.0)
+        for idx, val in kat["expect"].items():
+            want[int(idx)] = val
+        assert np.array_equal(out, want), kat["name"]
+
+
+# ---- the two restatements against each other, both numerics, bulk -------------------------------
+
+@pytest.mark.parametrize("qt", TYPES)
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_c_and_torch_agree_bulk(c_oracle, qt, numerics):
+    from sensenova_u1_amd import synthetic
+    bs, ts = go.GGML_QUANT_SIZES[qt]
+    n_blocks = 100_000 if bs == 32 else 20_000
+    packed = synthetic.make_packed(qt, n_blocks // 50, 50 * bs, seed=qt)
+    for out_dtype in (torch.float32, torch.float16, torch.bfloat16):
+        a = c_oracle.dequantize(packed, qt, out_dtype, numerics)
+        b = go.dequantize_gguf_tensor(packed, qt, numerics).to(out_dtype)
+        assert torch.equal(a.view(torch.int16 if out_dtype != torch.float32 else torch.int32),
+                           b.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("qt", TYPES)
+def test_fp16_chain_is_not_the_fp32_chain(qt):
+    """The two numerics modes really differ (a few percent of bf16 weights), so parity tests
+    can tell which chain a kernel follows."""
+    from sensenova_u1_amd import synthetic
+    packed = synthetic.make_packed(qt, 64, 1024, seed=1)
+    a = go.dequantize_gguf_tensor(packed, qt, 0).to(torch.bfloat16)
+    b = go.dequantize_gguf_tensor(packed, qt, 1).to(torch.bfloat16)
+    frac = (a.view(torch.int16) != b.view(torch.int16)).float().mean().item()
+    assert 0.01 < frac < 0.5, frac
+
+
+def test_fp16_chain_each_rounding_against_numpy():
+    """numerics 1 for Q4_K, step by step with numpy float16 arithmetic (an implementation of
+    IEEE half that is neither torch's nor the C file's)."""
+    rng = np.random.default_rng(6)
+    sc, mn, q = rng.integers(0, 64, 8), rng.integers(0, 64, 8), rng.integers(0, 16, 256)
+    d, dmin = np.float16(0.0123), np.float16(0.0077)
+    packed = _blocks(go.pack_q4_k(d, dmin, sc, mn, q))
+    got = go.dequantize_gguf_tensor(packed, go.Q4_K, 1).numpy().flatten()
+    D = (d * sc.astype(np.float16)).astype(np.float16)
+    DM = (dmin * mn.astype(np.float16)).astype(np.float16)
+    want = ((D.repeat(32) * q.astype(np.float16)).astype(np.float16) - DM.repeat(32)).astype(np.float16)
+    assert got.dtype == np.float16 and np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+# ---- linear and routing -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("qt", TYPES)
+def test_linear_against_fp64_bruteforce(c_oracle, qt):
+    from sensenova_u1_amd import synthetic
+    packed = synthetic.make_packed(qt, 24, 512, seed=7)
+    x = synthetic.make_activations(3, 512, seed=8)
+    bias = torch.linspace(-1, 1, 24).to(torch.bfloat16)
+    w = go.dequantize_gguf_tensor(packed, qt, 1).to(torch.bfloat16).double()
+    exact = x.double() @ w.T + bias.double()
+    for y in (go.gguf_linear_forward(x, packed, qt, bias), c_oracle.linear(x, packed, qt, bias)):
+        assert y.dtype == torch.bfloat16
+        # a bf16 result is within half an ulp (2^-9 relative) of the exact value, give or take
+        # the fp32 accumulation error
+        assert torch.all((y.double() - exact).abs() <= exact.abs() * 2.0 ** -8 + 1e-6)
+    assert go.rel_l2(go.gguf_linear_forward(x, packed, qt, bias), c_oracle.linear(x, packed, qt, bias)) < 3e-4
+
+
+def test_linear_transposed_operand_would_fail(c_oracle):
+    """N != K and a weight with one hot row: a transposed or mis-strided weight cannot pass."""
+    n, k = 3, 64
+    w = np.zeros((n, k), dtype=np.float32)
+    w[1, :] = np.linspace(-1, 1, k)
+    packed = torch.from_numpy(go.quantize_q8_0(w))
+    x = torch.ones(1, k, dtype=torch.bfloat16)
+    y = c_oracle.linear(x, packed, go.Q8_0).float()
+    assert y[0, 0] == 0 and y[0, 2] == 0
+    deq = c_oracle.dequantize(packed, go.Q8_0, torch.float32, 1).to(torch.bfloat16).double()
+    assert abs(float(y[0, 1]) - float(deq[1].sum())) <= 2.0 ** -8 * abs(float(deq[1].sum())) + 1e-3
+
+
+def test_grouped_is_two_linears(c_oracle):
+    from sensenova_u1_amd import synthetic
+    wu = synthetic.make_packed(go.Q8_0, 16, 128, seed=1)
+    wg = synthetic.make_packed(go.Q4_K, 16, 256, seed=2)[:, :144]   # one Q4_K block per row: K = 256
+    wu = synthetic.make_packed(go.Q8_0, 16, 256, seed=1)
+    x = synthetic.make_activations(9, 256, seed=3)
+    ind = torch.tensor([0, 1, 1, 0, 0, 1, 0, 1, 1], dtype=torch.bool)
+    for fn in (go.grouped_linear_forward, c_oracle.grouped_linear):
+        y = fn(x, ind, wu, go.Q8_0, wg, go.Q4_K)
+        yu = go.gguf_linear_forward(x[~ind], wu, go.Q8_0)
+        yg = go.gguf_linear_forward(x[ind], wg, go.Q4_K)
+        assert go.rel_l2(y[~ind], yu) < 3e-4 and go.rel_l2(y[ind], yg) < 3e-4
+    y = go.grouped_linear_forward(x, torch.zeros(9, dtype=torch.bool), wu, go.Q8_0, wg, go.Q4_K)
+    assert torch.equal(y, go.gguf_linear_forward(x, wu, go.Q8_0))
+
+
+def test_silu_mul_rounding_chain(c_oracle):
+    g = torch.linspace(-8, 8, 4001).to(torch.bfloat16)
+    u = torch.linspace(3, -3, 4001).to(torch.bfloat16)
+    want = torch.nn.functional.silu(g) * u
+    got = c_oracle.silu_mul(g, u)
+    assert (got.view(torch.int16) != want.view(torch.int16)).float().mean() < 0.01
+    assert go.rel_l2(got, want) < 1e-3
