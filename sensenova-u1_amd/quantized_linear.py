@@ -85,6 +85,14 @@ class GGUFParameter(torch.nn.Parameter):
             return type(result)(retag(r) for r in result)
         return result
 
+    def __deepcopy__(self, memo):
+        if id(self) in memo:
+            return memo[id(self)]
+        clone = GGUFParameter(self.as_tensor().detach().clone(memory_format=torch.preserve_format),
+                              requires_grad=self.requires_grad, quant_type=self.quant_type)
+        memo[id(self)] = clone
+        return clone
+
     def __reduce_ex__(self, proto):
         return (_rebuild_gguf_parameter, (self.as_tensor().detach(), int(self.quant_type)))
 

@@ -1,0 +1,64 @@
+"""The C-ABI library loads on a CPU-only host and exports every symbol include/sngguf.h declares.
+No compute call is made here (that needs a GPU)."""
+import ctypes
+import os
+import re
+
+from sensenova_u1_amd import ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sngguf.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sngguf_\w+)\s*\(", text)))
+
+
+def test_header_symbols_exported():
+    lib = ops.load_library()
+    names = _declared_symbols()
+    assert len(names) >= 9
+    for name in names:
+        assert hasattr(lib, name), f"libsngguf.so does not export {name}"
+    assert set(names) == set(ops.EXPORTED_SYMBOLS)
+
+
+def test_host_only_entry_points():
+    lib = ops.load_library()
+    assert lib.sngguf_version() >= 100
+    assert (lib.sngguf_block_size(8), lib.sngguf_type_size(8)) == (32, 34)
+    assert (lib.sngguf_block_size(12), lib.sngguf_type_size(12)) == (256, 144)
+    assert (lib.sngguf_block_size(14), lib.sngguf_type_size(14)) == (256, 210)
+    assert lib.sngguf_block_size(13) == 0 and lib.sngguf_type_size(2) == 0
+    assert lib.sngguf_grouped_workspace_bytes(1000) >= 4 * 1000 + 4
+    assert lib.sngguf_strerror(0) == b"ok"
+    for code in range(-6, 0):
+        assert lib.sngguf_strerror(code) not in (b"ok", b"unknown error")
+
+
+def test_argument_validation_needs_no_device():
+    """Bad arguments are rejected before anything touches the GPU, so this runs on a CPU host."""
+    lib = ops.load_library()
+    buf = ctypes.create_string_buffer(4096 + 64)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 63) // 64 * 64)
+    odd = ctypes.c_void_p(p.value + 2)
+    E_TYPE, E_SHAPE, E_NULL, E_ALIGN = -1, -2, -3, -4
+    assert lib.sngguf_dequantize(p, 13, 1, 256, p, 0, 0, None) == E_TYPE        # Q5_K not implemented
+    assert lib.sngguf_dequantize(p, 8, 1, 32, p, 7, 0, None) == E_TYPE          # bad out dtype
+    assert lib.sngguf_dequantize(p, 8, 1, 32, p, 0, 5, None) == E_TYPE          # bad numerics
+    assert lib.sngguf_dequantize(p, 8, 1, 33, p, 0, 0, None) == E_SHAPE         # cols % 32
+    assert lib.sngguf_dequantize(p, 12, 1, 128, p, 0, 0, None) == E_SHAPE       # cols % 256
+    assert lib.sngguf_dequantize(p, 8, -1, 32, p, 0, 0, None) == E_SHAPE
+    assert lib.sngguf_dequantize(None, 8, 1, 32, p, 0, 0, None) == E_NULL
+    assert lib.sngguf_dequantize(odd, 8, 1, 32, p, 0, 0, None) == E_ALIGN
+    assert lib.sngguf_dequantize(p, 8, 0, 32, None, 0, 0, None) == 0            # empty: nothing to do
+    assert lib.sngguf_linear(p, 1, p, 8, 4, 48, None, p, 1, None) == E_SHAPE    # K % 32
+    assert lib.sngguf_linear(p, 1, p, 14, 4, 64, None, p, 1, None) == E_SHAPE   # K % 256
+    assert lib.sngguf_linear(None, 1, p, 8, 4, 64, None, p, 1, None) == E_NULL
+    assert lib.sngguf_linear(p, 1, p, 8, 4, 64, None, odd, 1, None) == E_ALIGN
+    assert lib.sngguf_linear(p, 0, p, 8, 4, 64, None, p, 1, None) == 0
+    assert lib.sngguf_gate_up_silu(p, 17, p, p, 8, 4, 64, p, 1, None) == E_SHAPE  # decode only
+    assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL
+    assert lib.sngguf_grouped_linear(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_NULL  # no workspace
+    assert lib.sngguf_grouped_linear(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_SHAPE  # n_text > M

@@ -1,0 +1,101 @@
+"""GPU: the module / loader boundary end to end - file -> load -> GGUFLinear.forward on the HIP
+kernels, against the oracle's GGUFLinear.forward_native restatement."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as go
+from sensenova_u1_amd import (GGUFLinear, GGUFParameter, gated_mlp, grouped_linear, load_gguf_checkpoint,
+                              set_gguf2meta_model, synthetic)
+from tests.test_loader import H, I, TinyModel, _make_file
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _load(tmp_path, dev, quant=8):
+    path = str(tmp_path / "m.gguf")
+    ref, packed = _make_file(path, quant)
+    sd = load_gguf_checkpoint(path)
+    with torch.device("meta"):
+        model = TinyModel()
+    return set_gguf2meta_model(model, sd, torch.bfloat16, dev).eval(), packed
+
+
+@pytest.mark.parametrize("quant", [8, 12, 14])
+def test_loaded_model_projections(tmp_path, dev, quant):
+    print(f"case module quant={quant}", flush=True)
+    model, packed = _load(tmp_path, dev, quant)
+    assert model.layers[0].q_proj.weight.device.type == "cuda"
+    for m in (1, 5, 16, 40):
+        x = synthetic.make_activations(m, H, seed=m)
+        for name in ("layers.0.q_proj", "layers.1.mlp.gate_proj_mot_gen", "timestep_embedder"):
+            mod = model.get_submodule(name)
+            want = go.gguf_linear_forward(x, torch.from_numpy(packed[name + ".weight"]), quant,
+                                          mod.bias.cpu() if mod.bias is not None else None)
+            got = mod(x.to(dev).reshape(1, m, H))
+            assert got.shape == (1, m, mod.out_features) and got.dtype == torch.bfloat16
+            assert go.rel_l2(got.cpu().reshape(m, -1), want) <= TOL
+
+
+def test_mlp_decode_and_prefill(tmp_path, dev):
+    """Qwen3MLP.forward through the modules: fused gate/up GEMV at decode, three GEMMs above."""
+    print("case module mlp", flush=True)
+    model, packed = _load(tmp_path, dev)
+    mlp = model.layers[0].mlp
+    w = {n: torch.from_numpy(packed[f"layers.0.mlp.{n}.weight"]) for n in ("gate_proj", "up_proj", "down_proj")}
+    for m in (1, 4, 16, 33):
+        x = synthetic.make_activations(m, H, seed=20 + m)
+        want, _ = go.mlp_forward(x, w["gate_proj"], w["up_proj"], w["down_proj"], (8, 8, 8))
+        got = gated_mlp(x.to(dev), mlp.gate_proj, mlp.up_proj, mlp.down_proj)
+        assert go.rel_l2(got.cpu(), want) <= 2 * TOL   # two chained projections
+
+
+def test_grouped_modules(tmp_path, dev):
+    print("case module grouped", flush=True)
+    model, packed = _load(tmp_path, dev)
+    layer = model.layers[1]
+    x = synthetic.make_activations(2 * 30, H, seed=5).reshape(2, 30, H)
+    ind = torch.zeros(2, 30, dtype=torch.bool)
+    ind[0, 10:] = True
+    ind[1, ::3] = True
+    got = grouped_linear(x.to(dev), ind.to(dev), layer.q_proj, layer.q_proj_mot_gen)
+    assert got.shape == (2, 30, H)
+    want = go.grouped_linear_forward(x.reshape(60, H), ind.reshape(60), torch.from_numpy(packed["layers.1.q_proj.weight"]),
+                                     8, torch.from_numpy(packed["layers.1.q_proj_mot_gen.weight"]), 8)
+    assert go.rel_l2(got.cpu().reshape(60, H), want) <= TOL
+    # the reference's production cases: all text -> understanding weights only, all image -> generation only
+    all_und = grouped_linear(x.to(dev), torch.zeros(2, 30, dtype=torch.bool, device=dev), layer.q_proj, layer.q_proj_mot_gen)
+    assert torch.equal(all_und, layer.q_proj(x.to(dev)))
+    all_gen = grouped_linear(x.to(dev), None, layer.q_proj, layer.q_proj_mot_gen, n_text=0)
+    assert torch.equal(all_gen, layer.q_proj_mot_gen(x.to(dev)))
+
+
+def test_weight_data_rebinding_between_forwards(dev):
+    """The offloader swaps weight.data between a pinned CPU copy and a fresh device tensor around
+    every forward (layer_offload.py:349-356,373-375)."""
+    print("case module rebinding", flush=True)
+    packed = synthetic.make_packed(8, 64, 256, seed=1)
+    lin = GGUFLinear(256, 64, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    lin.weight = GGUFParameter(packed.pin_memory(), quant_type=8)
+    x = synthetic.make_activations(3, 256, seed=2).to(dev)
+    want = go.gguf_linear_forward(x, packed, 8)
+    cpu_copy = lin.weight.data
+    for _ in range(3):
+        lin.weight.data = cpu_copy.to(dev, non_blocking=True)
+        y = lin(x)
+        lin.weight.data = cpu_copy
+        assert go.rel_l2(y.cpu(), want) <= TOL
+
+
+def test_other_compute_dtypes_use_hip_dequantize(dev):
+    print("case module fp16 compute", flush=True)
+    packed = synthetic.make_packed(12, 64, 512, seed=3)
+    for dt in (torch.float16, torch.float32):
+        lin = GGUFLinear(512, 64, bias=True, compute_dtype=dt, device="meta")
+        lin.weight = GGUFParameter(packed.to(dev), quant_type=12)
+        lin.bias = torch.nn.Parameter(torch.linspace(-1, 1, 64, device=dev, dtype=dt), requires_grad=False)
+        x = synthetic.make_activations(9, 512, seed=4).to(dev).to(dt)
+        want = go.gguf_linear_forward(x, packed, 12, lin.bias, compute_dtype=dt)
+        got = lin(x)
+        assert got.dtype == dt and go.rel_l2(got.cpu(), want) <= TOL
