@@ -1,0 +1,501 @@
+// Q8_0 decode GEMV on the matrix cores (1 <= M <= 16, K % 256 == 0).
+//
+// A workgroup owns 16 weight rows (for the SiLU-gated pair: the same 16 rows of the gate and of
+// the up matrix, on separate wavefronts); its wavefronts split K between them and add their
+// partial sums through LDS at the end.  Per wavefront and step of CB blocks (CB * 34 packed
+// bytes per row, CB = 16 when K allows it):
+//   * the 16-row slab is fetched with coalesced 16-byte loads (consecutive lanes walk along a
+//     row) into registers one step ahead, then dropped into the wavefront's private LDS slab, so
+//     HBM sees long contiguous runs although blocks are 34 bytes long and every 128-byte line
+//     is requested by one wavefront (or by two neighbours of one workgroup at the same time);
+//   * lane (r = lane % 16, g = lane / 16) picks quants 8g..8g+7 and the scale of each block of
+//     row r out of LDS with 4-byte aligned reads (blocks at even positions sit 2 bytes off a
+//     dword boundary and are realigned with v_alignbit), decodes them to eight bf16 (rounding
+//     chain by numerics mode) and feeds them as the A operand of v_mfma_f32_16x16x32_bf16; the
+//     B operand is x[m = lane % 16][32 b + 8 g ..].  One MFMA contracts one 32-element block
+//     for 16 weight rows and up to 16 activation rows, so the cost per packed byte does not
+//     depend on M and the cross-lane reduction happens inside the matrix core.
+// Nothing dequantized is written to memory.
+#include <stdlib.h>
+
+#include "sngguf_common.hpp"
+
+namespace sngguf {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
+        const uint32_t u = dw ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
+        const half2_t d2 = {d, d};
+        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
+        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        const float d = f16_to_f32(d_bits);
+        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
+        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
+    }
+}
+
+// CB: blocks per step.  GATED: wavefronts [0, W) work on qa (gate), [W, 2W) on qb (up).
+template <int NUM, int CB, bool GATED, int WMAX>
+__global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,
+                                                            const uint8_t* __restrict__ qa,
+                                                            const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                            const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+    constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
+    constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
+    constexpr int kPieces = 16 * kRowPieces;      // per slab
+    constexpr int kLoads = (kPieces + 63) / 64;   // per lane (5 or 9; the last one is partial)
+    constexpr int kSlab = 16 * kRowStep;          // LDS bytes per wavefront (4352 or 8704)
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int W = GATED ? waves >> 1 : waves;     // wavefronts that share one row group's K
+    const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
+    const uint8_t* __restrict__ q = (GATED && wave >= W) ? qb : qa;
+    const int r = lane & 15, g = lane >> 4;
+    const int64_t row_bytes = (K >> 5) * 34;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+
+    // this wavefront's share of the K steps
+    const int steps = (int)(K / (32 * CB));
+    const int s0 = (int)((int64_t)kw * steps / W), s1 = (int)((int64_t)(kw + 1) * steps / W);
+
+    // per-lane slab pieces: piece f = lane + 64 i is bytes [16 (f % P), +16) of slab row f / P
+    uint32_t off[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; i++) {
+        const int f = lane + 64 * i;
+        const bool ok = f < kPieces;
+        const int fr = ok ? f / kRowPieces : 0, fp = ok ? f % kRowPieces : 0;
+        int64_t n = n0 + fr;
+        if (n >= N) n = N - 1;  // rows past the end are decoded from the last row and never stored
+        off[i] = (uint32_t)((n - n0) * row_bytes + 16 * fp);
+    }
+    const uint8_t* __restrict__ base = q + n0 * row_bytes;
+    const bool tail_lane = lane + 64 * (kLoads - 1) < kPieces;  // does the last, partial load cover this lane
+    uint8_t* slab = lds + wave * kSlab;
+
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    u32x4_t pre[kLoads];
+    auto fetch = [&](int s) {
+        const uint8_t* p = base + (int64_t)s * kRowStep;
+#pragma unroll
+        for (int i = 0; i < kLoads - 1; i++) pre[i] = *reinterpret_cast<const u32x4_t*>(p + off[i]);
+        if (tail_lane) pre[kLoads - 1] = *reinterpret_cast<const u32x4_t*>(p + off[kLoads - 1]);
+    };
+    // Lane (r, g) supplies B-operand column r.  Columns >= M are never stored, so those lanes
+    // re-read the last activation row instead of being masked.
+    const bool has_x = r < M;
+    const bf16_t* xrow = x + (int64_t)(has_x ? r : M - 1) * K + 8 * g;
+    const uint8_t* lrow = slab + r * kRowStep + 8 * g;
+
+    // One step: slab of step s is in `pre`, its activations in `xc`.  The next step's activations
+    // (into `xn`) and slab (into `pre`) are requested before this step's MFMAs, so a full step of
+    // decode work covers their latency.
+    auto step = [&](int s, u32x4_t (&xc)[CB], u32x4_t (&xn)[CB]) {
+#pragma unroll
+        for (int i = 0; i < kLoads - 1; i++) *reinterpret_cast<u32x4_t*>(slab + 16 * (lane + 64 * i)) = pre[i];
+        if (tail_lane) *reinterpret_cast<u32x4_t*>(slab + 16 * (lane + 64 * (kLoads - 1))) = pre[kLoads - 1];
+        if (s + 1 < s1) {
+#pragma unroll
+            for (int b = 0; b < CB; b++) xn[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)(s + 1) * CB + b) * 32);
+            fetch(s + 1);
+        }
+#pragma unroll
+        for (int b = 0; b < CB; b++) {
+            // block b of row r starts at byte 34 b: scale, then quants; this lane wants quants 8g..8g+7
+            const uint16_t d = *reinterpret_cast<const uint16_t*>(slab + r * kRowStep + 34 * b);
+            uint32_t q0, q1;
+            if ((b & 1) == 0) {
+                // 34 b is a multiple of 4: the quants start 2 bytes into a dword
+                const uint32_t* w = reinterpret_cast<const uint32_t*>(lrow + 34 * b);
+                const uint32_t w0 = w[0], w1 = w[1], w2 = w[2];
+                q0 = __builtin_amdgcn_alignbit(w1, w0, 16);
+                q1 = __builtin_amdgcn_alignbit(w2, w1, 16);
+            } else {
+                const uint32_t* w = reinterpret_cast<const uint32_t*>(lrow + 34 * b + 2);
+                q0 = w[0];
+                q1 = w[1];
+            }
+            uint32_t a0, a1, a2, a3;
+            q8_dword_bf16<NUM>(d, q0, a0, a1);
+            q8_dword_bf16<NUM>(d, q1, a2, a3);
+            const u32x4_t a = {a0, a1, a2, a3};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                          __builtin_bit_cast(bf16x8_t, xc[b]), acc, 0, 0, 0);
+        }
+    };
+    u32x4_t xa[CB], xb[CB];
+    if (s0 < s1) {
+#pragma unroll
+        for (int b = 0; b < CB; b++) xa[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)s0 * CB + b) * 32);
+        fetch(s0);
+    }
+    for (int s = s0; s < s1; s += 2) {
+        step(s, xa, xb);
+        if (s + 1 < s1) step(s + 1, xb, xa);
+    }
+
+    // ---- add the wavefronts' partial sums (the slabs are dead: reuse them) -------------------------
+    __syncthreads();
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][64]
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave != 0 || !has_x) return;
+    // D[i][j]: j = lane % 16 is the activation row, register v holds weight row 4 * (lane / 16) + v
+    f32x4_t sum = red[lane];
+    for (int w = 1; w < W; w++) {
+        const f32x4_t t = red[w * 64 + lane];
+        sum[0] += t[0]; sum[1] += t[1]; sum[2] += t[2]; sum[3] += t[3];
+    }
+    const int m = r;
+    const int64_t n = n0 + 4 * g;
+    float o[4];
+    if constexpr (GATED) {
+        f32x4_t up = red[W * 64 + lane];
+        for (int w = 1; w < W; w++) {
+            const f32x4_t t = red[(W + w) * 64 + lane];
+            up[0] += t[0]; up[1] += t[1]; up[2] += t[2]; up[3] += t[3];
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const float gt = bf16_to_f32(f32_to_bf16(sum[v]));
+            const float ut = bf16_to_f32(f32_to_bf16(up[v]));
+            const float sl = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+            o[v] = sl * ut;
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
+    }
+    bf16_t* yr = y + (int64_t)m * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+            if (n + v < N) yr[v] = f32_to_bf16(o[v]);
+    }
+}
+
+
+// ---- line-aligned variant (K % 2048 == 0) ----------------------------------------------------------
+// 2048 elements of a Q8_0 row are 64 blocks = 2176 bytes = exactly 17 cache lines of 128 bytes, so
+// when K is a multiple of 2048 every row starts on a line boundary and a wavefront can work on
+// whole "spans" of 17 lines.  HBM delivers markedly more when every wavefront load covers whole
+// lines, so this variant fetches lines (two per row and step, eight full lines per wavefront
+// load) instead of block-aligned runs, and keeps them in a four-line ring per row in LDS:
+// line L of the span sits at ring bytes [128 (L % 4), +128).  A step still decodes 8 blocks
+// (272 bytes, 2.125 lines); the fetch schedule - lines 0..3 before step 0, two more lines per
+// step, line 16 for the last step - always has the lines a step needs in the ring and only
+// overwrites lines whose blocks are done.  A block that runs over the end of the ring is read
+// with wrapped addresses.
+constexpr int kRing = 512;        // ring bytes per row
+constexpr int kRingRow = 528;     // LDS bytes per row: 132 dwords, rows fall on distinct banks
+constexpr int kSpanBytes = 2176;  // 64 blocks = 17 lines
+
+template <int NUM, bool GATED, int WMAX, bool XLDS>
+__global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
+                                                                 const uint8_t* __restrict__ qa,
+                                                                 const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                                 const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int W = GATED ? waves >> 1 : waves;
+    const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
+    const uint8_t* __restrict__ q = (GATED && wave >= W) ? qb : qa;
+    const int r = lane & 15, g = lane >> 4;
+    const int64_t row_bytes = (K >> 5) * 34;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int spans = (int)(K >> 11);
+    const int t0 = (int)((int64_t)kw * spans / W), t1 = (int)((int64_t)(kw + 1) * spans / W);
+
+    // Two-line fetch: piece lane + 64 i is bytes [16 c, +16) of the 256-byte window of row
+    // (lane / 16) + 4 i, c = lane % 16.  One-line fetch: row (lane / 8) + 8 i, piece lane % 8.
+    uint32_t goff2[4], goff1[2];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int64_t n = n0 + (lane >> 4) + 4 * i;
+        if (n >= N) n = N - 1;  // rows past the end are decoded from the last row and never stored
+        goff2[i] = (uint32_t)((n - n0) * row_bytes + 16 * (lane & 15));
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        int64_t n = n0 + (lane >> 3) + 8 * i;
+        if (n >= N) n = N - 1;
+        goff1[i] = (uint32_t)((n - n0) * row_bytes + 2048 + 16 * (lane & 7));
+    }
+    const uint8_t* __restrict__ base = q + n0 * row_bytes;
+    uint8_t* slab = lds + wave * (16 * kRingRow);
+    uint8_t* lw2 = slab + (lane >> 4) * kRingRow + 16 * (lane & 15);  // + 4 i rows, + 256 for odd groups
+    uint8_t* lw1 = slab + (lane >> 3) * kRingRow + 16 * (lane & 7);   // + 8 i rows (line 16 -> ring slot 0)
+    const uint8_t* lr = slab + r * kRingRow;                           // this lane's weight row
+
+    // Lane (r, g) supplies B-operand column r = activation row r.  Columns >= M are never stored,
+    // so those lanes re-read the last activation row instead of being masked.
+    const bool has_x = r < M;
+    const bf16_t* xrow = x + (int64_t)(has_x ? r : M - 1) * K + 8 * g;
+    // XLDS: the activations (M * K bf16, a few KB at decode) are copied into LDS once per
+    // workgroup and the B fragments come from there; otherwise they are fetched from global
+    // memory one step ahead.
+    const int64_t xs_stride = 2 * K + 64;   // bytes per activation row in LDS (+64: rows on different banks)
+    uint8_t* xs = lds + waves * (16 * kRingRow);
+    const uint8_t* xsrow = xs + (has_x ? r : M - 1) * xs_stride + 16 * g;
+
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    u32x4_t pa[4], pb[4];     // fetched lines on their way to the ring
+    u32x4_t xa[8], xb[8];     // activation fragments of the current / next step (global path)
+
+    auto fetch2 = [&](int t, int grp, u32x4_t (&dst)[4]) {
+        const uint8_t* p = base + (int64_t)t * kSpanBytes + 256 * grp;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i] = *reinterpret_cast<const u32x4_t*>(p + goff2[i]);
+    };
+    auto store2 = [&](int grp, const u32x4_t (&src)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            *reinterpret_cast<u32x4_t*>(lw2 + 4 * i * kRingRow + ((grp & 1) << 8)) = src[i];
+    };
+    auto fetch_x = [&](int t, int s, u32x4_t (&dst)[8]) {
+        if constexpr (!XLDS) {
+#pragma unroll
+            for (int b = 0; b < 8; b++)
+                dst[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)t * 64 + s * 8 + b) * 32);
+        }
+    };
+
+    if constexpr (XLDS) {
+        // weights of the first step are requested before the activations are staged
+        if (t0 < t1) {
+            fetch2(t0, 0, pa);
+            fetch2(t0, 1, pb);
+        }
+        const int pieces_per_row = (int)(K >> 3);  // 16-byte pieces
+        for (int f = tid; f < M * pieces_per_row; f += blockDim.x) {
+            const int m = f / pieces_per_row, c = f - m * pieces_per_row;
+            *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + 8 * c);
+        }
+        __syncthreads();
+    } else if (t0 < t1) {
+        fetch_x(t0, 0, xa);
+        fetch2(t0, 0, pa);
+        fetch2(t0, 1, pb);
+    }
+    for (int t = t0; t < t1; t++) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            u32x4_t (&xc)[8] = (s & 1) ? xb : xa;
+            u32x4_t (&xn)[8] = (s & 1) ? xa : xb;
+            // -- lines fetched during the previous step go into the ring
+            if (s == 0) {
+                store2(0, pa);
+                store2(1, pb);
+            } else if (s < 7) {
+                store2(s + 1, pa);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4_t*>(lw1 + 8 * i * kRingRow) = pa[i];
+            }
+            // -- requests for the next step: activations first, so that waiting for them does not
+            //    also wait for the weight lines
+            if (s < 7) {
+                fetch_x(t, s + 1, xn);
+                if (s < 6) {
+                    fetch2(t, s + 2, pa);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+                        pa[i] = *reinterpret_cast<const u32x4_t*>(base + (int64_t)t * kSpanBytes + goff1[i]);
+                }
+            } else if (t + 1 < t1) {
+                fetch_x(t + 1, 0, xn);
+                fetch2(t + 1, 0, pa);
+                fetch2(t + 1, 1, pb);
+            }
+            // -- decode and contract the 8 blocks of this step
+#pragma unroll
+            for (int bb = 0; bb < 8; bb++) {
+                const int b = 8 * s + bb;                 // block within the span
+                const int ro = (34 * b) & (kRing - 1);    // ring offset of the block (compile-time)
+                const int qo = (b & 1) ? ro + 2 : ro;     // first 4-byte aligned dword this lane reads, before + 8 g
+                const int nd = (b & 1) ? 2 : 3;           // dwords read
+                const uint16_t d = *reinterpret_cast<const uint16_t*>(lr + ro);
+                uint32_t w[3];
+                if (qo + 24 + 4 * nd <= kRing) {
+                    const uint32_t* src = reinterpret_cast<const uint32_t*>(lr + qo + 8 * g);
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        if (k < nd) w[k] = src[k];
+                } else {  // the block runs over the end of the ring
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        if (k < nd) w[k] = *reinterpret_cast<const uint32_t*>(lr + ((qo + 8 * g + 4 * k) & (kRing - 1)));
+                }
+                uint32_t q0, q1;
+                if (b & 1) {
+                    q0 = w[0];
+                    q1 = w[1];
+                } else {  // quants start 2 bytes into the first dword
+                    q0 = __builtin_amdgcn_alignbit(w[1], w[0], 16);
+                    q1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
+                }
+                uint32_t a0, a1, a2, a3;
+                q8_dword_bf16<NUM>(d, q0, a0, a1);
+                q8_dword_bf16<NUM>(d, q1, a2, a3);
+                const u32x4_t a = {a0, a1, a2, a3};
+                u32x4_t xfrag;
+                if constexpr (XLDS) xfrag = *reinterpret_cast<const u32x4_t*>(xsrow + ((int64_t)t * 64 + b) * 64);
+                else xfrag = xc[bb];
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                              __builtin_bit_cast(bf16x8_t, xfrag), acc, 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- add the wavefronts' partial sums (the rings are dead: reuse them) ---------------------------
+    __syncthreads();
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][64]
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave != 0 || !has_x) return;
+    f32x4_t sum = red[lane];
+    for (int w = 1; w < W; w++) {
+        const f32x4_t v = red[w * 64 + lane];
+        sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+    }
+    const int m = r;
+    const int64_t n = n0 + 4 * g;
+    float o[4];
+    if constexpr (GATED) {
+        f32x4_t up = red[W * 64 + lane];
+        for (int w = 1; w < W; w++) {
+            const f32x4_t v = red[(W + w) * 64 + lane];
+            up[0] += v[0]; up[1] += v[1]; up[2] += v[2]; up[3] += v[3];
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const float gt = bf16_to_f32(f32_to_bf16(sum[v]));
+            const float ut = bf16_to_f32(f32_to_bf16(up[v]));
+            const float sl = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+            o[v] = sl * ut;
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
+    }
+    bf16_t* yr = y + (int64_t)m * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+            if (n + v < N) yr[v] = f32_to_bf16(o[v]);
+    }
+}
+
+template <int NUM>
+static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                       const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+    const int64_t groups = (N + 15) / 16;
+    const int spans = (int)(K >> 11);
+    int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
+    if (gated && w > 4) w = 4;
+    while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 16) w--;   // plenty of row groups: fewer, longer wavefronts
+    if (const char* e = getenv("SNGGUF_KSPLIT")) w = atoi(e);
+    const int waves = gated ? 2 * w : w;
+    const size_t ring_bytes = (size_t)waves * 16 * kRingRow;
+    // stage the activations in LDS when they are small enough to leave room for three workgroups
+    // per compute unit (or, for few row groups, one)
+    const size_t x_bytes = (size_t)M * (2 * K + 64);
+    const size_t x_budget = groups >= 512 ? 16 * 1024 : 96 * 1024;
+    const bool xlds = x_bytes <= x_budget && !getenv("SNGGUF_NOXLDS");
+    const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0);
+    const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
+#define SNGGUF_LAUNCH(G, WM) \
+    do { \
+        if (xlds) gemv_q8_span_kernel<NUM, G, WM, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
+        else gemv_q8_span_kernel<NUM, G, WM, false><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
+    } while (0)
+    if (gated) {
+        if (waves <= 4) SNGGUF_LAUNCH(true, 4);
+        else SNGGUF_LAUNCH(true, 8);
+    } else {
+        if (waves <= 4) SNGGUF_LAUNCH(false, 4);
+        else SNGGUF_LAUNCH(false, 8);
+    }
+#undef SNGGUF_LAUNCH
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
+// How many wavefronts share the K range of one 16-row group: enough that the launch fills the
+// chip (about 12 wavefronts on each of the 256 compute units), at least one step each.
+static int pick_k_split(int64_t groups, int steps, bool gated) {
+    const int64_t per_group = gated ? 2 : 1;
+    int64_t w = (256 * 12 + groups * per_group - 1) / (groups * per_group);
+    if (w < 1) w = 1;
+    if (w > steps) w = steps;
+    const int64_t cap = gated ? 4 : 8;  // at most 8 wavefronts per workgroup (register budget)
+    if (w > cap) w = cap;
+    if (const char* e = getenv("SNGGUF_KSPLIT")) w = atoi(e);
+    return (int)w;
+}
+
+template <int NUM, int CB>
+static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                     const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+    const int64_t groups = (N + 15) / 16;
+    const int steps = (int)(K / (32 * CB));
+    const int w = pick_k_split(groups, steps, gated);
+    const int waves = gated ? 2 * w : w;
+    const size_t lds_bytes = (size_t)waves * 16 * CB * 34;
+    const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
+    // WMAX only sets the register budget the compiler may assume for the workgroup size
+#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y)
+    if (gated) {
+        if (waves <= 4) SNGGUF_LAUNCH(true, 4);
+        else SNGGUF_LAUNCH(true, 8);
+    } else {
+        if (waves <= 4) SNGGUF_LAUNCH(false, 4);
+        else SNGGUF_LAUNCH(false, 8);
+    }
+#undef SNGGUF_LAUNCH
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
+template <int NUM>
+static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
+                     const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+    // The line-aligned variant needs whole 2048-element spans per wavefront; with few row groups
+    // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
+    // every 256 elements) is the better fit.
+    const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
+    if (K % 2048 == 0 && span_waves >= 2048 && !getenv("SNGGUF_NOSPAN"))
+        return launch_span<NUM>(x, M, qa, qb, N, K, bias, y, gated, stream);
+    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, y, gated, stream);
+}
+
+// Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).
+int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
+                        void* y, int numerics, bool gated, hipStream_t stream) {
+    const bf16_t* xp = static_cast<const bf16_t*>(x);
+    const uint8_t* a = static_cast<const uint8_t*>(qa);
+    const uint8_t* b = static_cast<const uint8_t*>(qb);
+    const bf16_t* bp = static_cast<const bf16_t*>(bias);
+    bf16_t* yp = static_cast<bf16_t*>(y);
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);
+    return SNGGUF_E_BADTYPE;
+}
+
+}  // namespace sngguf
