@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libsngguf.so")
-SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemm.hip"]
+SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemm.hip", "gemm_q8.hip"]
 
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIP_FLAGS = [
@@ -46,7 +46,7 @@ def _compile(src: str, obj: str, extra: list[str]) -> None:
 
 def build_library(force: bool = True, extra_flags: list[str] | None = None, jobs: int = 4) -> str:
     """Compile and link libsngguf.so; returns its path.  ``force=False`` skips an up-to-date library."""
-    srcs = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "sngguf_common.hpp"),
+    srcs = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "sngguf_common.hpp"), os.path.join(CSRC, "gemm_args.hpp"),
                                                         os.path.join(PKG_DIR, "..", "include", "sngguf.h")]
     if not force and os.path.exists(LIB_PATH) and all(os.path.getmtime(LIB_PATH) >= os.path.getmtime(s) for s in srcs):
         return LIB_PATH

@@ -11,7 +11,10 @@
 // multiplies the first weight set (text rows -> understanding weights), group 1 the second
 // (image rows -> generation weights).  blockIdx.y enumerates the row tiles of group 0, then
 // those of group 1; a plain linear is the case "all rows in group 0, no map".
+#include <stdlib.h>
+
 #include "sngguf_common.hpp"
+#include "gemm_args.hpp"
 
 namespace sngguf {
 
@@ -20,17 +23,6 @@ constexpr int BN = 128;      // weight rows (output columns) per tile
 constexpr int BK = 64;       // K step
 constexpr int LDS_LD = 72;   // bf16 elements per LDS row: 144 bytes, keeps 16-byte reads conflict-free
 
-struct GemmArgs {
-    const bf16_t* x;
-    bf16_t* y;
-    int64_t M, N, K;
-    const int32_t* rowmap;  // M entries, grouped order -> row of x / y; NULL = identity
-    const int32_t* n0_dev;  // device count of group-0 rows; NULL = use n0
-    int64_t n0;
-    const uint8_t* q[2];
-    const bf16_t* bias[2];
-    int group_mask;         // bit g: rows of group g are computed by this launch
-};
 
 template <int QT, int NUM>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
@@ -220,7 +212,14 @@ static int launch_num(const GemmArgs& a, int numerics, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
+int launch_gemm_q8_tiles(const GemmArgs& a, int numerics, hipStream_t stream);
+
 static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
+    // Q8_0 problems with enough 256 x 256 tiles to occupy the chip: the large-tile kernel;
+    // everything else: the 128 x 128 kernel below
+    const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
+    if (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0 && a.M >= 384 && big_tiles >= 128 && !getenv("SNGGUF_GEMM_V1"))
+        return launch_gemm_q8_tiles(a, numerics, stream);
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(a, numerics, stream);
     case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(a, numerics, stream);

@@ -1,0 +1,23 @@
+// Argument block shared by the dequant-GEMM kernels.
+#pragma once
+
+#include "sngguf_common.hpp"
+
+namespace sngguf {
+
+// The M rows are seen through an optional row map as [group 0 | group 1]; group 0 multiplies
+// weight set 0 (text rows -> understanding weights), group 1 weight set 1 (image rows ->
+// generation weights).  A plain linear is "all rows in group 0, no map".
+struct GemmArgs {
+    const bf16_t* x;
+    bf16_t* y;
+    int64_t M, N, K;
+    const int32_t* rowmap;  // M entries, grouped order -> row of x / y; NULL = identity
+    const int32_t* n0_dev;  // device count of group-0 rows; NULL = use n0
+    int64_t n0;
+    const uint8_t* q[2];
+    const bf16_t* bias[2];
+    int group_mask;         // bit g: rows of group g are computed by this launch
+};
+
+}  // namespace sngguf

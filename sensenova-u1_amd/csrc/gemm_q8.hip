@@ -1,0 +1,317 @@
+// Q8_0 dequant-GEMM, large-tile variant (K % 64 == 0): 256 x 256 output tile per workgroup,
+// K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32, 128
+// accumulator registers each, two wavefronts per SIMD - and two LDS stages.
+//
+// Per K step and workgroup: the 256 x 64 activation tile (32 KB) is copied global -> registers ->
+// LDS.  The packed weight tile (256 rows x 68 bytes) is fetched two steps ahead with coalesced
+// dword loads (consecutive lanes walk along a row), parked in a small per-wavefront LDS slab,
+// and picked up one step later one 34-byte block per thread (wavefronts 0-3 the first block of
+// the step, 4-7 the second), decoded to 32 bf16 with the rounding chain of the numerics mode and
+// written to the other LDS stage while the matrix cores work on the current one.  Weight rows are
+// the MFMA A operand, activation rows the B operand (v_mfma_f32_32x32x16_bf16), so a lane ends
+// up with runs of four consecutive output columns of one activation row.
+//
+// Tiles are numbered so that the workgroups that land on one XCD (workgroup id modulo 8) cover
+// few activation row tiles times all column tiles: those activation tiles stay in that XCD's L2
+// while the (smaller) packed weight tiles stream through.
+#include "gemm_args.hpp"
+#include "sngguf_common.hpp"
+
+namespace sngguf {
+
+namespace {
+
+constexpr int TM = 256;      // activation rows per tile
+constexpr int TN = 256;      // weight rows (output columns) per tile
+constexpr int TK = 64;       // K step
+constexpr int kTileBytes = 256 * 64 * 2;          // one operand tile in LDS (rows of 128 bytes, swizzled)
+constexpr int kRawDwords = 64 * 9;                // raw slab of one wavefront: 64 rows x 9 dwords
+constexpr int kLdsBytes = 4 * kTileBytes + 8 * kRawDwords * 4;  // two stages of both tiles + raw slabs
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
+        const uint32_t u = dw ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
+        const half2_t d2 = {d, d};
+        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
+        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        const float d = f16_to_f32(d_bits);
+        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
+        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
+    }
+}
+
+// Same with the scale already copied into both halves of d2.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16_d2(uint32_t d2_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const uint32_t u = dw ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const half2_t d2 = __builtin_bit_cast(half2_t, d2_bits);
+        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
+        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        q8_dword_bf16<NUM>((uint16_t)(d2_bits & 0xFFFF), dw, p01, p23);
+    }
+}
+
+template <int NUM>
+__global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 wavefronts: rows wm * 64, columns wn * 128
+
+    // ---- tile of this workgroup ---------------------------------------------------------------------
+    const int64_t n0 = a.n0_dev ? (int64_t)*a.n0_dev : a.n0;
+    const int64_t t0 = (a.group_mask & 1) ? (n0 + TM - 1) / TM : 0;            // row tiles of group 0
+    const int64_t t1 = (a.group_mask & 2) ? (a.M - n0 + TM - 1) / TM : 0;      // row tiles of group 1
+    const int64_t ntn = (a.N + TN - 1) / TN;
+    const int64_t total = (t0 + t1) * ntn;
+    const int64_t pid = blockIdx.x;
+    if (pid >= total) return;
+    // consecutive tile numbers on one XCD: workgroup ids are dealt round-robin over 8 XCDs
+    const int64_t per = total >> 3, rem = total & 7;
+    const int64_t xcd = pid & 7, idx = pid >> 3;
+    const int64_t tile = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    const int64_t ty = tile / ntn, tn = tile - ty * ntn;
+    int g;
+    int64_t row_begin, row_end;
+    if (ty < t0) {
+        g = 0; row_begin = ty * TM; row_end = n0;
+    } else {
+        g = 1; row_begin = n0 + (ty - t0) * TM; row_end = a.M;
+    }
+    if (row_end > row_begin + TM) row_end = row_begin + TM;
+    const uint8_t* __restrict__ q = a.q[g];
+    const bf16_t* __restrict__ bias = a.bias[g];
+    const int64_t nb0 = tn * TN;
+    const int64_t row_bytes = (a.K >> 5) * 34;
+    const int ksteps = (int)(a.K / TK);
+
+    // ---- LDS: two stages of (activation tile, weight tile) + one raw-weight slab per wavefront ------------
+    // A tile is 256 rows of 64 bf16 (128 bytes, no padding); the eight 16-byte chunks of a row are
+    // stored at chunk ^ (row % 8), which keeps fragment reads and row-wise writes off each
+    // other's banks.
+    bf16_t* xs[2] = {reinterpret_cast<bf16_t*>(lds), reinterpret_cast<bf16_t*>(lds + 2 * kTileBytes)};
+    bf16_t* ws[2] = {reinterpret_cast<bf16_t*>(lds + kTileBytes), reinterpret_cast<bf16_t*>(lds + 3 * kTileBytes)};
+    uint32_t* raw = reinterpret_cast<uint32_t*>(lds + 4 * kTileBytes) + wave * kRawDwords;
+
+    // ---- per-thread assignments ---------------------------------------------------------------------------
+    // activations: 256 rows x 8 pieces of 16 bytes; piece tid + 512 i = row (tid / 8) + 64 i, piece tid % 8.
+    // Rows past the end of the group re-read the group's last row: they only feed output rows
+    // that are never stored.
+    const bf16_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int64_t rr = row_begin + (tid >> 3) + 64 * i;
+        if (rr >= row_end) rr = row_end - 1;
+        const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+        xsrc[i] = a.x + gr * a.K + 8 * (tid & 7);
+    }
+    const int xdst = (tid >> 3) * 64 + 8 * ((tid & 7) ^ ((tid >> 3) & 7));  // + 64 i rows
+    // weights: wavefront w decodes block `wblk` = w / 4 of the K step for rows 64 (w % 4) .. + 63, one
+    // row per lane.  Those 64 x 9 dwords (scale + quants, 36 of each row's 68 bytes) are fetched with
+    // consecutive lanes walking along a row (9 lanes per row), parked in the wavefront's raw slab
+    // and picked up row-wise one step later.
+    const int wblk = wave >> 2;
+    const int wrow_l = 64 * (wave & 3) + lane;  // row of the tile this lane decodes
+    uint32_t goff[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int f = lane + 64 * i, fr = f / 9, fj = f - 9 * fr;
+        int64_t n = nb0 + 64 * (wave & 3) + fr;
+        if (n >= a.N) n = a.N - 1;
+        goff[i] = (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 4 * fj);
+    }
+    const uint8_t* __restrict__ wbase = q + nb0 * row_bytes;
+    const int wsw = wrow_l & 7;
+    // v_perm_b32 selectors (bytes 0-3 = second operand, 4-7 = first operand)
+    const uint32_t sel_q = wblk ? 0x07060504u : 0x05040302u;  // quant dword: next dword as is / 2 bytes off
+    const uint32_t sel_d = wblk ? 0x03020302u : 0x01000100u;  // block scale copied into both halves
+    bf16_t* wdst[2] = {ws[0] + wrow_l * 64, ws[1] + wrow_l * 64};
+
+    // fragment reads: row (lane % 32) of a 32-row tile, logical chunk 2 ks + lane / 32
+    int foff[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) foff[ks] = (lane & 31) * 64 + 8 * ((2 * ks + (lane >> 5)) ^ (lane & 7));
+
+    f32x16_t acc[4][2];  // [column tile i][row tile j]
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    uint32_t gw[9];   // raw dwords on their way from global memory to the raw slab
+    uint32_t rw[9];   // this lane's block, read back from the raw slab
+    u32x4_t xv[4];    // activation pieces of the next K step
+
+#define SNGGUF_FETCH_W(kb)                                                                                   \
+    do {                                                                                                     \
+        const uint8_t* p_ = wbase + (int64_t)(kb) * 68;                                                      \
+        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) gw[i_] = *reinterpret_cast<const uint32_t*>(p_ + goff[i_]); \
+    } while (0)
+#define SNGGUF_PARK_W()                                                                                      \
+    do {                                                                                                     \
+        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) raw[lane + 64 * i_] = gw[i_];                       \
+    } while (0)
+#define SNGGUF_PICK_W()                                                                                      \
+    do {                                                                                                     \
+        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) rw[i_] = raw[9 * lane + i_];                        \
+    } while (0)
+#define SNGGUF_LOAD_X(kb)                                                                                    \
+    do {                                                                                                     \
+        _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++)                                                     \
+            xv[i_] = *reinterpret_cast<const u32x4_t*>(xsrc[i_] + (int64_t)(kb) * TK);                       \
+    } while (0)
+#define SNGGUF_STORE_X(stage)                                                                                \
+    do {                                                                                                     \
+        _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++)                                                     \
+            *reinterpret_cast<u32x4_t*>(xs[stage] + xdst + 64 * 64 * i_) = xv[i_];                           \
+    } while (0)
+// decode quarter `part` (8 elements = quant dwords 2 part, 2 part + 1) of the block in rw into LDS.
+// First block of a pair: scale in the low half of dword 0, quants from byte 2; second block: scale in
+// the high half of dword 0, quants from dword 1.  Both cases are one v_perm_b32 per dword with a
+// per-wavefront byte selector (sel_q, sel_d), so the code has no branch.
+#define SNGGUF_DECODE_W(stage, part)                                                                         \
+    do {                                                                                                     \
+        const uint32_t q0_ = __builtin_amdgcn_perm(rw[1 + 2 * (part)], rw[2 * (part)], sel_q);               \
+        const uint32_t q1_ = __builtin_amdgcn_perm(rw[2 + 2 * (part)], rw[1 + 2 * (part)], sel_q);           \
+        uint32_t o0_, o1_, o2_, o3_;                                                                         \
+        q8_dword_bf16_d2<NUM>(d2, q0_, o0_, o1_);                                                            \
+        q8_dword_bf16_d2<NUM>(d2, q1_, o2_, o3_);                                                            \
+        *reinterpret_cast<u32x4_t*>(wdst[stage] + 8 * ((4 * wblk + (part)) ^ wsw)) = u32x4_t{o0_, o1_, o2_, o3_}; \
+    } while (0)
+// One K step on LDS stage CUR.  On entry the raw slab holds the packed blocks of step kb + 1; they
+// are decoded into the other stage while the MFMAs run (NEXT), and the blocks of step kb + 2,
+// requested at the top, replace them in the slab at the end (FETCH).
+#define SNGGUF_K_STEP(kb, CUR, NEXT, FETCH)                                                                  \
+    do {                                                                                                     \
+        if (NEXT) {                                                                                          \
+            SNGGUF_LOAD_X((kb) + 1);                                                                         \
+            SNGGUF_PICK_W();                                                                                 \
+        }                                                                                                    \
+        if (FETCH) SNGGUF_FETCH_W((kb) + 2);                                                                 \
+        const bf16_t* a_base_ = ws[CUR] + wn * 128 * 64;                                                     \
+        const bf16_t* b_base_ = xs[CUR] + wm * 64 * 64;                                                      \
+        uint32_t d2 = 0;                                                                                     \
+        if (NEXT) d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                           \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
+            bf16x8_t af_[4], bf_[2];                                                                         \
+            _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
+                af_[i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[ks]);               \
+            _Pragma("unroll") for (int j = 0; j < 2; j++)                                                    \
+                bf_[j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[ks]);               \
+            _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
+                _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[i], bf_[j], acc[i][j], 0, 0, 0); \
+            if (NEXT) SNGGUF_DECODE_W((CUR) ^ 1, ks);                                                        \
+        }                                                                                                    \
+        if (NEXT) SNGGUF_STORE_X((CUR) ^ 1);                                                                 \
+        if (FETCH) SNGGUF_PARK_W();                                                                          \
+        __syncthreads();                                                                                     \
+    } while (0)
+
+    // ---- prologue: stage 0 holds K step 0, the raw slab holds step 1 ------------------------------------------
+    SNGGUF_LOAD_X(0);
+    SNGGUF_FETCH_W(0);
+    SNGGUF_PARK_W();
+    if (ksteps > 1) SNGGUF_FETCH_W(1);
+    SNGGUF_PICK_W();
+    SNGGUF_STORE_X(0);
+    {
+        const uint32_t d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);
+#pragma unroll
+        for (int part = 0; part < 4; part++) SNGGUF_DECODE_W(0, part);
+    }
+    if (ksteps > 1) SNGGUF_PARK_W();
+    __syncthreads();
+
+    for (int kb = 0; kb < ksteps; kb += 2) {
+        {
+            const bool next = kb + 1 < ksteps, fetch = kb + 2 < ksteps;
+            SNGGUF_K_STEP(kb, 0, next, fetch);
+        }
+        if (kb + 1 < ksteps) {
+            const bool next = kb + 2 < ksteps, fetch = kb + 3 < ksteps;
+            SNGGUF_K_STEP(kb + 1, 1, next, fetch);
+        }
+    }
+#undef SNGGUF_K_STEP
+#undef SNGGUF_DECODE_W
+#undef SNGGUF_STORE_X
+#undef SNGGUF_LOAD_X
+#undef SNGGUF_PICK_W
+#undef SNGGUF_PARK_W
+#undef SNGGUF_FETCH_W
+
+    // ---- epilogue: D[i][j], i = weight row (n), j = activation row (m) ----------------------------------------
+    // lane: j = lane % 32; register v: i = 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    const bool fast = (a.N & 3) == 0;  // rows of y are 8-byte aligned and a run of four columns never straddles N
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int vg = 0; vg < 4; vg++) {
+            const int64_t n = nb0 + wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
+            float b[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < a.N) b[e] = bf16_to_f32(bias[n + e]);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int64_t rr = row_begin + wm * 64 + j * 32 + (lane & 31);
+                if (rr >= row_end || n >= a.N) continue;
+                const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+                bf16_t* yp = a.y + gr * a.N + n;
+                const float o0 = acc[i][j][4 * vg] + b[0], o1 = acc[i][j][4 * vg + 1] + b[1];
+                const float o2 = acc[i][j][4 * vg + 2] + b[2], o3 = acc[i][j][4 * vg + 3] + b[3];
+                if (fast) {
+                    *reinterpret_cast<u32x2_t*>(yp) = u32x2_t{pack_bf16(o0, o1), pack_bf16(o2, o3)};
+                } else {
+                    yp[0] = f32_to_bf16(o0);
+                    if (n + 1 < a.N) yp[1] = f32_to_bf16(o1);
+                    if (n + 2 < a.N) yp[2] = f32_to_bf16(o2);
+                    if (n + 3 < a.N) yp[3] = f32_to_bf16(o3);
+                }
+            }
+        }
+    }
+}
+
+template <int NUM>
+int launch_tiles(const GemmArgs& a, hipStream_t stream) {
+    // 144 KB of dynamic LDS: above the default limit, so it is requested once per kernel
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q8_kernel<NUM>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
+    const int64_t row_tiles = (a.M + TM - 1) / TM + 1;  // a split adds at most one partial tile
+    const int64_t ntn = (a.N + TN - 1) / TN;
+    gemm_q8_kernel<NUM><<<dim3((unsigned)(row_tiles * ntn)), dim3(512), kLdsBytes, stream>>>(a);
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
+}  // namespace
+
+// Q8_0, K % 64 == 0 (rows are then 4-byte aligned); both row groups must be Q8_0.
+int launch_gemm_q8_tiles(const GemmArgs& a, int numerics, hipStream_t stream) {
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_tiles<SNGGUF_NUM_GGML_FP32>(a, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_tiles<SNGGUF_NUM_UPSTREAM_FP16>(a, stream);
+    return SNGGUF_E_BADTYPE;
+}
+
+}  // namespace sngguf

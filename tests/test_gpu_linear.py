@@ -94,6 +94,42 @@ def test_gemm_ragged_bias(dev, qt):
         _check(got, want)
 
 
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_gemm_q8_0_large_tile_kernel(dev, c_oracle, numerics):
+    """M >= 384 with K % 64 == 0 takes the 256 x 256 tile kernel: ragged M / N, bias, one K step,
+    odd and even step counts."""
+    print(f"case gemm tiles numerics={numerics}", flush=True)
+    for m, n, k in [(2816, 2816, 64), (3000, 2900, 192), (4100, 2050, 128), (8300, 1030, 64)]:
+        packed = synthetic.make_packed(go.Q8_0, n, k, seed=m + n + k)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
+        want = go.gguf_linear_forward(x, packed, go.Q8_0, bias, numerics=numerics)
+        got = ops.linear(x.to(dev), packed.to(dev), go.Q8_0, bias.to(dev), numerics).cpu()
+        _check(got, want)
+    rows = torch.tensor([0, 255, 256, 8299])
+    sub = c_oracle.linear(x[rows], packed, go.Q8_0, bias, numerics)
+    _check(got[rows], sub)
+
+
+def test_grouped_linear_large_tiles(dev):
+    """Grouped routing through the tile kernel: indicator form and contiguous split, group sizes
+    that are not multiples of the tile."""
+    print("case grouped tiles", flush=True)
+    m, n, k = 4500, 2100, 128
+    wu = synthetic.make_packed(go.Q8_0, n, k, seed=11)
+    wg = synthetic.make_packed(go.Q8_0, n, k, seed=12)
+    x = synthetic.make_activations(m, k, seed=13)
+    ind = torch.rand(m, generator=torch.Generator().manual_seed(14)) < 0.7
+    got = ops.grouped_linear(x.to(dev), ind.to(dev), 0, wu.to(dev), go.Q8_0, wg.to(dev), go.Q8_0).cpu()
+    _check(got, go.grouped_linear_forward(x, ind, wu, go.Q8_0, wg, go.Q8_0))
+    split = torch.arange(m) >= 530
+    got = ops.grouped_linear(x.to(dev), None, 530, wu.to(dev), go.Q8_0, wg.to(dev), go.Q8_0).cpu()
+    _check(got, go.grouped_linear_forward(x, split, wu, go.Q8_0, wg, go.Q8_0))
+    yu = ops.linear(x.to(dev), wu.to(dev), go.Q8_0).cpu()
+    yg = ops.linear(x.to(dev), wg.to(dev), go.Q8_0).cpu()
+    assert torch.equal(got[~split], yu[~split]) and torch.equal(got[split], yg[split])
+
+
 def test_gemm_q8_0_odd_block_count(dev):
     print("case gemm odd blocks", flush=True)
     packed = synthetic.make_packed(go.Q8_0, 70, 96, seed=1)
