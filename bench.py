@@ -28,6 +28,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HIDDEN, INTER, KV = 4096, 12288, 1024
+# HBM bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
+# what the same counters read for a plain 256 MiB copy (profiles/*_pmc.txt give commands and raw
+# values); None = not measured for this build.
+MEASURED_TRAFFIC = {"gemv_gate_up_m1": None, "gemm_gate_m4096": None}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 Q8_0 = 8
@@ -57,6 +61,9 @@ def main() -> None:
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--gemm-steps", type=int, default=3)
     ap.add_argument("--numerics", type=int, default=1, help="1 = upstream fp16 chain (drop-in), 0 = ggml fp32")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 256 MiB elementwise device copies (a known-size reference for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE hardware counters when profiling with rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -74,6 +81,14 @@ def main() -> None:
     dev = torch.device("cuda:0")
     num = args.numerics
     K, W, L = args.steps, args.warmup, args.layers
+
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (256 * 1024 * 1024,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            torch.bitwise_not(src, out=dst)  # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- synthetic weights, resident in HBM --------------------------------------------------
     layers = []
@@ -168,18 +183,18 @@ def main() -> None:
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "device_ms_per_step": round(ev1 / K, 6),
         "roofline": {
-            "kernel": "gemv_kernel<Q8_0, gated> (fused gate/up + SiLU, M=1)",
+            "kernel": "sngguf::gemv_q8_span_kernel<upstream_fp16, gated> (fused gate/up + SiLU, M=1)",
             "bound": "hbm",
             "achieved": round(gu_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gu_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC["gemv_gate_up_m1"],
             "bytes_per_launch": gu_bytes,
             "avg_launch_us": round(gu_ms * 1e3, 3),
         },
         "down_proj": {
-            "kernel": "gemv_kernel<Q8_0> (down 12288->4096, M=1)",
+            "kernel": "sngguf::gemv_q8_mfma_kernel<upstream_fp16> (down 12288->4096, M=1)",
             "achieved": round(dn_bytes / (dn_ms * 1e-3) / 1e9, 1),
             "unit": "GB/s",
             "avg_launch_us": round(dn_ms * 1e3, 3),
@@ -232,13 +247,14 @@ def main() -> None:
             "flop_per_step": flops,
             "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
             "roofline": {
-                "kernel": "gemm_kernel<Q8_0> (gate 4096->12288, M=4096)",
+                "kernel": "sngguf::gemm_q8_kernel<upstream_fp16> (gate 4096->12288, M=4096)",
                 "bound": "mfma",
                 "achieved": round(gate_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
                 "frac": round(gate_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                "traffic": None,
+                "traffic": MEASURED_TRAFFIC["gemm_gate_m4096"],
+                "flop_per_launch": 2.0 * m * INTER * HIDDEN,
                 "avg_launch_us": round(gate_ms * 1e3, 2),
             },
         }
