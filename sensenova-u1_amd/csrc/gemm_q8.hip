@@ -2,10 +2,10 @@
 // K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32, 128
 // accumulator registers each, two wavefronts per SIMD - and two LDS stages.
 //
-// Per K step and workgroup: the 256 x 64 activation tile (32 KB) is copied global -> registers ->
-// LDS.  The packed weight tile (256 rows x 68 bytes) is fetched two steps ahead with coalesced
-// dword loads (consecutive lanes walk along a row), parked in a small per-wavefront LDS slab,
-// and picked up one step later one 34-byte block per thread (wavefronts 0-3 the first block of
+// Per K step and workgroup: the 256 x 64 activation tile (32 KB) is copied global ->
+// LDS, directly.  The packed weight tile (256 rows x 68 bytes) is fetched in 12-byte pieces
+// straight into a small per-wavefront LDS slab, and
+// picked up one step later one 34-byte block per thread (wavefronts 0-3 the first block of
 // the step, 4-7 the second), decoded to 32 bf16 with the rounding chain of the numerics mode and
 // written to the other LDS stage while the matrix cores work on the current one.  Weight rows are
 // the MFMA A operand, activation rows the B operand (v_mfma_f32_32x32x16_bf16), so a lane ends
@@ -25,7 +25,7 @@ constexpr int TM = 256;      // activation rows per tile
 constexpr int TN = 256;      // weight rows (output columns) per tile
 constexpr int TK = 64;       // K step
 constexpr int kTileBytes = 256 * 64 * 2;          // one operand tile in LDS (rows of 128 bytes, swizzled)
-constexpr int kRawDwords = 64 * 9;                // raw slab of one wavefront: 64 rows x 9 dwords
+constexpr int kRawDwords = 64 * 12;               // raw slab of one wavefront: 64 rows x 3 pieces of 16 bytes
 constexpr int kLdsBytes = 4 * kTileBytes + 8 * kRawDwords * 4;  // two stages of both tiles + raw slabs
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -109,7 +109,11 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     uint32_t* raw = reinterpret_cast<uint32_t*>(lds + 4 * kTileBytes) + wave * kRawDwords;
 
     // ---- per-thread assignments ---------------------------------------------------------------------------
-    // activations: 256 rows x 8 pieces of 16 bytes; piece tid + 512 i = row (tid / 8) + 64 i, piece tid % 8.
+    // activations: 256 rows x 8 pieces of 16 bytes, copied global -> LDS directly
+    // (global_load_lds_dwordx4: lane l of a wavefront writes LDS bytes [16 l, +16) after a uniform
+    // base, so one instruction fills eight consecutive 128-byte tile rows).  Instruction i of
+    // wavefront w covers rows 64 i + 8 w .. + 7; the lane that fills physical chunk p of row r
+    // fetches logical chunk p ^ (r % 8), i.e. the swizzle is applied on the global side.
     // Rows past the end of the group re-read the group's last row: they only feed output rows
     // that are never stored.
     const bf16_t* xsrc[4];
@@ -118,22 +122,22 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
         int64_t rr = row_begin + (tid >> 3) + 64 * i;
         if (rr >= row_end) rr = row_end - 1;
         const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-        xsrc[i] = a.x + gr * a.K + 8 * (tid & 7);
+        xsrc[i] = a.x + gr * a.K + 8 * ((tid & 7) ^ ((tid >> 3) & 7));
     }
-    const int xdst = (tid >> 3) * 64 + 8 * ((tid & 7) ^ ((tid >> 3) & 7));  // + 64 i rows
+    const int xrow0 = 8 * wave;  // first tile row this wavefront fills with instruction 0 (+ 64 i)
     // weights: wavefront w decodes block `wblk` = w / 4 of the K step for rows 64 (w % 4) .. + 63, one
-    // row per lane.  Those 64 x 9 dwords (scale + quants, 36 of each row's 68 bytes) are fetched with
-    // consecutive lanes walking along a row (9 lanes per row), parked in the wavefront's raw slab
-    // and picked up row-wise one step later.
+    // row per lane.  Those 64 x 36 bytes (scale + quants, 36 of each row's 68 bytes) are fetched as
+    // 12-byte pieces with consecutive lanes walking along a row (3 lanes per row) into the
+    // wavefront's raw slab and picked up row-wise one step later.
     const int wblk = wave >> 2;
     const int wrow_l = 64 * (wave & 3) + lane;  // row of the tile this lane decodes
-    uint32_t goff[9];
+    uint32_t goff[3];
 #pragma unroll
-    for (int i = 0; i < 9; i++) {
-        const int f = lane + 64 * i, fr = f / 9, fj = f - 9 * fr;
+    for (int i = 0; i < 3; i++) {
+        const int f = lane + 64 * i, fr = f / 3, fj = f - 3 * fr;  // 12-byte piece fj of slab row fr
         int64_t n = nb0 + 64 * (wave & 3) + fr;
         if (n >= a.N) n = a.N - 1;
-        goff[i] = (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 4 * fj);
+        goff[i] = (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 12 * fj);
     }
     const uint8_t* __restrict__ wbase = q + nb0 * row_bytes;
     const int wsw = wrow_l & 7;
@@ -155,32 +159,28 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    uint32_t gw[9];   // raw dwords on their way from global memory to the raw slab
     uint32_t rw[9];   // this lane's block, read back from the raw slab
-    u32x4_t xv[4];    // activation pieces of the next K step
 
-#define SNGGUF_FETCH_W(kb)                                                                                   \
+// global -> raw slab, directly (global_load_lds_dwordx3: lane l writes its 12 bytes at 16 l after a
+// uniform base, i.e. every piece occupies a 16-byte slot whose last dword is not written; three
+// such slots make one row of the slab): pieces [I0, I1) of step kb
+#define SNGGUF_FETCH_W(kb, I0, I1)                                                                           \
     do {                                                                                                     \
         const uint8_t* p_ = wbase + (int64_t)(kb) * 68;                                                      \
-        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) gw[i_] = *reinterpret_cast<const uint32_t*>(p_ + goff[i_]); \
-    } while (0)
-#define SNGGUF_PARK_W()                                                                                      \
-    do {                                                                                                     \
-        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) raw[lane + 64 * i_] = gw[i_];                       \
+        _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p_ + goff[i_]), \
+                                             (__attribute__((address_space(3))) void*)(raw + 256 * i_), 12, 0, 0); \
     } while (0)
 #define SNGGUF_PICK_W()                                                                                      \
     do {                                                                                                     \
-        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) rw[i_] = raw[9 * lane + i_];                        \
+        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) rw[i_] = raw[12 * lane + 4 * (i_ / 3) + i_ % 3];                        \
     } while (0)
-#define SNGGUF_LOAD_X(kb)                                                                                    \
+#define SNGGUF_LOAD_X(kb, stage, I0, I1)                                                                     \
     do {                                                                                                     \
-        _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++)                                                     \
-            xv[i_] = *reinterpret_cast<const u32x4_t*>(xsrc[i_] + (int64_t)(kb) * TK);                       \
-    } while (0)
-#define SNGGUF_STORE_X(stage)                                                                                \
-    do {                                                                                                     \
-        _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++)                                                     \
-            *reinterpret_cast<u32x4_t*>(xs[stage] + xdst + 64 * 64 * i_) = xv[i_];                           \
+        _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
+            __builtin_amdgcn_global_load_lds(                                                                \
+                (const __attribute__((address_space(1))) void*)(xsrc[i_] + (int64_t)(kb) * TK),              \
+                (__attribute__((address_space(3))) void*)(xs[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
     } while (0)
 // decode quarter `part` (8 elements = quant dwords 2 part, 2 part + 1) of the block in rw into LDS.
 // First block of a pair: scale in the low half of dword 0, quants from byte 2; second block: scale in
@@ -195,49 +195,68 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
         q8_dword_bf16_d2<NUM>(d2, q1_, o2_, o3_);                                                            \
         *reinterpret_cast<u32x4_t*>(wdst[stage] + 8 * ((4 * wblk + (part)) ^ wsw)) = u32x4_t{o0_, o1_, o2_, o3_}; \
     } while (0)
-// One K step on LDS stage CUR.  On entry the raw slab holds the packed blocks of step kb + 1; they
-// are decoded into the other stage while the MFMAs run (NEXT), and the blocks of step kb + 2,
-// requested at the top, replace them in the slab at the end (FETCH).
+// One K step on LDS stage CUR.  On entry the raw slab holds the packed blocks of step kb + 1: they
+// are picked up (NEXT) and decoded into the other stage while the MFMAs run; once picked up, the
+// slab is refilled with the blocks of step kb + 2 (FETCH), and the other stage's activation tile
+// with that of step kb + 1.  Global requests are spread over the MFMA slices instead of being
+// issued in one burst: a burst from all eight wavefronts right after the barrier fills the
+// address pipeline and holds every wavefront - and with it the matrix cores - at its next request.
 #define SNGGUF_K_STEP(kb, CUR, NEXT, FETCH)                                                                  \
     do {                                                                                                     \
-        if (NEXT) {                                                                                          \
-            SNGGUF_LOAD_X((kb) + 1);                                                                         \
-            SNGGUF_PICK_W();                                                                                 \
-        }                                                                                                    \
-        if (FETCH) SNGGUF_FETCH_W((kb) + 2);                                                                 \
+        if (NEXT) SNGGUF_PICK_W();                                                                           \
         const bf16_t* a_base_ = ws[CUR] + wn * 128 * 64;                                                     \
         const bf16_t* b_base_ = xs[CUR] + wm * 64 * 64;                                                      \
         uint32_t d2 = 0;                                                                                     \
         if (NEXT) d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                           \
+        bf16x8_t af_[2][4], bf_[2][2];  /* fragments of this 16-wide K slice and of the next one */          \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                        \
+            af_[0][i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[0]);                 \
+        _Pragma("unroll") for (int j = 0; j < 2; j++)                                                        \
+            bf_[0][j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[0]);                 \
         _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
-            bf16x8_t af_[4], bf_[2];                                                                         \
-            _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
-                af_[i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[ks]);               \
-            _Pragma("unroll") for (int j = 0; j < 2; j++)                                                    \
-                bf_[j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[ks]);               \
+            if (ks < 3) {                                                                                    \
+                _Pragma("unroll") for (int i = 0; i < 4; i++)                                                \
+                    af_[(ks + 1) & 1][i] =                                                                   \
+                        *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[(ks + 1) & 3]);      \
+                _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
+                    bf_[(ks + 1) & 1][j] =                                                                   \
+                        *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[(ks + 1) & 3]);      \
+            }                                                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                                               \
             _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
                 _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[i], bf_[j], acc[i][j], 0, 0, 0); \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[ks & 1][i], bf_[ks & 1][j],      \
+                                                                        acc[i][j], 0, 0, 0);                 \
+            __builtin_amdgcn_sched_barrier(0);                                                               \
+            if (FETCH) {                                                                                     \
+                if (ks == 0) SNGGUF_FETCH_W((kb) + 2, 0, 2);                                                 \
+                if (ks == 1) SNGGUF_FETCH_W((kb) + 2, 2, 3);                                                 \
+            }                                                                                                \
+            if (NEXT) {                                                                                      \
+                if (ks == 1) SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 0, 1);                                       \
+                if (ks == 2) SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 1, 3);                                       \
+                if (ks == 3) SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 3, 4);                                       \
+            }                                                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                                               \
             if (NEXT) SNGGUF_DECODE_W((CUR) ^ 1, ks);                                                        \
         }                                                                                                    \
-        if (NEXT) SNGGUF_STORE_X((CUR) ^ 1);                                                                 \
-        if (FETCH) SNGGUF_PARK_W();                                                                          \
+        /* the next activation tile and the next raw blocks must have landed in LDS */                      \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                     \
         __syncthreads();                                                                                     \
     } while (0)
 
-    // ---- prologue: stage 0 holds K step 0, the raw slab holds step 1 ------------------------------------------
-    SNGGUF_LOAD_X(0);
-    SNGGUF_FETCH_W(0);
-    SNGGUF_PARK_W();
-    if (ksteps > 1) SNGGUF_FETCH_W(1);
+    // ---- prologue: stage 0 holds K step 0, the raw slab step 1 ------------------------------------------------
+    SNGGUF_LOAD_X(0, 0, 0, 4);
+    SNGGUF_FETCH_W(0, 0, 3);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     SNGGUF_PICK_W();
-    SNGGUF_STORE_X(0);
     {
         const uint32_t d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);
 #pragma unroll
         for (int part = 0; part < 4; part++) SNGGUF_DECODE_W(0, part);
     }
-    if (ksteps > 1) SNGGUF_PARK_W();
+    if (ksteps > 1) SNGGUF_FETCH_W(1, 0, 3);  // after the pick-up: the slab is free again
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int kb = 0; kb < ksteps; kb += 2) {
@@ -252,10 +271,8 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     }
 #undef SNGGUF_K_STEP
 #undef SNGGUF_DECODE_W
-#undef SNGGUF_STORE_X
 #undef SNGGUF_LOAD_X
 #undef SNGGUF_PICK_W
-#undef SNGGUF_PARK_W
 #undef SNGGUF_FETCH_W
 
     // ---- epilogue: D[i][j], i = weight row (n), j = activation row (m) ----------------------------------------
