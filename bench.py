@@ -28,10 +28,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HIDDEN, INTER, KV = 4096, 12288, 1024
-# HBM bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
-# what the same counters read for a plain 256 MiB copy (profiles/*_pmc.txt give commands and raw
-# values); None = not measured for this build.
-MEASURED_TRAFFIC = {"gemv_gate_up_m1": None, "gemm_gate_m4096": None}
+# HBM bytes per launch of the dominant kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
+# each scaled by what the same counter reads for the plain 256 MiB elementwise copy that
+# --calibrate-copy runs in the same process; None = not measured for this build.
+MEASURED_TRAFFIC = {"gemv_gate_up_m1": 107405926, "gemm_gate_m4096": 1063299000}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 Q8_0 = 8
@@ -67,7 +67,7 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by output rows, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard by output rows; no multi-GPU code is part of it)", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -79,8 +79,8 @@ int64_t sngguf_block_size(int qtype);
  * on the GGUFParameter built at src/sensenova_u1/utils/gguf_loader.py:43, and the upstream
  * operator seam ops.ggml_dequantize(qweight, qtype, rows, cols).
  *
- *  q      packed blocks, row-major [rows][cols / block * type_size] bytes, 2-byte aligned
- *  out    [rows][cols] elements of out_dtype, aligned to its element size
+ *  q      packed blocks, row-major [rows][cols / block * type_size] bytes, base 16-byte aligned
+ *  out    [rows][cols] elements of out_dtype, base 16-byte aligned
  * With SNGGUF_OUT_F32 + SNGGUF_NUM_GGML_FP32 the result is the exact ggml value; with
  * SNGGUF_OUT_F16 + SNGGUF_NUM_UPSTREAM_FP16 it is bit-identical to the upstream fp16 tensor.
  */
@@ -94,7 +94,8 @@ int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols,
  * 444,450,456,504,602,608,614,709,744 executes once the loader has swapped the module.
  *
  *  x, y, bias   bf16, row-major, x and y 16-byte aligned, bias may be NULL
- *  q            packed blocks [N][K / block * type_size], 4-byte aligned rows
+ *  q            packed blocks [N][K / block * type_size], base 16-byte aligned (rows follow each
+ *               other without padding, as in a GGUF file)
  * The weight is rounded to bf16 exactly as `numerics` says, products are accumulated in
  * fp32, bias is added in fp32 and the sum is rounded once to bf16.  M <= 16 takes the fused
  * dequant-GEMV (packed bytes streamed once, nothing dequantized is written to memory);

@@ -11,7 +11,6 @@
 // multiplies the first weight set (text rows -> understanding weights), group 1 the second
 // (image rows -> generation weights).  blockIdx.y enumerates the row tiles of group 0, then
 // those of group 1; a plain linear is the case "all rows in group 0, no map".
-#include <stdlib.h>
 
 #include "sngguf_common.hpp"
 #include "gemm_args.hpp"
@@ -218,7 +217,7 @@ static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t s
     // Q8_0 problems with enough 256 x 256 tiles to occupy the chip: the large-tile kernel;
     // everything else: the 128 x 128 kernel below
     const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-    if (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0 && a.M >= 384 && big_tiles >= 128 && !getenv("SNGGUF_GEMM_V1"))
+    if (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0 && a.M >= 384 && big_tiles >= 128)
         return launch_gemm_q8_tiles(a, numerics, stream);
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(a, numerics, stream);

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 
 template <int NUM>
 int launch_tiles(const GemmArgs& a, hipStream_t stream) {
-    // 144 KB of dynamic LDS: above the default limit, so it is requested once per kernel
+    // 152 KB of dynamic LDS: above the default limit, so it is requested once per kernel
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q8_kernel<NUM>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (attr != hipSuccess) return SNGGUF_E_LAUNCH;

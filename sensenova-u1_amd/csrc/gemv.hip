@@ -7,7 +7,6 @@
 // HBM to registers once, are decoded to bf16 pairs there, multiplied with the bf16
 // activations (v_dot2_f32_bf16, fp32 accumulate) and reduced across the wavefront with DPP;
 // no dequantized weight ever reaches memory.
-#include <stdlib.h>
 
 #include "sngguf_common.hpp"
 
@@ -317,7 +316,7 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
     bf16_t* yp = static_cast<bf16_t*>(y);
-    if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0 && !getenv("SNGGUF_GEMV_V1"))
+    if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);

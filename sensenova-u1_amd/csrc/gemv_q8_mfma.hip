@@ -16,7 +16,6 @@
 //     for 16 weight rows and up to 16 activation rows, so the cost per packed byte does not
 //     depend on M and the cross-lane reduction happens inside the matrix core.
 // Nothing dequantized is written to memory.
-#include <stdlib.h>
 
 #include "sngguf_common.hpp"
 
@@ -412,20 +411,29 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
     if (gated && w > 4) w = 4;
     while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 16) w--;   // plenty of row groups: fewer, longer wavefronts
-    if (const char* e = getenv("SNGGUF_KSPLIT")) w = atoi(e);
     const int waves = gated ? 2 * w : w;
     const size_t ring_bytes = (size_t)waves * 16 * kRingRow;
     // stage the activations in LDS when they are small enough to leave room for three workgroups
     // per compute unit (or, for few row groups, one)
     const size_t x_bytes = (size_t)M * (2 * K + 64);
     const size_t x_budget = groups >= 512 ? 16 * 1024 : 96 * 1024;
-    const bool xlds = x_bytes <= x_budget && !getenv("SNGGUF_NOXLDS");
+    const bool xlds = x_bytes <= x_budget;
     const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0);
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
+    // the rings of 8 wavefronts plus staged activations can exceed the default dynamic-LDS limit:
+    // raise it once per kernel instance
+#define SNGGUF_LAUNCH_ONE(G, WM, XL) \
+    do { \
+        static const hipError_t attr = hipFuncSetAttribute( \
+            reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL>), \
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+        if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
+        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
+    } while (0)
 #define SNGGUF_LAUNCH(G, WM) \
     do { \
-        if (xlds) gemv_q8_span_kernel<NUM, G, WM, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
-        else gemv_q8_span_kernel<NUM, G, WM, false><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
+        if (xlds) SNGGUF_LAUNCH_ONE(G, WM, true); \
+        else SNGGUF_LAUNCH_ONE(G, WM, false); \
     } while (0)
     if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
@@ -435,6 +443,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
         else SNGGUF_LAUNCH(false, 8);
     }
 #undef SNGGUF_LAUNCH
+#undef SNGGUF_LAUNCH_ONE
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
@@ -447,7 +456,6 @@ static int pick_k_split(int64_t groups, int steps, bool gated) {
     if (w > steps) w = steps;
     const int64_t cap = gated ? 4 : 8;  // at most 8 wavefronts per workgroup (register budget)
     if (w > cap) w = cap;
-    if (const char* e = getenv("SNGGUF_KSPLIT")) w = atoi(e);
     return (int)w;
 }
 
@@ -480,7 +488,7 @@ static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
     // every 256 elements) is the better fit.
     const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
-    if (K % 2048 == 0 && span_waves >= 2048 && !getenv("SNGGUF_NOSPAN"))
+    if (K % 2048 == 0 && span_waves >= 2048)
         return launch_span<NUM>(x, M, qa, qb, N, K, bias, y, gated, stream);
     return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, y, gated, stream);
 }
