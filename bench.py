@@ -59,7 +59,10 @@ def main() -> None:
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
-    ap.add_argument("--gemm-steps", type=int, default=3)
+    ap.add_argument("--gemm-steps", type=int, default=20)
+    ap.add_argument("--gemm-warmup", type=int, default=10,
+                    help="untimed tower-layer passes before the GEMM leg (about 20 ms: the shader clock settles "
+                         "under the matrix-core load within that time)")
     ap.add_argument("--numerics", type=int, default=1, help="1 = upstream fp16 chain (drop-in), 0 = ggml fp32")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB elementwise device copies (a known-size reference for scaling the "
@@ -231,10 +234,10 @@ def main() -> None:
             ops.linear_into(xs[HIDDEN], tower[i % 2][4], Q8_0, None, ys[INTER], num)
 
         gs = args.gemm_steps
-        wall, ev = run_region(tower_step, gs, 1)
+        wall, ev = run_region(tower_step, gs, args.gemm_warmup)
         flops = sum(2.0 * m * n * k for _, n, k in shapes)
         tflops = flops / (wall / gs * 1e-3) / 1e12
-        _, ev_gate = run_region(gate_only, gs * 2, 1)
+        _, ev_gate = run_region(gate_only, gs * 2, args.gemm_warmup)
         gate_ms = ev_gate / (gs * 2)
         gate_tflops = 2.0 * m * INTER * HIDDEN / (gate_ms * 1e-3) / 1e12
         result["gemm"] = {
@@ -243,6 +246,7 @@ def main() -> None:
             "value": round(tflops, 2),
             "unit": "TFLOP/s",
             "steps": gs,
+            "warmup": args.gemm_warmup,
             "ms_per_step": round(wall / gs, 4),
             "flop_per_step": flops,
             "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),

@@ -17,6 +17,20 @@
 #include "gemm_args.hpp"
 #include "sngguf_common.hpp"
 
+// One scheduling region per 16-wide K slice: the eight matrix instructions of the slice with the
+// decode arithmetic of the next step's weights and the fragment reads of the next slice slotted
+// between them, so that the vector ALU and LDS work under the matrix cores instead of after them.
+#define SNGGUF_INTERLEAVE()                                                  \
+    do {                                                                     \
+        _Pragma("unroll") for (int m_ = 0; m_ < 8; m_++) {                   \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               \
+            if (m_ < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   \
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);               \
+        }                                                                    \
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                   \
+        __builtin_amdgcn_sched_barrier(0);                                   \
+    } while (0)
+
 namespace sngguf {
 
 namespace {
@@ -203,16 +217,19 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 // address pipeline and holds every wavefront - and with it the matrix cores - at its next request.
 #define SNGGUF_K_STEP(kb, CUR, NEXT, FETCH)                                                                  \
     do {                                                                                                     \
-        if (NEXT) SNGGUF_PICK_W();                                                                           \
         const bf16_t* a_base_ = ws[CUR] + wn * 128 * 64;                                                     \
         const bf16_t* b_base_ = xs[CUR] + wm * 64 * 64;                                                      \
-        uint32_t d2 = 0;                                                                                     \
-        if (NEXT) d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                           \
         bf16x8_t af_[2][4], bf_[2][2];  /* fragments of this 16-wide K slice and of the next one */          \
         _Pragma("unroll") for (int i = 0; i < 4; i++)                                                        \
             af_[0][i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[0]);                 \
         _Pragma("unroll") for (int j = 0; j < 2; j++)                                                        \
             bf_[0][j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[0]);                 \
+        if (NEXT) SNGGUF_PICK_W();                                                                           \
+        /* The slab is refilled during this step: its reads must not sink below this point (the  */          \
+        /* scheduler is otherwise free to delay the dwords that are decoded last).                */          \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                   \
+        uint32_t d2 = 0;                                                                                     \
+        if (NEXT) d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                           \
         _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
             if (ks < 3) {                                                                                    \
                 _Pragma("unroll") for (int i = 0; i < 4; i++)                                                \
@@ -222,12 +239,10 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
                     bf_[(ks + 1) & 1][j] =                                                                   \
                         *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[(ks + 1) & 3]);      \
             }                                                                                                \
-            __builtin_amdgcn_sched_barrier(0);                                                               \
             _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
                 _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[ks & 1][i], bf_[ks & 1][j],      \
                                                                         acc[i][j], 0, 0, 0);                 \
-            __builtin_amdgcn_sched_barrier(0);                                                               \
             if (FETCH) {                                                                                     \
                 if (ks == 0) SNGGUF_FETCH_W((kb) + 2, 0, 2);                                                 \
                 if (ks == 1) SNGGUF_FETCH_W((kb) + 2, 2, 3);                                                 \
@@ -237,8 +252,8 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
                 if (ks == 2) SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 1, 3);                                       \
                 if (ks == 3) SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 3, 4);                                       \
             }                                                                                                \
-            __builtin_amdgcn_sched_barrier(0);                                                               \
             if (NEXT) SNGGUF_DECODE_W((CUR) ^ 1, ks);                                                        \
+            SNGGUF_INTERLEAVE();                                                                             \
         }                                                                                                    \
         /* the next activation tile and the next raw blocks must have landed in LDS */                      \
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                     \
@@ -259,7 +274,14 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (int kb = 0; kb < ksteps; kb += 2) {
+    int kb = 0;
+    // steady state: both flags are known, so every K slice is one straight-line region in which
+    // the decode arithmetic can be slotted between the matrix instructions
+    for (; kb + 3 < ksteps; kb += 2) {
+        SNGGUF_K_STEP(kb, 0, true, true);
+        SNGGUF_K_STEP(kb + 1, 1, true, true);
+    }
+    for (; kb < ksteps; kb += 2) {
         {
             const bool next = kb + 1 < ksteps, fetch = kb + 2 < ksteps;
             SNGGUF_K_STEP(kb, 0, next, fetch);
@@ -270,6 +292,7 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
         }
     }
 #undef SNGGUF_K_STEP
+#undef SNGGUF_INTERLEAVE
 #undef SNGGUF_DECODE_W
 #undef SNGGUF_LOAD_X
 #undef SNGGUF_PICK_W
@@ -277,6 +300,45 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 
     // ---- epilogue: D[i][j], i = weight row (n), j = activation row (m) ----------------------------------------
     // lane: j = lane % 32; register v: i = 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    if ((a.N & 7) == 0) {
+        // Rows of y are 16-byte aligned: stage the tile in LDS as bf16 [256 m][256 n] (all K-loop
+        // buffers are dead after the last barrier) and write it out as 16-byte pieces, 32 lanes
+        // along one output row, so that every store instruction fills whole lines.  Storing
+        // straight from the accumulator layout would scatter 8-byte pieces over 32 rows.
+        constexpr int kYRow = 2 * TN + 16;  // bytes; the padding spreads rows over the banks
+        static_assert(TM * kYRow <= kLdsBytes, "output tile must fit the K-loop buffers");
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                const int nl = wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
+                float b[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias && nb0 + nl < a.N) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b[e] = bf16_to_f32(bias[nb0 + nl + e]);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int ml = wm * 64 + j * 32 + (lane & 31);
+                    *reinterpret_cast<u32x2_t*>(lds + ml * kYRow + 2 * nl) =
+                        u32x2_t{pack_bf16(acc[i][j][4 * vg] + b[0], acc[i][j][4 * vg + 1] + b[1]),
+                                pack_bf16(acc[i][j][4 * vg + 2] + b[2], acc[i][j][4 * vg + 3] + b[3])};
+                }
+            }
+        }
+        __syncthreads();
+        const int64_t n = nb0 + 8 * (tid & 31);
+        if (n >= a.N) return;
+#pragma unroll 4
+        for (int p = 0; p < TM / 16; p++) {
+            const int ml = (tid >> 5) + 16 * p;
+            const int64_t rr = row_begin + ml;
+            if (rr >= row_end) break;
+            const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+            *reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n) = *reinterpret_cast<const u32x4_t*>(lds + ml * kYRow + 16 * (tid & 31));
+        }
+        return;
+    }
     const bool fast = (a.N & 3) == 0;  // rows of y are 8-byte aligned and a run of four columns never straddles N
 #pragma unroll
     for (int i = 0; i < 4; i++) {

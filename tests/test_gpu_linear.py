@@ -57,6 +57,27 @@ def test_gemv_q8_0_odd_block_count(dev):
         _check(ops.linear(x.to(dev), packed.to(dev), go.Q8_0).cpu(), go.gguf_linear_forward(x, packed, go.Q8_0))
 
 
+@pytest.mark.parametrize("numerics", [0, 1])
+@pytest.mark.parametrize("m", [1, 16, 512])
+def test_q8_0_fp16_subnormal_products(dev, numerics, m):
+    """Block scales so small that every d * q is an fp16 subnormal (d = 3 * 2^-24, |q| <= 127):
+    the decode must keep them (a path that flushes fp16 subnormals would return zeros).  K covers
+    the line-aligned (2048) and the block-aligned (256) GEMV fetch schemes and both GEMM kernels."""
+    import numpy as np
+    print(f"case fp16 subnormal products numerics={numerics} m={m}", flush=True)
+    for n, k in [(2048, 2048), (48, 256), (512, 512)]:
+        rng = np.random.default_rng(n + k)
+        raw = np.empty((n, k // 32, 34), dtype=np.uint8)
+        raw[..., :2] = np.array([3], dtype=np.uint16).view(np.uint8)      # fp16 bits 0x0003 = 3 * 2^-24
+        raw[..., 2:] = rng.integers(-127, 128, size=(n, k // 32, 32), dtype=np.int8).view(np.uint8)
+        packed = torch.from_numpy(raw.reshape(n, -1))
+        x = (synthetic.make_activations(m, k, seed=k).float() * 4096).to(torch.bfloat16)
+        want = go.gguf_linear_forward(x, packed, go.Q8_0, None, numerics=numerics)
+        assert want.float().abs().max() > 0
+        got = ops.linear(x.to(dev), packed.to(dev), go.Q8_0, None, numerics).cpu()
+        _check(got, want)
+
+
 def test_gemv_fp64_bruteforce_tiny(dev):
     """Independent of torch's matmul: exact fp64 dot products on the bf16-rounded weights."""
     print("case gemv fp64", flush=True)
@@ -99,7 +120,7 @@ def test_gemm_q8_0_large_tile_kernel(dev, c_oracle, numerics):
     """M >= 384 with K % 64 == 0 takes the 256 x 256 tile kernel: ragged M / N, bias, one K step,
     odd and even step counts."""
     print(f"case gemm tiles numerics={numerics}", flush=True)
-    for m, n, k in [(2816, 2816, 64), (3000, 2900, 192), (4100, 2050, 128), (8300, 1030, 64)]:
+    for m, n, k in [(2816, 2816, 64), (3000, 2904, 320), (3000, 2900, 192), (4100, 2050, 128), (8300, 1030, 64)]:
         packed = synthetic.make_packed(go.Q8_0, n, k, seed=m + n + k)
         x = synthetic.make_activations(m, k, seed=m)
         bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
@@ -115,7 +136,11 @@ def test_grouped_linear_large_tiles(dev):
     """Grouped routing through the tile kernel: indicator form and contiguous split, group sizes
     that are not multiples of the tile."""
     print("case grouped tiles", flush=True)
-    m, n, k = 4500, 2100, 128
+    _grouped_large_tiles(dev, 4500, 2100, 128)   # rows of y 8-byte aligned
+    _grouped_large_tiles(dev, 4500, 2104, 256)   # rows of y 16-byte aligned: coalesced store path
+
+
+def _grouped_large_tiles(dev, m, n, k):
     wu = synthetic.make_packed(go.Q8_0, n, k, seed=11)
     wg = synthetic.make_packed(go.Q8_0, n, k, seed=12)
     x = synthetic.make_activations(m, k, seed=13)
