@@ -308,6 +308,9 @@ static int launch_num(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* 
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
                         void* y, int numerics, bool gated, hipStream_t stream);
 
+int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
+                        const void* bias, void* y, int numerics, bool gated, hipStream_t stream);
+
 // M in 1..16, N >= 1, K a positive multiple of the block size (checked by the caller).
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                 const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
@@ -318,6 +321,10 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     bf16_t* yp = static_cast<bf16_t*>(y);
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
+#ifndef SNGGUF_KQ_V1
+    if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q6_K)
+        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
+#endif
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
     case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);

@@ -48,6 +48,28 @@ def test_gemv_shapes_bias_ragged(dev, c_oracle, qt):
         _check(got, c_oracle.linear(x, packed, qt, bias))
 
 
+@pytest.mark.parametrize("qt", [go.Q4_K, go.Q6_K])
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_gemv_k_quants_two_row_groups(dev, c_oracle, qt, numerics):
+    """N >= 32768 puts two 16-row groups on one wavefront: ragged N (last group half empty, last
+    row group missing), bias, one and several super-blocks per wavefront, plain and SiLU-gated."""
+    print(f"case gemv k-quant wide qt={qt} numerics={numerics}", flush=True)
+    for n, k, m in [(32776, 256, 16), (32791, 768, 5), (32768, 1024, 1)]:
+        packed = synthetic.make_packed(qt, n, k, seed=n + k)
+        x = synthetic.make_activations(m, k, seed=9)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16)
+        got = ops.linear(x.to(dev), packed.to(dev), qt, bias.to(dev), numerics).cpu()
+        _check(got, c_oracle.linear(x, packed, qt, bias, numerics))
+    n, k, m = 32784, 512, 3
+    gate = synthetic.make_packed(qt, n, k, seed=21)
+    up = synthetic.make_packed(qt, n, k, seed=22)
+    x = synthetic.make_activations(m, k, seed=23)
+    g = go.gguf_linear_forward(x, gate, qt, numerics=numerics)
+    u = go.gguf_linear_forward(x, up, qt, numerics=numerics)
+    got = ops.gate_up_silu(x.to(dev), gate.to(dev), up.to(dev), qt, numerics).cpu()
+    _check(got, c_oracle.silu_mul(g, u))
+
+
 def test_gemv_q8_0_odd_block_count(dev):
     """K = 32 * odd: rows are 2-byte aligned and not a whole number of 64-element units."""
     print("case gemv odd blocks", flush=True)
