@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libsngguf.so")
-SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemm.hip", "gemm_q8.hip"]
+SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemm.hip", "gemm_tiles.hip"]
 
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIP_FLAGS = [
@@ -33,8 +33,14 @@ def _hipcc() -> str:
     return exe
 
 
+# per-source additions.  gemv_kq_mfma.hip widens fp16 to fp32 with matrix instructions whose
+# results the vector ALU consumes at once: they must land in ordinary VGPRs, not in accumulation
+# registers that need one v_accvgpr_read per value.
+SOURCE_FLAGS = {"gemv_kq_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _compile(src: str, obj: str, extra: list[str]) -> None:
-    cmd = [_hipcc(), *HIP_FLAGS, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIP_FLAGS, *SOURCE_FLAGS.get(src, []), *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")

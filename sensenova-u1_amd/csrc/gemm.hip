@@ -211,14 +211,14 @@ static int launch_num(const GemmArgs& a, int numerics, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
-int launch_gemm_q8_tiles(const GemmArgs& a, int numerics, hipStream_t stream);
+int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t stream);
 
 static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
-    // Q8_0 problems with enough 256 x 256 tiles to occupy the chip: the large-tile kernel;
+    // Q8_0 / Q4_K problems with enough 256 x 256 tiles to occupy the chip: the large-tile kernel;
     // everything else: the 128 x 128 kernel below
     const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-    if (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0 && a.M >= 384 && big_tiles >= 128)
-        return launch_gemm_q8_tiles(a, numerics, stream);
+    const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0) || qtype == SNGGUF_TYPE_Q4_K;
+    if (tile_type && a.M >= 384 && big_tiles >= 128) return launch_gemm_tiles(a, qtype, numerics, stream);
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(a, numerics, stream);
     case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(a, numerics, stream);

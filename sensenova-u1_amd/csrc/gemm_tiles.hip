@@ -1,15 +1,18 @@
-// Q8_0 dequant-GEMM, large-tile variant (K % 64 == 0): 256 x 256 output tile per workgroup,
-// K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32, 128
-// accumulator registers each, two wavefronts per SIMD - and two LDS stages.
+// Dequant-GEMM, large-tile variant for Q8_0 (K % 64 == 0) and Q4_K: 256 x 256 output tile per
+// workgroup, K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32,
+// 128 accumulator registers each, two wavefronts per SIMD - and two LDS stages.
 //
-// Per K step and workgroup: the 256 x 64 activation tile (32 KB) is copied global ->
-// LDS, directly.  The packed weight tile (256 rows x 68 bytes) is fetched in 12-byte pieces
-// straight into a small per-wavefront LDS slab, and
-// picked up one step later one 34-byte block per thread (wavefronts 0-3 the first block of
-// the step, 4-7 the second), decoded to 32 bf16 with the rounding chain of the numerics mode and
-// written to the other LDS stage while the matrix cores work on the current one.  Weight rows are
-// the MFMA A operand, activation rows the B operand (v_mfma_f32_32x32x16_bf16), so a lane ends
-// up with runs of four consecutive output columns of one activation row.
+// Per K step and workgroup: the 256 x 64 activation tile (32 KB) is copied global -> LDS,
+// directly.  The packed bytes a thread needs for its 32 weights of the step are copied global ->
+// a small per-wavefront LDS slab, also directly, as three pieces per row: Q8_0 the 36 bytes that
+// hold one block and the scale (12-byte pieces); Q4_K the 16-byte super-block head (d, dmin, packed
+// sub-scales) and the 32 quant bytes of the step's 64-element chunk (16-byte pieces).  One step
+// later each thread picks up its row (wavefronts 0-3 the first 32 elements of the step, 4-7 the
+// second: the second Q8_0 block, or the high nibbles of the Q4_K chunk), decodes it to 32 bf16
+// with the rounding chain of the numerics mode and writes it to the other LDS stage while the
+// matrix cores work on the current one.  Weight rows are the MFMA A operand, activation rows the
+// B operand (v_mfma_f32_32x32x16_bf16), so a lane ends up with runs of four consecutive output
+// columns of one activation row.
 //
 // Tiles are numbered so that the workgroups that land on one XCD (workgroup id modulo 8) cover
 // few activation row tiles times all column tiles: those activation tiles stay in that XCD's L2
@@ -80,8 +83,52 @@ __device__ __forceinline__ void q8_dword_bf16_d2(uint32_t d2_bits, uint32_t dw, 
     }
 }
 
+// Q4_K: (D, DM) = (d * sc, dmin * mn) of sub-block j from the super-block head, as the bit pattern
+// the decode uses: NUM 1 the fp16 product copied into both halves of a dword, NUM 0 the fp32 product.
 template <int NUM>
-__global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
+__device__ __forceinline__ void q4k_sub_block_scales(uint32_t dd, uint32_t s0, uint32_t s1, uint32_t s2, int j,
+                                                     uint32_t& D_bits, uint32_t& DM_bits) {
+    typedef Num<NUM> A;
+    const int i = j & 3;
+    const uint32_t lo_sc = (s0 >> (8 * i)) & 63u, lo_mn = (s1 >> (8 * i)) & 63u;
+    const uint32_t b = (s2 >> (8 * i)) & 0xFFu;
+    const uint32_t hi_sc = (b & 0x0Fu) | (((s0 >> (8 * i + 6)) & 3u) << 4), hi_mn = (b >> 4) | (((s1 >> (8 * i + 6)) & 3u) << 4);
+    const uint32_t sc = j < 4 ? lo_sc : hi_sc, mn = j < 4 ? lo_mn : hi_mn;
+    const typename A::T D = A::scale((uint16_t)(dd & 0xFFFF)) * A::integer((int)sc);
+    const typename A::T DM = A::scale((uint16_t)(dd >> 16)) * A::integer((int)mn);
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const uint32_t Dh = __builtin_bit_cast(uint16_t, D), Mh = __builtin_bit_cast(uint16_t, DM);
+        D_bits = Dh | (Dh << 16);
+        DM_bits = Mh | (Mh << 16);
+    } else {
+        D_bits = __builtin_bit_cast(uint32_t, D);
+        DM_bits = __builtin_bit_cast(uint32_t, DM);
+    }
+}
+
+// Four 4-bit quants (one per byte of v) -> q * D - DM as two packed bf16 pairs; NUM 1 rounds to fp16
+// after the product and after the subtraction, NUM 0 works in fp32 (both products exact).
+template <int NUM>
+__device__ __forceinline__ void q4k_dword_bf16(uint32_t D_bits, uint32_t DM_bits, uint32_t v, uint32_t& p01, uint32_t& p23) {
+    // 0x6400 | n is the half 1024 + n
+    const half2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const half2_t q01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u)) - k1024;
+    const half2_t q23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u)) - k1024;
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const half2_t D2 = __builtin_bit_cast(half2_t, D_bits), M2 = __builtin_bit_cast(half2_t, DM_bits);
+        const half2_t a = q01 * D2 - M2, b = q23 * D2 - M2;   // two roundings each (no contraction)
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        const float D = __builtin_bit_cast(float, D_bits), DM = __builtin_bit_cast(float, DM_bits);
+        p01 = pack_bf16(D * (float)q01[0] - DM, D * (float)q01[1] - DM);
+        p23 = pack_bf16(D * (float)q23[0] - DM, D * (float)q23[1] - DM);
+    }
+}
+
+template <int QT, int NUM>
+__global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
+    constexpr bool kQ4K = QT == SNGGUF_TYPE_Q4_K;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -111,7 +158,7 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     const uint8_t* __restrict__ q = a.q[g];
     const bf16_t* __restrict__ bias = a.bias[g];
     const int64_t nb0 = tn * TN;
-    const int64_t row_bytes = (a.K >> 5) * 34;
+    const int64_t row_bytes = kQ4K ? (a.K >> 8) * 144 : (a.K >> 5) * 34;
     const int ksteps = (int)(a.K / TK);
 
     // ---- LDS: two stages of (activation tile, weight tile) + one raw-weight slab per wavefront ------------
@@ -139,25 +186,30 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
         xsrc[i] = a.x + gr * a.K + 8 * ((tid & 7) ^ ((tid >> 3) & 7));
     }
     const int xrow0 = 8 * wave;  // first tile row this wavefront fills with instruction 0 (+ 64 i)
-    // weights: wavefront w decodes block `wblk` = w / 4 of the K step for rows 64 (w % 4) .. + 63, one
-    // row per lane.  Those 64 x 36 bytes (scale + quants, 36 of each row's 68 bytes) are fetched as
-    // 12-byte pieces with consecutive lanes walking along a row (3 lanes per row) into the
-    // wavefront's raw slab and picked up row-wise one step later.
+    // weights: wavefront w decodes elements 32 `wblk` .. + 31 (wblk = w / 4) of the K step for rows
+    // 64 (w % 4) .. + 63, one row per lane.  The bytes it needs are fetched as three pieces per row,
+    // consecutive lanes walking along a row (3 lanes per row), into the wavefront's raw slab and
+    // picked up row-wise one step later.  Q8_0: 12-byte pieces of the 36 bytes that hold the block
+    // and its scale.  Q4_K: piece 0 is the super-block head, pieces 1 and 2 the 32 quant bytes of the
+    // step's chunk; the head moves every fourth step, the quants every step.
     const int wblk = wave >> 2;
     const int wrow_l = 64 * (wave & 3) + lane;  // row of the tile this lane decodes
     uint32_t goff[3];
+    bool head_piece[3];
 #pragma unroll
     for (int i = 0; i < 3; i++) {
-        const int f = lane + 64 * i, fr = f / 3, fj = f - 3 * fr;  // 12-byte piece fj of slab row fr
+        const int f = lane + 64 * i, fr = f / 3, fj = f - 3 * fr;  // piece fj of slab row fr
         int64_t n = nb0 + 64 * (wave & 3) + fr;
         if (n >= a.N) n = a.N - 1;
-        goff[i] = (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 12 * fj);
+        head_piece[i] = fj == 0;
+        goff[i] = kQ4K ? (uint32_t)((n - nb0) * row_bytes + 16 * fj) : (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 12 * fj);
     }
     const uint8_t* __restrict__ wbase = q + nb0 * row_bytes;
     const int wsw = wrow_l & 7;
     // v_perm_b32 selectors (bytes 0-3 = second operand, 4-7 = first operand)
     const uint32_t sel_q = wblk ? 0x07060504u : 0x05040302u;  // quant dword: next dword as is / 2 bytes off
     const uint32_t sel_d = wblk ? 0x03020302u : 0x01000100u;  // block scale copied into both halves
+    const int nib_shift = 4 * wblk;                           // Q4_K: low or high nibbles
     bf16_t* wdst[2] = {ws[0] + wrow_l * 64, ws[1] + wrow_l * 64};
 
     // fragment reads: row (lane % 32) of a 32-row tile, logical chunk 2 ks + lane / 32
@@ -173,21 +225,35 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    uint32_t rw[9];   // this lane's block, read back from the raw slab
+    uint32_t rw[12];  // this lane's pieces, read back from the raw slab (Q8_0 uses 9 dwords)
 
-// global -> raw slab, directly (global_load_lds_dwordx3: lane l writes its 12 bytes at 16 l after a
-// uniform base, i.e. every piece occupies a 16-byte slot whose last dword is not written; three
-// such slots make one row of the slab): pieces [I0, I1) of step kb
+// global -> raw slab, directly: lane l writes its piece into the 16-byte slot l after a uniform base
+// (a 12-byte piece leaves the slot's last dword unwritten); three slots make one row of the slab.
+// Pieces [I0, I1) of step kb.
 #define SNGGUF_FETCH_W(kb, I0, I1)                                                                           \
     do {                                                                                                     \
-        const uint8_t* p_ = wbase + (int64_t)(kb) * 68;                                                      \
-        _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p_ + goff[i_]), \
-                                             (__attribute__((address_space(3))) void*)(raw + 256 * i_), 12, 0, 0); \
+        if constexpr (kQ4K) {                                                                                \
+            const uint8_t* ph_ = wbase + (int64_t)((kb) >> 2) * 144;                                         \
+            const uint8_t* pq_ = ph_ + 32 * ((kb) & 3);                                                      \
+            _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
+                __builtin_amdgcn_global_load_lds(                                                            \
+                    (const __attribute__((address_space(1))) void*)((head_piece[i_] ? ph_ : pq_) + goff[i_]),\
+                    (__attribute__((address_space(3))) void*)(raw + 256 * i_), 16, 0, 0);                    \
+        } else {                                                                                             \
+            const uint8_t* p_ = wbase + (int64_t)(kb) * 68;                                                  \
+            _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
+                __builtin_amdgcn_global_load_lds(                                                            \
+                    (const __attribute__((address_space(1))) void*)(p_ + goff[i_]),                          \
+                    (__attribute__((address_space(3))) void*)(raw + 256 * i_), 12, 0, 0);                    \
+        }                                                                                                    \
     } while (0)
 #define SNGGUF_PICK_W()                                                                                      \
     do {                                                                                                     \
-        _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) rw[i_] = raw[12 * lane + 4 * (i_ / 3) + i_ % 3];                        \
+        if constexpr (kQ4K) {                                                                                \
+            _Pragma("unroll") for (int i_ = 0; i_ < 12; i_++) rw[i_] = raw[12 * lane + i_];                  \
+        } else {                                                                                             \
+            _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) rw[i_] = raw[12 * lane + 4 * (i_ / 3) + i_ % 3]; \
+        }                                                                                                    \
     } while (0)
 #define SNGGUF_LOAD_X(kb, stage, I0, I1)                                                                     \
     do {                                                                                                     \
@@ -196,17 +262,32 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
                 (const __attribute__((address_space(1))) void*)(xsrc[i_] + (int64_t)(kb) * TK),              \
                 (__attribute__((address_space(3))) void*)(xs[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
     } while (0)
-// decode quarter `part` (8 elements = quant dwords 2 part, 2 part + 1) of the block in rw into LDS.
-// First block of a pair: scale in the low half of dword 0, quants from byte 2; second block: scale in
-// the high half of dword 0, quants from dword 1.  Both cases are one v_perm_b32 per dword with a
-// per-wavefront byte selector (sel_q, sel_d), so the code has no branch.
+// Scales of the 32 elements this thread decodes out of rw (the pieces of step kbn): Q8_0 the block
+// scale copied into both halves of sc_a (first block of a pair: low half of dword 0, second: high
+// half); Q4_K (D, DM) of sub-block 2 (kbn % 4) + wblk.
+#define SNGGUF_SCALES_W(kbn)                                                                                 \
+    do {                                                                                                     \
+        if constexpr (kQ4K) q4k_sub_block_scales<NUM>(rw[0], rw[1], rw[2], rw[3], 2 * ((kbn) & 3) + wblk, sc_a, sc_b); \
+        else sc_a = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                              \
+    } while (0)
+// decode quarter `part` (8 elements) of this thread's 32 into LDS.  Q8_0: quant dwords 2 part,
+// 2 part + 1 of the block - for the first block of a pair they start 2 bytes into dword 0, for the
+// second at dword 1; one v_perm_b32 per dword with a per-wavefront byte selector covers both cases
+// without a branch.  Q4_K: the low (wblk 0) or high (wblk 1) nibbles of quant bytes 8 part .. + 7.
 #define SNGGUF_DECODE_W(stage, part)                                                                         \
     do {                                                                                                     \
-        const uint32_t q0_ = __builtin_amdgcn_perm(rw[1 + 2 * (part)], rw[2 * (part)], sel_q);               \
-        const uint32_t q1_ = __builtin_amdgcn_perm(rw[2 + 2 * (part)], rw[1 + 2 * (part)], sel_q);           \
         uint32_t o0_, o1_, o2_, o3_;                                                                         \
-        q8_dword_bf16_d2<NUM>(d2, q0_, o0_, o1_);                                                            \
-        q8_dword_bf16_d2<NUM>(d2, q1_, o2_, o3_);                                                            \
+        if constexpr (kQ4K) {                                                                                \
+            const uint32_t v0_ = (rw[4 + 2 * (part)] >> nib_shift) & 0x0F0F0F0Fu;                            \
+            const uint32_t v1_ = (rw[5 + 2 * (part)] >> nib_shift) & 0x0F0F0F0Fu;                            \
+            q4k_dword_bf16<NUM>(sc_a, sc_b, v0_, o0_, o1_);                                                  \
+            q4k_dword_bf16<NUM>(sc_a, sc_b, v1_, o2_, o3_);                                                  \
+        } else {                                                                                             \
+            const uint32_t q0_ = __builtin_amdgcn_perm(rw[1 + 2 * (part)], rw[2 * (part)], sel_q);           \
+            const uint32_t q1_ = __builtin_amdgcn_perm(rw[2 + 2 * (part)], rw[1 + 2 * (part)], sel_q);       \
+            q8_dword_bf16_d2<NUM>(sc_a, q0_, o0_, o1_);                                                      \
+            q8_dword_bf16_d2<NUM>(sc_a, q1_, o2_, o3_);                                                      \
+        }                                                                                                    \
         *reinterpret_cast<u32x4_t*>(wdst[stage] + 8 * ((4 * wblk + (part)) ^ wsw)) = u32x4_t{o0_, o1_, o2_, o3_}; \
     } while (0)
 // One K step on LDS stage CUR.  On entry the raw slab holds the packed blocks of step kb + 1: they
@@ -228,8 +309,8 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
         /* The slab is refilled during this step: its reads must not sink below this point (the  */          \
         /* scheduler is otherwise free to delay the dwords that are decoded last).                */          \
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                   \
-        uint32_t d2 = 0;                                                                                     \
-        if (NEXT) d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                           \
+        uint32_t sc_a = 0, sc_b = 0;                                                                         \
+        if (NEXT) SNGGUF_SCALES_W((kb) + 1);                                                                 \
         _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
             if (ks < 3) {                                                                                    \
                 _Pragma("unroll") for (int i = 0; i < 4; i++)                                                \
@@ -266,7 +347,8 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     SNGGUF_PICK_W();
     {
-        const uint32_t d2 = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);
+        uint32_t sc_a = 0, sc_b = 0;
+        SNGGUF_SCALES_W(0);
 #pragma unroll
         for (int part = 0; part < 4; part++) SNGGUF_DECODE_W(0, part);
     }
@@ -294,6 +376,7 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
 #undef SNGGUF_K_STEP
 #undef SNGGUF_INTERLEAVE
 #undef SNGGUF_DECODE_W
+#undef SNGGUF_SCALES_W
 #undef SNGGUF_LOAD_X
 #undef SNGGUF_PICK_W
 #undef SNGGUF_FETCH_W
@@ -372,24 +455,28 @@ __global__ __launch_bounds__(512) void gemm_q8_kernel(GemmArgs a) {
     }
 }
 
-template <int NUM>
+template <int QT, int NUM>
 int launch_tiles(const GemmArgs& a, hipStream_t stream) {
     // 152 KB of dynamic LDS: above the default limit, so it is requested once per kernel
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q8_kernel<NUM>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<QT, NUM>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
     const int64_t row_tiles = (a.M + TM - 1) / TM + 1;  // a split adds at most one partial tile
     const int64_t ntn = (a.N + TN - 1) / TN;
-    gemm_q8_kernel<NUM><<<dim3((unsigned)(row_tiles * ntn)), dim3(512), kLdsBytes, stream>>>(a);
+    gemm_tile_kernel<QT, NUM><<<dim3((unsigned)(row_tiles * ntn)), dim3(512), kLdsBytes, stream>>>(a);
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
 }  // namespace
 
-// Q8_0, K % 64 == 0 (rows are then 4-byte aligned); both row groups must be Q8_0.
-int launch_gemm_q8_tiles(const GemmArgs& a, int numerics, hipStream_t stream) {
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_tiles<SNGGUF_NUM_GGML_FP32>(a, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_tiles<SNGGUF_NUM_UPSTREAM_FP16>(a, stream);
+// Q8_0 with K % 64 == 0 (rows are then 4-byte aligned) or Q4_K; both row groups of that type.
+int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
+#define SNGGUF_CASE(QT, NUM) if (qtype == QT && numerics == NUM) return launch_tiles<QT, NUM>(a, stream)
+    SNGGUF_CASE(SNGGUF_TYPE_Q8_0, SNGGUF_NUM_GGML_FP32);
+    SNGGUF_CASE(SNGGUF_TYPE_Q8_0, SNGGUF_NUM_UPSTREAM_FP16);
+    SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_GGML_FP32);
+    SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_UPSTREAM_FP16);
+#undef SNGGUF_CASE
     return SNGGUF_E_BADTYPE;
 }
 

@@ -24,29 +24,54 @@ namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+// fp16 -> fp32 on the matrix core.  With A = the 16 x 16 identity, v_mfma_f32_16x16x16_f16 computes
+// D = I . B + C, and because a lane's B elements (column lane % 16, rows 4 (lane / 16) .. + 3) sit
+// at the same positions as its D elements, every lane gets back its own four fp16 values as
+// exact fp32 (+ c).  The K-quant decode is bound by the vector ALU while the matrix cores are
+// nearly idle, so this takes one conversion per element off the busy unit.  fp16 subnormals are
+// widened exactly; a signed zero comes back as + 0, and a non-finite element (a scale product
+// beyond the fp16 range) turns the other values of its weight row in that instruction into NaN
+// (0 . inf) - the row's dot product is non-finite either way.
+__device__ __forceinline__ half4_t identity_row(int lane) {
+    half4_t a;
+#pragma unroll
+    for (int e = 0; e < 4; e++) a[e] = (4 * (lane >> 4) + e == (lane & 15)) ? (_Float16)1.0f : (_Float16)0.0f;
+    return a;
+}
+__device__ __forceinline__ f32x4_t widen_f16x4(half4_t ident, half2_t lo, half2_t hi, f32x4_t c) {
+    const half4_t b = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(ident, b, c, 0, 0, 0);
+}
+
 // Four small unsigned integers (one per byte of v, each < 256) -> (v - zero) * D - DM as two packed
 // bf16 pairs.  NUM 1: every operation rounds to fp16 (0x6400 | b is the half 1024 + b, so the
-// integer is formed without a convert); NUM 0: exact fp32 products, one rounding in the subtraction.
+// integer is formed without a convert); NUM 0: exact fp32 products, one rounding in the subtraction
+// (the - 1024 - zero rides on the accumulator input of the widening instruction).  Must be called
+// by all 64 lanes; `ident` is identity_row(lane).
 template <int NUM, bool HAS_MIN>
-__device__ __forceinline__ void kq_dword_bf16(uint32_t v, float zero, typename Num<NUM>::T D, typename Num<NUM>::T DM,
-                                              uint32_t& p01, uint32_t& p23) {
+__device__ __forceinline__ void kq_dword_bf16(half4_t ident, uint32_t v, float zero, typename Num<NUM>::T D,
+                                              typename Num<NUM>::T DM, uint32_t& p01, uint32_t& p23) {
     const half2_t h01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u));
     const half2_t h23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u));
-    const _Float16 off = (_Float16)(1024.0f + zero);
-    const half2_t off2 = {off, off};
-    const half2_t q01 = h01 - off2, q23 = h23 - off2;  // exact small integers
     if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const _Float16 off = (_Float16)(1024.0f + zero);
+        const half2_t off2 = {off, off};
         const half2_t D2 = {D, D};
-        half2_t a = q01 * D2, b = q23 * D2;
+        half2_t a = (h01 - off2) * D2, b = (h23 - off2) * D2;
         if constexpr (HAS_MIN) {
             const half2_t M2 = {DM, DM};
             a = a - M2;
             b = b - M2;
         }
-        p01 = pack_bf16((float)a[0], (float)a[1]);
-        p23 = pack_bf16((float)b[0], (float)b[1]);
+        const f32x4_t w = widen_f16x4(ident, a, b, f32x4_t{0.f, 0.f, 0.f, 0.f});
+        p01 = pack_bf16(w[0], w[1]);
+        p23 = pack_bf16(w[2], w[3]);
     } else {
-        float w[4] = {D * (float)q01[0], D * (float)q01[1], D * (float)q23[0], D * (float)q23[1]};
+        const float c = -(1024.0f + zero);
+        const f32x4_t qf = widen_f16x4(ident, h01, h23, f32x4_t{c, c, c, c});
+        float w[4] = {D * qf[0], D * qf[1], D * qf[2], D * qf[3]};
         if constexpr (HAS_MIN) {
 #pragma unroll
             for (int e = 0; e < 4; e++) w[e] = w[e] - DM;
@@ -69,7 +94,7 @@ template <> struct Slab<SNGGUF_TYPE_Q6_K> {
 // The four A operands of half a super-block (sub-blocks 4 HALF .. 4 HALF + 3) of one row, fed to
 // `emit(jj, a)` with jj = 0..3.  `row` points at the row's super-block in the slab; g = lane / 16.
 template <int NUM, int HALF, typename Emit>
-__device__ __forceinline__ void decode_q4_k(const uint8_t* row, int g, Emit&& emit) {
+__device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
     typedef Num<NUM> A;
     const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
     const typename A::T d = A::scale((uint16_t)(head[0] & 0xFFFF)), dmin = A::scale((uint16_t)(head[0] >> 16));
@@ -85,15 +110,15 @@ __device__ __forceinline__ void decode_q4_k(const uint8_t* row, int g, Emit&& em
             const typename A::T D = d * A::integer((int)sc), DM = dmin * A::integer((int)mn);
             const uint32_t v0 = (hi ? qs[0] >> 4 : qs[0]) & 0x0F0F0F0Fu, v1 = (hi ? qs[1] >> 4 : qs[1]) & 0x0F0F0F0Fu;
             uint32_t a0, a1, a2, a3;
-            kq_dword_bf16<NUM, true>(v0, 0.f, D, DM, a0, a1);
-            kq_dword_bf16<NUM, true>(v1, 0.f, D, DM, a2, a3);
+            kq_dword_bf16<NUM, true>(ident, v0, 0.f, D, DM, a0, a1);
+            kq_dword_bf16<NUM, true>(ident, v1, 0.f, D, DM, a2, a3);
             emit(j - 4 * HALF, u32x4_t{a0, a1, a2, a3});
         }
     }
 }
 
 template <int NUM, int HALF, typename Emit>
-__device__ __forceinline__ void decode_q6_k(const uint8_t* row, int g, Emit&& emit) {
+__device__ __forceinline__ void decode_q6_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
     typedef Num<NUM> A;
     constexpr int h = HALF;  // 128-element half of the super-block = sub-blocks 4 h .. 4 h + 3
     const u32x2_t scales = *reinterpret_cast<const u32x2_t*>(row + 192 + 8 * h);  // int8 sub-scales 8 h .. 8 h + 7
@@ -114,7 +139,7 @@ __device__ __forceinline__ void decode_q6_k(const uint8_t* row, int g, Emit&& em
             for (int w = 0; w < 2; w++) {
                 const uint32_t lo = (top ? ql[w] >> 4 : ql[w]) & 0x0F0F0F0Fu;
                 const uint32_t hb = ((qh[w] >> (2 * p)) & 0x03030303u) << 4;
-                kq_dword_bf16<NUM, false>(lo | hb, 32.f, D, D, a[2 * w], a[2 * w + 1]);
+                kq_dword_bf16<NUM, false>(ident, lo | hb, 32.f, D, D, a[2 * w], a[2 * w + 1]);
             }
             emit(p, u32x4_t{a[0], a[1], a[2], a[3]});
         }
@@ -140,6 +165,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
     const uint8_t* __restrict__ q = (GATED && wave >= W) ? qb : qa;
     const int r = lane & 15, g = lane >> 4;
+    const half4_t ident = identity_row(lane);
     const int64_t nsb = K >> 8;
     const int64_t row_bytes = nsb * S::ts;
     const int64_t n0 = (int64_t)blockIdx.x * kRows;
@@ -212,8 +238,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                 acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                                   __builtin_bit_cast(bf16x8_t, xa[jj]), acc[rg], 0, 0, 0);
             };
-            if constexpr (kQ6) decode_q6_k<NUM, 0>(row, g, emit);
-            else decode_q4_k<NUM, 0>(row, g, emit);
+            if constexpr (kQ6) decode_q6_k<NUM, 0>(ident, row, g, emit);
+            else decode_q4_k<NUM, 0>(ident, row, g, emit);
         }
         if (s + 1 < s1) load_x(s + 1, 0, xa);
 #pragma unroll
@@ -223,8 +249,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                 acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                                   __builtin_bit_cast(bf16x8_t, xb[jj]), acc[rg], 0, 0, 0);
             };
-            if constexpr (kQ6) decode_q6_k<NUM, 1>(row, g, emit);
-            else decode_q4_k<NUM, 1>(row, g, emit);
+            if constexpr (kQ6) decode_q6_k<NUM, 1>(ident, row, g, emit);
+            else decode_q4_k<NUM, 1>(ident, row, g, emit);
         }
     };
     if (s0 < s1) {

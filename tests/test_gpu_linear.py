@@ -154,6 +154,25 @@ def test_gemm_q8_0_large_tile_kernel(dev, c_oracle, numerics):
     _check(got[rows], sub)
 
 
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_gemm_q4_k_large_tile_kernel(dev, c_oracle, numerics):
+    """Q4_K through the 256 x 256 tile kernel (M >= 384, at least 128 tiles): every chunk position of
+    a super-block (K steps 0..3 and beyond), ragged M / N, both output paths, bias."""
+    print(f"case gemm q4_k tiles numerics={numerics}", flush=True)
+    for m, n, k in [(3000, 2904, 256), (4100, 2050, 512), (3072, 3080, 1280)]:
+        packed = synthetic.make_packed(go.Q4_K, n, k, seed=m + n + k)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
+        want = go.gguf_linear_forward(x, packed, go.Q4_K, bias, numerics=numerics)
+        got = ops.linear(x.to(dev), packed.to(dev), go.Q4_K, bias.to(dev), numerics).cpu()
+        err = _check(got, want)
+        other = go.gguf_linear_forward(x, packed, go.Q4_K, bias, numerics=1 - numerics)
+        assert err <= go.rel_l2(got, other) + 1e-6
+    rows = torch.tensor([0, 255, 256, 3071])
+    sub = c_oracle.linear(x[rows], packed, go.Q4_K, bias, numerics)
+    _check(got[rows], sub)
+
+
 def test_grouped_linear_large_tiles(dev):
     """Grouped routing through the tile kernel: indicator form and contiguous split, group sizes
     that are not multiples of the tile."""
