@@ -34,20 +34,22 @@ HIDDEN, INTER, KV = 4096, 12288, 1024
 MEASURED_TRAFFIC = {"gemv_gate_up_m1": 107405926, "gemm_gate_m4096": 1063299000}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
-Q8_0 = 8
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}   # elements, bytes per block
 
 
-def q8_bytes(n: int, k: int) -> int:
-    return n * (k // 32) * 34
+def packed_bytes(qt: int, n: int, k: int) -> int:
+    bs, ts = BLOCK[qt]
+    return n * (k // bs) * ts
 
 
-def linear_bytes(m: int, n: int, k: int) -> int:
+def linear_bytes(m: int, n: int, k: int, qt: int = Q8_0) -> int:
     """Algorithmic bytes of one quantized linear: packed weight once, bf16 x once, bf16 y once."""
-    return q8_bytes(n, k) + 2 * m * k + 2 * m * n
+    return packed_bytes(qt, n, k) + 2 * m * k + 2 * m * n
 
 
-def mlp_bytes(m: int) -> int:
-    return 2 * linear_bytes(m, INTER, HIDDEN) + linear_bytes(m, HIDDEN, INTER)
+def mlp_bytes(m: int, gate_up_type: int = Q8_0, down_type: int = Q8_0) -> int:
+    return 2 * linear_bytes(m, INTER, HIDDEN, gate_up_type) + linear_bytes(m, HIDDEN, INTER, down_type)
 
 
 def main() -> None:
@@ -59,6 +61,7 @@ def main() -> None:
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the K-quant (configs[3]) and grouped (configs[4]) legs")
     ap.add_argument("--gemm-steps", type=int, default=20)
     ap.add_argument("--gemm-warmup", type=int, default=10,
                     help="untimed tower-layer passes before the GEMM leg (about 20 ms: the shader clock settles "
@@ -132,22 +135,23 @@ def main() -> None:
         t1 = time.perf_counter()
         return (t1 - t0) * 1e3, e0.elapsed_time(e1)
 
-    def mlp_leg(m: int, n_steps: int, warmup: int):
+    def mlp_leg(m: int, n_steps: int, warmup: int, layers=layers, gate_up_type: int = Q8_0, down_type: int = Q8_0):
         x = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
         h = torch.empty((m, INTER), dtype=torch.bfloat16, device=dev)
         y = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
+        nl = len(layers)
 
         def step(i):
-            gate, up, down = layers[i % L]
-            ops.gate_up_silu_into(x, gate, up, Q8_0, h, num)
-            ops.linear_into(h, down, Q8_0, None, y, num)
+            gate, up, down = layers[i % nl]
+            ops.gate_up_silu_into(x, gate, up, gate_up_type, h, num)
+            ops.linear_into(h, down, down_type, None, y, num)
 
         def gate_up_only(i):
-            gate, up, _ = layers[i % L]
-            ops.gate_up_silu_into(x, gate, up, Q8_0, h, num)
+            gate, up, _ = layers[i % nl]
+            ops.gate_up_silu_into(x, gate, up, gate_up_type, h, num)
 
         def down_only(i):
-            ops.linear_into(h, layers[i % L][2], Q8_0, None, y, num)
+            ops.linear_into(h, layers[i % nl][2], down_type, None, y, num)
 
         wall, ev = run_region(step, n_steps, warmup)
         _, ev_gu = run_region(gate_up_only, n_steps, warmup)
@@ -263,6 +267,75 @@ def main() -> None:
             },
         }
         del tower, xs, ys
+
+    # ---- configs[3]: K-quant mix (Q4_K q/k/v/o/gate/up, Q6_K down) at M = 1, 16 and 4096 -----------------
+    if not args.no_extra:
+        klayers = []
+        for i in range(L):
+            klayers.append((synthetic.make_packed(Q4_K, INTER, HIDDEN, seed=2000 + 3 * i, device=dev),
+                            synthetic.make_packed(Q4_K, INTER, HIDDEN, seed=2001 + 3 * i, device=dev),
+                            synthetic.make_packed(Q6_K, HIDDEN, INTER, seed=2002 + 3 * i, device=dev)))
+        kq = {}
+        for m in (1, 16):
+            k2 = max(64, K // 4)
+            wall, ev, gu, dn = mlp_leg(m, k2, min(W, 16), klayers, Q4_K, Q6_K)
+            nbytes = mlp_bytes(m, Q4_K, Q6_K)
+            gbps = nbytes / (wall / k2 * 1e-3) / 1e9
+            kq[f"mlp_M{m}"] = {"value": round(gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
+                               "bytes_per_step": nbytes, "ms_per_step": round(wall / k2, 6),
+                               "gate_up_us": round(gu * 1e3, 3), "down_us": round(dn * 1e3, 3)}
+        del klayers
+        if not args.no_gemm:
+            m = 4096
+            kshapes = [("q", HIDDEN, HIDDEN, Q4_K), ("k", KV, HIDDEN, Q4_K), ("v", KV, HIDDEN, Q4_K), ("o", HIDDEN, HIDDEN, Q4_K),
+                       ("gate", INTER, HIDDEN, Q4_K), ("up", INTER, HIDDEN, Q4_K), ("down", HIDDEN, INTER, Q6_K)]
+            ktower = [[synthetic.make_packed(qt, n, k, seed=6000 + 10 * r + j, device=dev) for j, (_, n, k, qt) in enumerate(kshapes)]
+                      for r in range(2)]
+            xs = {k: synthetic.make_activations(m, k, seed=k, device=dev) for k in (HIDDEN, INTER)}
+            ys = {n: torch.empty((m, n), dtype=torch.bfloat16, device=dev) for n in (HIDDEN, KV, INTER)}
+
+            def ktower_step(i):
+                ws = ktower[i % 2]
+                for j, (_, n, k, qt) in enumerate(kshapes):
+                    ops.linear_into(xs[k], ws[j], qt, None, ys[n], num)
+
+            gs = max(4, args.gemm_steps // 2)
+            wall, ev = run_region(ktower_step, gs, max(2, args.gemm_warmup // 2))
+            flops = sum(2.0 * m * n * k for _, n, k, _ in kshapes)
+            tflops = flops / (wall / gs * 1e-3) / 1e12
+            kq["tower_M4096"] = {"value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(wall / gs, 4),
+                                 "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2)}
+            del ktower, xs, ys
+        kq["workload"] = ("configs[3]: Q4_K for q/k/v/o/gate/up, Q6_K for down; decode MLP at M=1,16 "
+                          "(GB/s over packed weights + activations) and the 7 tower projections at M=4096")
+        result["k_quants"] = kq
+
+    # ---- configs[4]: one MoT layer, 512 text rows -> understanding weights, 4096 image rows -> generation
+    # weights, each of the 7 linears through the modality-grouped launcher (Q8_0) ---------------------------
+    if not args.no_extra and not args.no_gemm:
+        n_text, m = 512, 512 + 4096
+        shapes = [("q", HIDDEN, HIDDEN), ("k", KV, HIDDEN), ("v", KV, HIDDEN), ("o", HIDDEN, HIDDEN),
+                  ("gate", INTER, HIDDEN), ("up", INTER, HIDDEN), ("down", HIDDEN, INTER)]
+        und = [synthetic.make_packed(Q8_0, n, k, seed=7000 + j, device=dev) for j, (_, n, k) in enumerate(shapes)]
+        gen = [synthetic.make_packed(Q8_0, n, k, seed=7100 + j, device=dev) for j, (_, n, k) in enumerate(shapes)]
+        xs = {k: synthetic.make_activations(m, k, seed=k + 1, device=dev) for k in (HIDDEN, INTER)}
+        ys = {n: torch.empty((m, n), dtype=torch.bfloat16, device=dev) for n in (HIDDEN, KV, INTER)}
+
+        def layer_step(i):
+            for j, (_, n, k) in enumerate(shapes):
+                ops.grouped_linear_into(xs[k], None, n_text, und[j], Q8_0, gen[j], Q8_0, None, None, ys[n], None, num)
+
+        gs = max(4, args.gemm_steps // 2)
+        wall, ev = run_region(layer_step, gs, max(2, args.gemm_warmup // 2))
+        flops = sum(2.0 * m * n * k for _, n, k in shapes)
+        tflops = flops / (wall / gs * 1e-3) / 1e12
+        result["grouped_layer"] = {
+            "workload": "configs[4], one of the 36 layers: 512 text rows -> understanding weights, 4096 image rows -> "
+                        "generation weights, 7 Q8_0 linears through the modality-grouped launcher (contiguous split)",
+            "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall / gs, 4),
+            "flop_per_layer": flops, "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        }
+        del und, gen, xs, ys
 
     # ---- CPU baseline: the oracle's port of GGUFLinear.forward_native on the host cores -----------
     if not args.no_cpu_baseline:
