@@ -1,4 +1,7 @@
-// Fused dequant-GEMV for decode (M <= 16).
+// Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the general path.  The dispatcher at
+// the end of this file sends Q8_0 with K % 256 == 0 and all Q4_K / Q6_K shapes to the matrix-core
+// kernels; what runs here is Q8_0 with other K (the unit decoders for the K-quants are kept as the
+// template's other instantiations, none of which the dispatcher requests).
 //
 // One wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate matrix
 // and row n of the up matrix).  A lane takes 64 weight elements per step - 68 bytes of Q8_0,
@@ -321,16 +324,11 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     bf16_t* yp = static_cast<bf16_t*>(y);
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
-#ifndef SNGGUF_KQ_V1
     if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q6_K)
         return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
-#endif
-    switch (qtype) {
-    case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
-    case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
-    case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
-    default: return SNGGUF_E_BADTYPE;
-    }
+    // Q8_0 rows that are not a whole number of 256-element runs
+    if (qtype == SNGGUF_TYPE_Q8_0) return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
+    return SNGGUF_E_BADTYPE;
 }
 
 }  // namespace sngguf
