@@ -45,44 +45,6 @@ constexpr int kTileBytes = 256 * 64 * 2;          // one operand tile in LDS (ro
 constexpr int kRawDwords = 64 * 12;               // raw slab of one wavefront: 64 rows x 3 pieces of 16 bytes
 constexpr int kLdsBytes = 4 * kTileBytes + 8 * kRawDwords * 4;  // two stages of both tiles + raw slabs
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
-template <int NUM>
-__device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
-    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
-        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
-        const uint32_t u = dw ^ 0x80808080u;
-        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
-        const half2_t d2 = {d, d};
-        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
-        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
-        p01 = pack_bf16((float)a[0], (float)a[1]);
-        p23 = pack_bf16((float)b[0], (float)b[1]);
-    } else {
-        const float d = f16_to_f32(d_bits);
-        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
-        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
-    }
-}
-
-// Same with the scale already copied into both halves of d2.
-template <int NUM>
-__device__ __forceinline__ void q8_dword_bf16_d2(uint32_t d2_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
-    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
-        const uint32_t u = dw ^ 0x80808080u;
-        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const half2_t d2 = __builtin_bit_cast(half2_t, d2_bits);
-        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
-        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
-        p01 = pack_bf16((float)a[0], (float)a[1]);
-        p23 = pack_bf16((float)b[0], (float)b[1]);
-    } else {
-        q8_dword_bf16<NUM>((uint16_t)(d2_bits & 0xFFFF), dw, p01, p23);
-    }
-}
-
 // Q4_K: (D, DM) = (d * sc, dmin * mn) of sub-block j from the super-block head, as the bit pattern
 // the decode uses: NUM 1 the fp16 product copied into both halves of a dword, NUM 0 the fp32 product.
 template <int NUM>

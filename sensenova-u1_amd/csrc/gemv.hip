@@ -1,15 +1,14 @@
-// Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the general path.  The dispatcher at
-// the end of this file sends Q8_0 with K % 256 == 0 and all Q4_K / Q6_K shapes to the matrix-core
-// kernels; what runs here is Q8_0 with other K (the unit decoders for the K-quants are kept as the
-// template's other instantiations, none of which the dispatcher requests).
+// Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the path for Q8_0 rows that are not a
+// whole number of 256-element runs (the dispatcher at the end of this file sends Q8_0 with
+// K % 256 == 0 and all Q4_K / Q6_K shapes to the matrix-core kernels).
 //
-// One wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate matrix
-// and row n of the up matrix).  A lane takes 64 weight elements per step - 68 bytes of Q8_0,
-// one 32-byte nibble chunk of Q4_K, three 16-byte runs of Q6_K - so that one step of the wave
-// reads one contiguous 4352 / 2304 / 3360-byte span of each row.  The packed bytes go from
-// HBM to registers once, are decoded to bf16 pairs there, multiplied with the bf16
-// activations (v_dot2_f32_bf16, fp32 accumulate) and reduced across the wavefront with DPP;
-// no dequantized weight ever reaches memory.
+// K % 64 == 0: one wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate
+// matrix and row n of the up matrix); a lane takes 64 weight elements (68 packed bytes) per step,
+// so that one step of the wave reads one contiguous 4352-byte span of each row.  The packed bytes
+// go from HBM to registers once, are decoded to bf16 pairs there, multiplied with the bf16
+// activations (v_dot2_f32_bf16, fp32 accumulate) and reduced across the wavefront with DPP; no
+// dequantized weight ever reaches memory.  Other K (odd block counts): a generic kernel built on
+// the 8-element decoders, one lane per 8 elements.
 
 #include "sngguf_common.hpp"
 
@@ -21,36 +20,7 @@ namespace sngguf {
 // element offset of 16-element run t (0..3) of unit u
 template <int QT>
 __device__ __forceinline__ int64_t unit_run_offset(int64_t u, int t) {
-    if constexpr (QT == SNGGUF_TYPE_Q6_K) {
-        // unit = (block, half h, 16-lane group j); run t is quadrant t of that half
-        const int64_t b = u >> 2;
-        const int h = (int)(u >> 1) & 1, j = (int)u & 1;
-        return b * 256 + 128 * h + 32 * t + 16 * j;
-    } else {
-        return u * 64 + 16 * t;
-    }
-}
-
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
-template <int NUM>
-__device__ __forceinline__ void q8_dword(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
-    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
-        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
-        const uint32_t u = dw ^ 0x80808080u;
-        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
-        const half2_t d2 = {d, d};
-        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
-        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
-        p01 = pack_bf16((float)a[0], (float)a[1]);
-        p23 = pack_bf16((float)b[0], (float)b[1]);
-    } else {
-        const float d = f16_to_f32(d_bits);
-        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
-        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
-    }
+    return u * 64 + 16 * t;
 }
 
 template <int NUM>
@@ -67,82 +37,15 @@ __device__ __forceinline__ void decode_unit_q8_0(const uint8_t* __restrict__ row
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const uint32_t q0 = __builtin_amdgcn_alignbit(L[i + 1], L[i], 16);  // block 0 quants sit 2 bytes off
-        q8_dword<NUM>(d0, q0, wp[2 * i], wp[2 * i + 1]);
-        q8_dword<NUM>(d1, L[9 + i], wp[16 + 2 * i], wp[16 + 2 * i + 1]);
-    }
-}
-
-template <int NUM>
-__device__ __forceinline__ void decode_unit_q4_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
-    typedef Num<NUM> A;
-    const uint8_t* blk = row + (u >> 2) * 144;
-    const int c = (int)u & 3;
-    const u32x4_t hdr = *reinterpret_cast<const u32x4_t*>(blk);
-    const u32x4_t qa = *reinterpret_cast<const u32x4_t*>(blk + 16 + 32 * c);
-    const u32x4_t qb = *reinterpret_cast<const u32x4_t*>(blk + 32 + 32 * c);
-    const typename A::T d = A::scale((uint16_t)(hdr[0] & 0xFFFF)), dmin = A::scale((uint16_t)(hdr[0] >> 16));
-    uint32_t sc0, mn0, sc1, mn1;
-    q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c, sc0, mn0);
-    q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * c + 1, sc1, mn1);
-    const typename A::T D0 = d * A::integer((int)sc0), M0 = dmin * A::integer((int)mn0);
-    const typename A::T D1 = d * A::integer((int)sc1), M1 = dmin * A::integer((int)mn1);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {  // dword i of the 32 quant bytes: elements 4i..4i+3 (low) and 32+4i.. (high)
-        const uint32_t q = i < 4 ? qa[i] : qb[i - 4];
-        float lo[4], hi[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const uint32_t byte = (q >> (8 * k)) & 0xFFu;
-            lo[k] = A::widen(D0 * A::integer((int)(byte & 0x0Fu)) - M0);
-            hi[k] = A::widen(D1 * A::integer((int)(byte >> 4)) - M1);
-        }
-        wp[2 * i] = pack_bf16(lo[0], lo[1]);
-        wp[2 * i + 1] = pack_bf16(lo[2], lo[3]);
-        wp[16 + 2 * i] = pack_bf16(hi[0], hi[1]);
-        wp[16 + 2 * i + 1] = pack_bf16(hi[2], hi[3]);
-    }
-}
-
-template <int NUM>
-__device__ __forceinline__ void decode_unit_q6_k(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
-    typedef Num<NUM> A;
-    const uint8_t* blk = row + (u >> 2) * 210;  // 2-byte aligned
-    const int h = (int)(u >> 1) & 1, j = (int)u & 1;
-    const u32x4_t la = ld_u128_a2(blk + 64 * h + 16 * j);        // ql[l], l = 16j..16j+15
-    const u32x4_t lb = ld_u128_a2(blk + 64 * h + 32 + 16 * j);   // ql[l + 32]
-    const u32x4_t hh = ld_u128_a2(blk + 128 + 32 * h + 16 * j);  // qh[l]
-    const typename A::T d = A::scale(ld_u16(blk + 208));
-    typename A::T D[4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) D[t] = d * A::integer((int8_t)blk[192 + 8 * h + j + 2 * t]);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {  // dword i: l = 16j + 4i .. +3
-        float v[4][4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const uint32_t a = (la[i] >> (8 * k)) & 0xFFu, b = (lb[i] >> (8 * k)) & 0xFFu, c = (hh[i] >> (8 * k)) & 0xFFu;
-            const int q1 = (int)((a & 0x0Fu) | ((c & 3u) << 4)) - 32;
-            const int q2 = (int)((b & 0x0Fu) | (((c >> 2) & 3u) << 4)) - 32;
-            const int q3 = (int)((a >> 4) | (((c >> 4) & 3u) << 4)) - 32;
-            const int q4 = (int)((b >> 4) | (((c >> 6) & 3u) << 4)) - 32;
-            v[0][k] = A::widen(D[0] * A::integer(q1));
-            v[1][k] = A::widen(D[1] * A::integer(q2));
-            v[2][k] = A::widen(D[2] * A::integer(q3));
-            v[3][k] = A::widen(D[3] * A::integer(q4));
-        }
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            wp[8 * t + 2 * i] = pack_bf16(v[t][0], v[t][1]);
-            wp[8 * t + 2 * i + 1] = pack_bf16(v[t][2], v[t][3]);
-        }
+        q8_dword_bf16<NUM>(d0, q0, wp[2 * i], wp[2 * i + 1]);
+        q8_dword_bf16<NUM>(d1, L[9 + i], wp[16 + 2 * i], wp[16 + 2 * i + 1]);
     }
 }
 
 template <int QT, int NUM>
 __device__ __forceinline__ void decode_unit(const uint8_t* __restrict__ row, int64_t u, uint32_t (&wp)[32]) {
-    if constexpr (QT == SNGGUF_TYPE_Q8_0) decode_unit_q8_0<NUM>(row, u, wp);
-    else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode_unit_q4_k<NUM>(row, u, wp);
-    else decode_unit_q6_k<NUM>(row, u, wp);
+    static_assert(QT == SNGGUF_TYPE_Q8_0, "the unit kernel is only instantiated for Q8_0");
+    decode_unit_q8_0<NUM>(row, u, wp);
 }
 
 __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {

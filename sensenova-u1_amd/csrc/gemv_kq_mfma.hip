@@ -22,7 +22,6 @@ namespace sngguf {
 
 namespace {
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 

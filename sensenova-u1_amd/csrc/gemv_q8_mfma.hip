@@ -21,28 +21,6 @@
 
 namespace sngguf {
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-// Four int8 quants of one dword times the block scale -> two packed bf16 pairs.
-template <int NUM>
-__device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
-    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
-        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
-        const uint32_t u = dw ^ 0x80808080u;
-        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const _Float16 d = __builtin_bit_cast(_Float16, d_bits);
-        const half2_t d2 = {d, d};
-        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
-        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
-        p01 = pack_bf16((float)a[0], (float)a[1]);
-        p23 = pack_bf16((float)b[0], (float)b[1]);
-    } else {
-        const float d = f16_to_f32(d_bits);
-        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
-        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
-    }
-}
-
 // CB: blocks per step.  GATED: wavefronts [0, W) work on qa (gate), [W, 2W) on qb (up).
 template <int NUM, int CB, bool GATED, int WMAX>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,

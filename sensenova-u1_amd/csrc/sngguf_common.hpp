@@ -184,6 +184,35 @@ __device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t
     else decode8_q6_k<NUM>(row, e0, w);
 }
 
+// ---- Q8_0: one dword of quants -> four bf16 (shared by the GEMV and GEMM kernels) ---------------
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// Four int8 quants of one dword times the block scale (given in both halves of d2_bits, fp16)
+// -> two packed bf16 pairs.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16_d2(uint32_t d2_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        // bytes -> fp16 without a convert: 0x6400 | u is the half 1024 + u, u = q + 128
+        const uint32_t u = dw ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const half2_t d2 = __builtin_bit_cast(half2_t, d2_bits);
+        const half2_t a = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias) * d2;
+        const half2_t b = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias) * d2;
+        p01 = pack_bf16((float)a[0], (float)a[1]);
+        p23 = pack_bf16((float)b[0], (float)b[1]);
+    } else {
+        const float d = f16_to_f32((uint16_t)(d2_bits & 0xFFFF));
+        p01 = pack_bf16(d * (float)(int8_t)(dw & 0xFF), d * (float)(int8_t)((dw >> 8) & 0xFF));
+        p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
+    }
+}
+// Same with the scale as the 16 bits of the block header.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    q8_dword_bf16_d2<NUM>((uint32_t)d_bits | ((uint32_t)d_bits << 16), dw, p01, p23);
+}
+
 // ---- wavefront sum ---------------------------------------------------------------------------
 // Butterfly over the 64 lanes: four DPP steps inside each row of 16 lanes, then two
 // ds_swizzle/bpermute steps across rows.  Every lane ends with the full sum.
