@@ -268,6 +268,27 @@ def main() -> None:
         }
         del tower, xs, ys
 
+    # ---- standalone dequantize (the reference's dequantize_gguf_tensor): packed [12288, 4096] -> fp16 -----------
+    if not args.no_extra:
+        deq = {}
+        for qt, name in ((Q8_0, "Q8_0"), (Q4_K, "Q4_K"), (Q6_K, "Q6_K")):
+            srcs = [synthetic.make_packed(qt, INTER, HIDDEN, seed=3000 + i, device=dev) for i in range(8)]
+            out = torch.empty((INTER, HIDDEN), dtype=torch.float16, device=dev)
+
+            def deq_step(i):
+                ops.dequantize_into(srcs[i % 8], qt, out, num)
+
+            n_deq = 64
+            wall, ev = run_region(deq_step, n_deq, 8)
+            nbytes = packed_bytes(qt, INTER, HIDDEN) + 2 * INTER * HIDDEN
+            gbps = nbytes / (ev / n_deq * 1e-3) / 1e9
+            deq[name] = {"value": round(gbps, 1), "unit": "GB/s", "us": round(ev / n_deq * 1e3, 2),
+                         "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2), "bytes": nbytes}
+            del srcs, out
+        deq["workload"] = ("packed [12288, 4096] -> fp16, bytes = packed read + fp16 written; the 100 MB output is "
+                           "rewritten every launch and fits the 256 MB last-level cache")
+        result["dequantize"] = deq
+
     # ---- configs[3]: K-quant mix (Q4_K q/k/v/o/gate/up, Q6_K down) at M = 1, 16 and 4096 -----------------
     if not args.no_extra:
         klayers = []

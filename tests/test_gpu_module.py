@@ -99,3 +99,38 @@ def test_other_compute_dtypes_use_hip_dequantize(dev):
         want = go.gguf_linear_forward(x, packed, 12, lin.bias, compute_dtype=dt)
         got = lin(x)
         assert got.dtype == dt and go.rel_l2(got.cpu(), want) <= TOL
+
+
+def test_mlp_forward_under_hip_graph(tmp_path, dev):
+    """The modules launch on torch's current stream, allocate only through torch's allocator and
+    never synchronise, so a decode step can be captured into a HIP graph.  The replay is checked
+    against the eager result three times with fresh inputs (and eager work between replays)."""
+    print("case module graph capture", flush=True)
+    from sensenova_u1_amd import modality
+    from sensenova_u1_amd.quantized_linear import GGUFLinear, GGUFParameter
+    torch.manual_seed(0)
+    hidden, inter = 512, 1536
+    mods = {}
+    for name, (n, k) in {"gate": (inter, hidden), "up": (inter, hidden), "down": (hidden, inter)}.items():
+        m = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device=dev)
+        m.weight = GGUFParameter(synthetic.make_packed(go.Q8_0, n, k, seed=len(name)).to(dev), quant_type=go.Q8_0)
+        mods[name] = m
+
+    def mlp(x):
+        return modality.gated_mlp(x, mods["gate"], mods["up"], mods["down"])
+
+    static_x = synthetic.make_activations(4, hidden, seed=1).to(dev)
+    for _ in range(3):
+        mlp(static_x)                       # warm-up outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = mlp(static_x)
+    for seed in (11, 12, 13):
+        x = synthetic.make_activations(4, hidden, seed=seed).to(dev)
+        want = mlp(x)                       # eager work between replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, want)
