@@ -28,6 +28,7 @@ extern "C" {
 enum {
     SNGGUF_TYPE_Q8_0 = 8,  /* 32 elements / 34 bytes:  f16 d; i8 qs[32]                         */
     SNGGUF_TYPE_Q4_K = 12, /* 256 elements / 144 bytes: f16 d, dmin; u8 scales[12]; u8 qs[128]  */
+    SNGGUF_TYPE_Q5_K = 13, /* 256 elements / 176 bytes: f16 d, dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] */
     SNGGUF_TYPE_Q6_K = 14  /* 256 elements / 210 bytes: u8 ql[128]; u8 qh[64]; i8 sc[16]; f16 d */
 };
 
@@ -75,7 +76,7 @@ int64_t sngguf_block_size(int qtype);
 
 /*
  * Standalone dequantize.  Replaces diffusers.quantizers.gguf.utils.dequantize_gguf_tensor
- * (+ dequantize_blocks_Q8_0 / _Q4_K / _Q6_K), the function GGUFLinear.forward_native calls
+ * (+ dequantize_blocks_Q8_0 / _Q4_K / _Q5_K / _Q6_K), the function GGUFLinear.forward_native calls
  * on the GGUFParameter built at src/sensenova_u1/utils/gguf_loader.py:43, and the upstream
  * operator seam ops.ggml_dequantize(qweight, qtype, rows, cols).
  *

@@ -32,11 +32,11 @@ import subprocess
 import numpy as np
 import torch
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 QK_K = 256
 K_SCALE_SIZE = 12
 # gguf.GGML_QUANT_SIZES: type -> (elements per block, bytes per block)
-GGML_QUANT_SIZES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+GGML_QUANT_SIZES = {Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
 
 NUM_GGML_FP32 = 0
 NUM_UPSTREAM_FP16 = 1
@@ -89,6 +89,22 @@ def dequantize_blocks_Q4_K(blocks, block_size, type_size, dtype=None):
     return (d * qs - dm).reshape((n_blocks, QK_K))
 
 
+def dequantize_blocks_Q5_K(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    d, dmin, scales, qh, qs = split_block_dims(blocks, 2, 2, K_SCALE_SIZE, QK_K // 8)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    dmin = _to(dmin.contiguous().view(torch.float16), dtype)
+    sc, m = get_scale_min(scales)
+    d = (d * sc).reshape((n_blocks, -1, 1))
+    dm = (dmin * m).reshape((n_blocks, -1, 1))
+    ql = qs.reshape((n_blocks, -1, 1, 32)) >> torch.tensor([0, 4], dtype=torch.uint8).reshape((1, 1, 2, 1))
+    qh = qh.reshape((n_blocks, -1, 1, 32)) >> torch.arange(8, dtype=torch.uint8).reshape((1, 1, 8, 1))
+    ql = (ql & 0x0F).reshape((n_blocks, -1, 32))
+    qh = (qh & 0x01).reshape((n_blocks, -1, 32))
+    q = ql | (qh << 4)
+    return (d * q - dm).reshape((n_blocks, QK_K))
+
+
 def dequantize_blocks_Q6_K(blocks, block_size, type_size, dtype=None):
     n_blocks = blocks.shape[0]
     ql, qh, scales, d = split_block_dims(blocks, QK_K // 2, QK_K // 4, QK_K // 16)
@@ -104,7 +120,8 @@ def dequantize_blocks_Q6_K(blocks, block_size, type_size, dtype=None):
     return (d * q).reshape((n_blocks, QK_K))
 
 
-dequantize_functions = {Q8_0: dequantize_blocks_Q8_0, Q4_K: dequantize_blocks_Q4_K, Q6_K: dequantize_blocks_Q6_K}
+dequantize_functions = {Q8_0: dequantize_blocks_Q8_0, Q4_K: dequantize_blocks_Q4_K, Q5_K: dequantize_blocks_Q5_K,
+                        Q6_K: dequantize_blocks_Q6_K}
 
 
 def dequantize_gguf_tensor(packed: torch.Tensor, quant_type: int, numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
@@ -193,6 +210,18 @@ def pack_q4_k(d, dmin, sc, mn, q) -> bytes:
         for l in range(32):
             qs.append(q[j + l] | (q[j + l + 32] << 4))
     return _f16_bytes(d) + _f16_bytes(dmin) + bytes(scales) + bytes(qs)
+
+
+def pack_q5_k(d, dmin, sc, mn, q) -> bytes:
+    """block_q5_K {f16 d, dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} from 8 scales, 8 mins (0..63), 256 quants (0..31)."""
+    q = [int(v) for v in q]
+    assert len(q) == 256 and all(0 <= v < 32 for v in q)
+    low = pack_q4_k(d, dmin, sc, mn, [v & 0x0F for v in q])   # same head, scale packing and nibble order
+    qh = [0] * 32
+    for j in range(8):
+        for l in range(32):
+            qh[l] |= (q[32 * j + l] >> 4) << j
+    return low[:16] + bytes(qh) + low[16:]
 
 
 def pack_q6_k(d, scales, q) -> bytes:

@@ -155,6 +155,41 @@ void sno_dequantize_row_q4_K(const uint8_t* src, float* y, int64_t k, int numeri
     }
 }
 
+/* block_q5_K { f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] } (176 bytes), ggml
+ * dequantize_row_q5_K: as Q4_K with a fifth bit per quant, bit j of qh[l] for element l of
+ * sub-block j.  upstream (numerics 1): dequantize_blocks_Q5_K, the rounding points of Q4_K. */
+void sno_dequantize_row_q5_K(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK_K;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 176;
+        float d = sno_f16_to_f32(rd16(blk));
+        float dmin = sno_f16_to_f32(rd16(blk + 2));
+        const uint8_t* scales = blk + 4;
+        const uint8_t* qh = blk + 16;
+        const uint8_t* qs = blk + 48;
+        float* out = y + b * QK_K;
+        for (int c = 0; c < 4; c++) {
+            uint8_t sc0, m0, sc1, m1;
+            scale_min_k4(2 * c, scales, &sc0, &m0);
+            scale_min_k4(2 * c + 1, scales, &sc1, &m1);
+            float d0 = d * (float)sc0, mm0 = dmin * (float)m0;
+            float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+            if (numerics) { d0 = r16(d0); mm0 = r16(mm0); d1 = r16(d1); mm1 = r16(mm1); }
+            for (int l = 0; l < 32; l++) {
+                float lo = (float)((qs[32 * c + l] & 0x0F) | (((qh[l] >> (2 * c)) & 1) << 4));
+                float hi = (float)((qs[32 * c + l] >> 4) | (((qh[l] >> (2 * c + 1)) & 1) << 4));
+                if (numerics) {
+                    out[64 * c + l] = r16(r16(d0 * lo) - mm0);
+                    out[64 * c + 32 + l] = r16(r16(d1 * hi) - mm1);
+                } else {
+                    out[64 * c + l] = d0 * lo - mm0;
+                    out[64 * c + 32 + l] = d1 * hi - mm1;
+                }
+            }
+        }
+    }
+}
+
 /* ggml dequantize_row_q6_K: per 128-element half, 32 lanes l give elements l, l+32, l+64,
  * l+96; y = d*scale[e/16]*(q-32).  Upstream: D=R(d*scale), y=R(D*(q-32)). */
 void sno_dequantize_row_q6_K(const uint8_t* src, float* y, int64_t k, int numerics) {
@@ -193,13 +228,14 @@ void sno_dequantize_row_q6_K(const uint8_t* src, float* y, int64_t k, int numeri
     }
 }
 
-int64_t sno_type_size(int qtype) { return qtype == 8 ? 34 : qtype == 12 ? 144 : qtype == 14 ? 210 : 0; }
-int64_t sno_block_size(int qtype) { return qtype == 8 ? 32 : (qtype == 12 || qtype == 14) ? 256 : 0; }
+int64_t sno_type_size(int qtype) { return qtype == 8 ? 34 : qtype == 12 ? 144 : qtype == 13 ? 176 : qtype == 14 ? 210 : 0; }
+int64_t sno_block_size(int qtype) { return qtype == 8 ? 32 : (qtype == 12 || qtype == 13 || qtype == 14) ? 256 : 0; }
 
 static int dequant_row(const uint8_t* src, int qtype, float* y, int64_t k, int numerics) {
     switch (qtype) {
     case 8: sno_dequantize_row_q8_0(src, y, k, numerics); return 0;
     case 12: sno_dequantize_row_q4_K(src, y, k, numerics); return 0;
+    case 13: sno_dequantize_row_q5_K(src, y, k, numerics); return 0;
     case 14: sno_dequantize_row_q6_K(src, y, k, numerics); return 0;
     default: return -1;
     }

@@ -23,7 +23,9 @@ namespace {
 constexpr int64_t kMaxDim = (int64_t)1 << 31;  // kernels index rows / columns with 32-bit tile counters
 
 inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
-inline bool known_type(int t) { return t == SNGGUF_TYPE_Q8_0 || t == SNGGUF_TYPE_Q4_K || t == SNGGUF_TYPE_Q6_K; }
+inline bool known_type(int t) {
+    return t == SNGGUF_TYPE_Q8_0 || t == SNGGUF_TYPE_Q4_K || t == SNGGUF_TYPE_Q5_K || t == SNGGUF_TYPE_Q6_K;
+}
 inline bool known_numerics(int n) { return n == SNGGUF_NUM_GGML_FP32 || n == SNGGUF_NUM_UPSTREAM_FP16; }
 
 // Shape / pointer checks shared by the matmul entry points.
@@ -57,11 +59,11 @@ const char* sngguf_strerror(int code) {
 }
 
 int64_t sngguf_type_size(int qtype) {
-    return qtype == SNGGUF_TYPE_Q8_0 ? 34 : qtype == SNGGUF_TYPE_Q4_K ? 144 : qtype == SNGGUF_TYPE_Q6_K ? 210 : 0;
+    return qtype == SNGGUF_TYPE_Q8_0 ? 34 : qtype == SNGGUF_TYPE_Q4_K ? 144 : qtype == SNGGUF_TYPE_Q5_K ? 176 : qtype == SNGGUF_TYPE_Q6_K ? 210 : 0;
 }
 
 int64_t sngguf_block_size(int qtype) {
-    return qtype == SNGGUF_TYPE_Q8_0 ? 32 : (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q6_K) ? 256 : 0;
+    return qtype == SNGGUF_TYPE_Q8_0 ? 32 : (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q5_K || qtype == SNGGUF_TYPE_Q6_K) ? 256 : 0;
 }
 
 int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,

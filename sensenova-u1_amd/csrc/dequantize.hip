@@ -69,6 +69,7 @@ int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(p, rows, cols, out, out_dtype, numerics, stream);
     case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(p, rows, cols, out, out_dtype, numerics, stream);
+    case SNGGUF_TYPE_Q5_K: return launch_num<SNGGUF_TYPE_Q5_K>(p, rows, cols, out, out_dtype, numerics, stream);
     case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(p, rows, cols, out, out_dtype, numerics, stream);
     default: return SNGGUF_E_BADTYPE;
     }

@@ -222,6 +222,7 @@ static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t s
     switch (qtype) {
     case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(a, numerics, stream);
     case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(a, numerics, stream);
+    case SNGGUF_TYPE_Q5_K: return launch_num<SNGGUF_TYPE_Q5_K>(a, numerics, stream);
     case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(a, numerics, stream);
     default: return SNGGUF_E_BADTYPE;
     }

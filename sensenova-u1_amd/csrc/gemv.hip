@@ -1,6 +1,6 @@
 // Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the path for Q8_0 rows that are not a
 // whole number of 256-element runs (the dispatcher at the end of this file sends Q8_0 with
-// K % 256 == 0 and all Q4_K / Q6_K shapes to the matrix-core kernels).
+// K % 256 == 0 and all Q4_K / Q5_K / Q6_K shapes to the matrix-core kernels).
 //
 // K % 64 == 0: one wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate
 // matrix and row n of the up matrix); a lane takes 64 weight elements (68 packed bytes) per step,
@@ -227,7 +227,7 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     bf16_t* yp = static_cast<bf16_t*>(y);
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
-    if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q6_K)
+    if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q5_K || qtype == SNGGUF_TYPE_Q6_K)
         return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
     // Q8_0 rows that are not a whole number of 256-element runs
     if (qtype == SNGGUF_TYPE_Q8_0) return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);

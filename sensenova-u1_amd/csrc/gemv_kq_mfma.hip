@@ -1,4 +1,4 @@
-// Q4_K / Q6_K decode GEMV on the matrix cores (1 <= M <= 16, K % 256 == 0).
+// Q4_K / Q5_K / Q6_K decode GEMV on the matrix cores (1 <= M <= 16, K % 256 == 0).
 //
 // Same shape as the Q8_0 kernel: a workgroup owns R * 16 weight rows (for the SiLU-gated pair the
 // same rows of the gate and of the up matrix, on separate wavefronts), its wavefronts split K by
@@ -6,7 +6,7 @@
 // (256 elements of each row):
 //   * the packed bytes of the R * 16 rows are fetched with 16-byte loads, consecutive lanes walking
 //     along a row, one super-block ahead, and dropped into the wavefront's private LDS slab.  Q4_K
-//     super-blocks (144 bytes) are 16-byte aligned; Q6_K super-blocks (210 bytes) are only 2-byte
+//     and Q5_K super-blocks (144 / 176 bytes) are 16-byte aligned; Q6_K super-blocks (210 bytes) are only 2-byte
 //     aligned and are fetched as 13 unaligned 16-byte pieces plus the 2-byte scale, which never
 //     touches a byte outside the super-block and puts every field at an aligned LDS address;
 //   * lane (r = lane % 16, g = lane / 16) decodes, for each 32-element sub-block j, elements
@@ -85,6 +85,10 @@ template <int QT> struct Slab;
 template <> struct Slab<SNGGUF_TYPE_Q4_K> {
     static constexpr int ts = 144, pieces = 9, stride = 144;
 };
+// Q5_K: 11 pieces per row and super-block (176 = 11 * 16); 44-dword rows fall on distinct bank groups
+template <> struct Slab<SNGGUF_TYPE_Q5_K> {
+    static constexpr int ts = 176, pieces = 11, stride = 176;
+};
 // Q6_K: 13 pieces (208 bytes) + the fp16 scale at byte 208; 240-byte rows fall on distinct banks
 template <> struct Slab<SNGGUF_TYPE_Q6_K> {
     static constexpr int ts = 210, pieces = 13, stride = 240;
@@ -112,6 +116,35 @@ __device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, i
             kq_dword_bf16<NUM, true>(ident, v0, 0.f, D, DM, a0, a1);
             kq_dword_bf16<NUM, true>(ident, v1, 0.f, D, DM, a2, a3);
             emit(j - 4 * HALF, u32x4_t{a0, a1, a2, a3});
+        }
+    }
+}
+
+// Q5_K: as Q4_K, the fifth bit of element l of sub-block j is bit j of qh[l]
+template <int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    typedef Num<NUM> A;
+    const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
+    const typename A::T d = A::scale((uint16_t)(head[0] & 0xFFFF)), dmin = A::scale((uint16_t)(head[0] >> 16));
+    const u32x2_t qh = *reinterpret_cast<const u32x2_t*>(row + 16 + 8 * g);
+#pragma unroll
+    for (int cc = 0; cc < 2; cc++) {
+        const int c = 2 * HALF + cc;
+        const u32x2_t qs = *reinterpret_cast<const u32x2_t*>(row + 48 + 32 * c + 8 * g);
+#pragma unroll
+        for (int hi = 0; hi < 2; hi++) {
+            const int j = 2 * c + hi;
+            uint32_t sc, mn;
+            q4k_scale_min(head[1], head[2], head[3], j, sc, mn);
+            const typename A::T D = d * A::integer((int)sc), DM = dmin * A::integer((int)mn);
+            uint32_t a[4];
+#pragma unroll
+            for (int w = 0; w < 2; w++) {
+                const uint32_t lo = (hi ? qs[w] >> 4 : qs[w]) & 0x0F0F0F0Fu;
+                const uint32_t hb = ((qh[w] >> j) & 0x01010101u) << 4;
+                kq_dword_bf16<NUM, true>(ident, lo | hb, 0.f, D, DM, a[2 * w], a[2 * w + 1]);
+            }
+            emit(j - 4 * HALF, u32x4_t{a[0], a[1], a[2], a[3]});
         }
     }
 }
@@ -238,6 +271,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                                                                   __builtin_bit_cast(bf16x8_t, xa[jj]), acc[rg], 0, 0, 0);
             };
             if constexpr (kQ6) decode_q6_k<NUM, 0>(ident, row, g, emit);
+            else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode_q5_k<NUM, 0>(ident, row, g, emit);
             else decode_q4_k<NUM, 0>(ident, row, g, emit);
         }
         if (s + 1 < s1) load_x(s + 1, 0, xa);
@@ -249,6 +283,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                                                                   __builtin_bit_cast(bf16x8_t, xb[jj]), acc[rg], 0, 0, 0);
             };
             if constexpr (kQ6) decode_q6_k<NUM, 1>(ident, row, g, emit);
+            else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode_q5_k<NUM, 1>(ident, row, g, emit);
             else decode_q4_k<NUM, 1>(ident, row, g, emit);
         }
     };
@@ -346,7 +381,7 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
 
 }  // namespace
 
-// Q4_K or Q6_K, 1 <= M <= 16, K % 256 == 0, 16-byte aligned x and q (checked by the caller).
+// Q4_K, Q5_K or Q6_K, 1 <= M <= 16, K % 256 == 0, 16-byte aligned x and q (checked by the caller).
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
@@ -358,6 +393,8 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
     if (qtype == QT && numerics == NUM) return launch_qt<QT, NUM>(xp, (int)M, a, b, N, K, bp, yp, gated, stream)
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_GGML_FP32);
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_UPSTREAM_FP16);
+    SNGGUF_CASE(SNGGUF_TYPE_Q5_K, SNGGUF_NUM_GGML_FP32);
+    SNGGUF_CASE(SNGGUF_TYPE_Q5_K, SNGGUF_NUM_UPSTREAM_FP16);
     SNGGUF_CASE(SNGGUF_TYPE_Q6_K, SNGGUF_NUM_GGML_FP32);
     SNGGUF_CASE(SNGGUF_TYPE_Q6_K, SNGGUF_NUM_UPSTREAM_FP16);
 #undef SNGGUF_CASE

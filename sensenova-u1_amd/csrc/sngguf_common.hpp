@@ -91,6 +91,7 @@ __device__ __forceinline__ uint32_t ld_u32(const uint8_t* p) { return *reinterpr
 template <int QT> struct Fmt;
 template <> struct Fmt<SNGGUF_TYPE_Q8_0> { static constexpr int bs = 32, ts = 34; };
 template <> struct Fmt<SNGGUF_TYPE_Q4_K> { static constexpr int bs = 256, ts = 144; };
+template <> struct Fmt<SNGGUF_TYPE_Q5_K> { static constexpr int bs = 256, ts = 176; };
 template <> struct Fmt<SNGGUF_TYPE_Q6_K> { static constexpr int bs = 256, ts = 210; };
 
 // Q4_K: 6-bit (scale, min) of sub-block j from the 12 packed bytes held as three dwords
@@ -152,6 +153,33 @@ __device__ __forceinline__ void decode8_q4_k(const uint8_t* __restrict__ row, in
     }
 }
 
+// Q5_K: Q4_K with a fifth quant bit, bit j of qh[l] for element l of sub-block j
+template <int NUM>
+__device__ __forceinline__ void decode8_q5_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
+    const uint8_t* blk = row + (e0 >> 8) * 176;  // 176 = 16 * 11: blocks stay 4-byte aligned when the row is
+    const int r = (int)(e0 & 255);
+    const int c = r >> 6;
+    const int hi = (r >> 5) & 1;
+    const int l0 = r & 31;
+    const int j = 2 * c + hi;
+    const uint32_t dd = ld_u32(blk);
+    uint32_t sc, mn;
+    q4k_scale_min(ld_u32(blk + 4), ld_u32(blk + 8), ld_u32(blk + 12), j, sc, mn);
+    const typename A::T D = A::scale((uint16_t)(dd & 0xFFFF)) * A::integer((int)sc);
+    const typename A::T DM = A::scale((uint16_t)(dd >> 16)) * A::integer((int)mn);
+    const uint8_t* qh = blk + 16 + l0;
+    const uint8_t* qs = blk + 48 + 32 * c + l0;
+    const uint32_t q0 = ld_u32(qs), q1 = ld_u32(qs + 4), h0 = ld_u32(qh), h1 = ld_u32(qh + 4);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t byte = ((i < 4 ? q0 : q1) >> (8 * (i & 3))) & 0xFFu;
+        const uint32_t hbit = (((i < 4 ? h0 : h1) >> (8 * (i & 3))) >> j) & 1u;
+        const int q = (int)((hi ? (byte >> 4) : (byte & 0x0Fu)) | (hbit << 4));
+        w[i] = A::widen(D * A::integer(q) - DM);
+    }
+}
+
 template <int NUM>
 __device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
     typedef Num<NUM> A;
@@ -181,6 +209,7 @@ template <int QT, int NUM>
 __device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
     if constexpr (QT == SNGGUF_TYPE_Q8_0) decode8_q8_0<NUM>(row, e0, w);
     else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode8_q4_k<NUM>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode8_q5_k<NUM>(row, e0, w);
     else decode8_q6_k<NUM>(row, e0, w);
 }
 

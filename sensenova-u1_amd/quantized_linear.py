@@ -24,6 +24,7 @@ from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType
 SUPPORTED_GGUF_QUANT_TYPES = (
     GGMLQuantizationType.Q8_0,
     GGMLQuantizationType.Q4_K,
+    GGMLQuantizationType.Q5_K,
     GGMLQuantizationType.Q6_K,
 )
 

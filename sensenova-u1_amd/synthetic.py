@@ -5,6 +5,7 @@ in HBM.
 * Q8_0: int8 quants uniform in [-127, 127], ``d = fp16(|N(0, 0.02)| / 127)``.
 * Q4_K: 4-bit quants uniform (all 128 quant bytes uniform), the 12 scale bytes uniform (so the
   eight 6-bit scales and mins are uniform over 0..63), ``d, dmin = fp16(|N(0, 0.01)|)``.
+* Q5_K: as Q4_K, with the 32 high-bit bytes uniform as well.
 * Q6_K: 6-bit quants uniform (ql, qh bytes uniform), int8 sub-scales uniform over the signed
   6-bit range [-32, 31], ``d = fp16(|N(0, 0.01)|)``.
 * activations: bf16 N(0, 1).
@@ -13,7 +14,7 @@ from __future__ import annotations
 
 import torch
 
-from .ops import GGML_QUANT_SIZES, Q4_K, Q6_K, Q8_0
+from .ops import GGML_QUANT_SIZES, Q4_K, Q5_K, Q6_K, Q8_0
 
 
 def _gen(seed: int, device) -> torch.Generator:
@@ -46,6 +47,10 @@ def make_packed(quant_type: int, n: int, k: int, seed: int = 0, device="cpu") ->
         blocks[..., 0:2] = _f16_bytes(absnormal(0.01))
         blocks[..., 2:4] = _f16_bytes(absnormal(0.01))
         blocks[..., 4:] = torch.randint(0, 256, (n, nb, 140), generator=g, device=device, dtype=torch.int16).to(torch.uint8)
+    elif quant_type == Q5_K:
+        blocks[..., 0:2] = _f16_bytes(absnormal(0.01))
+        blocks[..., 2:4] = _f16_bytes(absnormal(0.01))
+        blocks[..., 4:] = torch.randint(0, 256, (n, nb, 172), generator=g, device=device, dtype=torch.int16).to(torch.uint8)
     elif quant_type == Q6_K:
         blocks[..., 0:192] = torch.randint(0, 256, (n, nb, 192), generator=g, device=device, dtype=torch.int16).to(torch.uint8)
         sc = torch.randint(-32, 32, (n, nb, 16), generator=g, device=device, dtype=torch.int16)

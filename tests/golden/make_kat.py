@@ -6,6 +6,7 @@ comments, so the file pins the oracle against the format definition itself.
 
     block_q8_0 { f16 d; int8 qs[32]; }                                   34 bytes
     block_q4_K { f16 d; f16 dmin; u8 scales[12]; u8 qs[128]; }          144 bytes
+    block_q5_K { f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]; } 176 bytes
     block_q6_K { u8 ql[128]; u8 qh[64]; int8 scales[16]; f16 d; }       210 bytes
 
 Run from this directory: ``python make_kat.py``.
@@ -62,6 +63,34 @@ exp["0"] = 3.0
 exp["32"] = 20.0
 exp["255"] = 8 * 15 - 17.5
 kats.append({"name": "q4_k high scale bits and nibble order", "type": 12, "hex": hexs, "fill": 0.0, "expect": exp,
+             "how": "see make_kat.py"})
+
+# --- Q5_K: the Q4_K head above (d = 1, dmin = 0.5, sc = [1,2,3,4,21,6,7,8], m = [0,0,0,2,0,0,0,35]), then
+# qh[32], then qs[128].  Element l of sub-block j takes its fifth bit from bit j of qh[l]:
+#   qs[0] = 0xA3, qh[0] = 0b00000011 -> element 0 = 3 + 16 = 19 (sub-block 0), element 32 = 10 + 16 = 26 (sub-block 1)
+#   qs[127] = 0xF0 (chunk 3, l = 31), qh[31] = 0b10000000 -> element 223 = 0 (sub-block 6, bit 6 clear),
+#                                                          element 255 = 15 + 16 = 31 (sub-block 7)
+#   qh[5] = 0b00010000 with qs[64 + 5] = 0x00 -> element 128 + 5 = 133 (sub-block 4, l = 5) = 16
+# value = d*sc_j*q - dmin*m_j: element 0 = 19, element 32 = 2*26 = 52, element 133 = 21*16 = 336,
+# element 255 = 8*31 - 17.5 = 230.5; the rest of sub-block 3 is -1, the rest of sub-block 7 is -17.5.
+qs = ["00"] * 128
+qs[0] = "a3"
+qs[127] = "f0"
+qh = ["00"] * 32
+qh[0] = "03"
+qh[31] = "80"
+qh[5] = "10"
+hexs = "003c" + "0038" + "41020304" + "00000082" + "05060738" + "".join(qh) + "".join(qs)
+exp = {}
+for e in range(96, 128):
+    exp[str(e)] = -1.0
+for e in range(224, 256):
+    exp[str(e)] = -17.5
+exp["0"] = 19.0
+exp["32"] = 52.0
+exp["133"] = 336.0
+exp["255"] = 8 * 31 - 17.5
+kats.append({"name": "q5_k fifth bit by sub-block", "type": 13, "hex": hexs, "fill": 0.0, "expect": exp,
              "how": "see make_kat.py"})
 
 # --- Q6_K: d = 2.0 (f16 0x4000, "0040"); scales all 1 except scales[9] = 0xFD = -3.

@@ -30,7 +30,8 @@ def test_host_only_entry_points():
     assert (lib.sngguf_block_size(8), lib.sngguf_type_size(8)) == (32, 34)
     assert (lib.sngguf_block_size(12), lib.sngguf_type_size(12)) == (256, 144)
     assert (lib.sngguf_block_size(14), lib.sngguf_type_size(14)) == (256, 210)
-    assert lib.sngguf_block_size(13) == 0 and lib.sngguf_type_size(2) == 0
+    assert (lib.sngguf_block_size(13), lib.sngguf_type_size(13)) == (256, 176)
+    assert lib.sngguf_block_size(11) == 0 and lib.sngguf_type_size(2) == 0
     assert lib.sngguf_grouped_workspace_bytes(1000) >= 4 * 1000 + 4
     assert lib.sngguf_strerror(0) == b"ok"
     for code in range(-6, 0):
@@ -44,7 +45,7 @@ def test_argument_validation_needs_no_device():
     p = ctypes.c_void_p((ctypes.addressof(buf) + 63) // 64 * 64)
     odd = ctypes.c_void_p(p.value + 2)
     E_TYPE, E_SHAPE, E_NULL, E_ALIGN = -1, -2, -3, -4
-    assert lib.sngguf_dequantize(p, 13, 1, 256, p, 0, 0, None) == E_TYPE        # Q5_K not implemented
+    assert lib.sngguf_dequantize(p, 11, 1, 256, p, 0, 0, None) == E_TYPE        # Q3_K not implemented
     assert lib.sngguf_dequantize(p, 8, 1, 32, p, 7, 0, None) == E_TYPE          # bad out dtype
     assert lib.sngguf_dequantize(p, 8, 1, 32, p, 0, 5, None) == E_TYPE          # bad numerics
     assert lib.sngguf_dequantize(p, 8, 1, 33, p, 0, 0, None) == E_SHAPE         # cols % 32

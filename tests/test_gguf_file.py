@@ -106,4 +106,5 @@ def test_quant_sizes_table():
     assert GGML_QUANT_SIZES[GGMLQuantizationType.Q8_0] == (32, 34)
     assert GGML_QUANT_SIZES[GGMLQuantizationType.Q4_K] == (256, 2 + 2 + 12 + 128)
     assert GGML_QUANT_SIZES[GGMLQuantizationType.Q6_K] == (256, 128 + 64 + 16 + 2)
+    assert GGML_QUANT_SIZES[GGMLQuantizationType.Q5_K] == (256, 2 + 2 + 12 + 32 + 128)
     assert int(GGMLQuantizationType.Q8_0) == 8 and int(GGMLQuantizationType.Q4_K) == 12 and int(GGMLQuantizationType.Q6_K) == 14

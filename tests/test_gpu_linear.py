@@ -9,7 +9,7 @@ from sensenova_u1_amd import ops, synthetic
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-3          # rel-L2 bound on bf16 outputs
-TYPES = [go.Q8_0, go.Q4_K, go.Q6_K]
+TYPES = [go.Q8_0, go.Q4_K, go.Q5_K, go.Q6_K]
 
 
 def _check(got, want, tol=TOL):
@@ -48,7 +48,7 @@ def test_gemv_shapes_bias_ragged(dev, c_oracle, qt):
         _check(got, c_oracle.linear(x, packed, qt, bias))
 
 
-@pytest.mark.parametrize("qt", [go.Q4_K, go.Q6_K])
+@pytest.mark.parametrize("qt", [go.Q4_K, go.Q5_K, go.Q6_K])
 @pytest.mark.parametrize("numerics", [0, 1])
 def test_gemv_k_quants_two_row_groups(dev, c_oracle, qt, numerics):
     """N >= 32768 puts two 16-row groups on one wavefront: ragged N (last group half empty, last
@@ -232,7 +232,7 @@ def test_gate_up_silu(dev, c_oracle, qt, m):
     _check(got, c_oracle.silu_mul(g, u))
 
 
-@pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q4_K), (go.Q6_K, go.Q6_K), (go.Q4_K, go.Q6_K)])
+@pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q4_K), (go.Q6_K, go.Q6_K), (go.Q4_K, go.Q6_K), (go.Q5_K, go.Q8_0)])
 def test_grouped_linear_indicator(dev, qt_pair):
     print(f"case grouped indicator {qt_pair}", flush=True)
     qu, qg = qt_pair

@@ -22,7 +22,7 @@ def _load(tmp_path, dev, quant=8):
     return set_gguf2meta_model(model, sd, torch.bfloat16, dev).eval(), packed
 
 
-@pytest.mark.parametrize("quant", [8, 12, 14])
+@pytest.mark.parametrize("quant", [8, 12, 13, 14])
 def test_loaded_model_projections(tmp_path, dev, quant):
     print(f"case module quant={quant}", flush=True)
     model, packed = _load(tmp_path, dev, quant)

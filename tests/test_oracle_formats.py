@@ -17,7 +17,7 @@ import torch
 from oracle import gguf_oracle as go
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = [go.Q8_0, go.Q4_K, go.Q6_K]
+TYPES = [go.Q8_0, go.Q4_K, go.Q5_K, go.Q6_K]
 
 
 def _blocks(raw: bytes) -> torch.Tensor:
@@ -137,6 +137,40 @@ def test_q4_k_random_round_trip_closed_form(c_oracle):
         assert np.array_equal(out, exact.astype(np.float32))
 
 
+# ---- Q5_K ------------------------------------------------------------------------------------
+
+def test_q5_k_one_hot_positions(c_oracle):
+    sc, mn = [1] * 8, [0] * 8
+    for pos in list(range(0, 256, 7)) + [31, 32, 63, 64, 255]:
+        q = [0] * 256
+        q[pos] = 25          # nibble 9 and the fifth bit
+        out = _both(c_oracle, _blocks(go.pack_q5_k(1.0, 0.0, sc, mn, q)), go.Q5_K)
+        want = torch.zeros(256)
+        want[pos] = 25.0
+        assert torch.equal(out, want), pos
+        q[pos] = 16          # the fifth bit alone
+        out = _both(c_oracle, _blocks(go.pack_q5_k(1.0, 0.0, sc, mn, q)), go.Q5_K)
+        want[pos] = 16.0
+        assert torch.equal(out, want), pos
+
+
+def test_q5_k_scale_packing_and_closed_form(c_oracle):
+    sc = [1, 17, 33, 63, 2, 18, 47, 62]
+    mn = [63, 5, 21, 40, 59, 3, 16, 32]
+    q = [(7 * i + 3) % 32 for i in range(256)]
+    out = _both(c_oracle, _blocks(go.pack_q5_k(2.0, 0.5, sc, mn, q)), go.Q5_K).numpy()
+    want = np.array([2.0 * sc[i // 32] * q[i] - 0.5 * mn[i // 32] for i in range(256)], dtype=np.float32)
+    assert np.array_equal(out, want)
+    rng = np.random.default_rng(6)
+    for _ in range(50):
+        sc, mn = rng.integers(0, 64, 8), rng.integers(0, 64, 8)
+        q = rng.integers(0, 32, 256)
+        d, dmin = np.float16(abs(rng.standard_normal()) * 0.01), np.float16(abs(rng.standard_normal()) * 0.01)
+        out = _both(c_oracle, _blocks(go.pack_q5_k(d, dmin, sc, mn, q)), go.Q5_K).numpy()
+        exact = np.float64(d) * sc.repeat(32) * q - np.float64(dmin) * mn.repeat(32)
+        assert np.array_equal(out, exact.astype(np.float32))
+
+
 # ---- Q6_K ------------------------------------------------------------------------------------
 
 def test_q6_k_one_hot_positions(c_oracle):
@@ -176,7 +210,7 @@ def test_known_answer_blocks(c_oracle):
     (hex bytes) with expected values worked out on paper; see the file's "how" fields."""
     with open(os.path.join(HERE, "golden", "kat_blocks.json")) as f:
         kats = json.load(f)
-    assert len(kats) >= 6
+    assert len(kats) >= 7
     for kat in kats:
         packed = _blocks(bytes.fromhex(kat["hex"]))
         qt = kat["type"]
