@@ -364,7 +364,7 @@ def main() -> None:
 
         gate, up, down = (t.cpu() for t in layers[0])
         x = synthetic.make_activations(1, HIDDEN, seed=7)
-        reps, times = 3, []
+        reps, times = 15, []
         go.mlp_forward(x, gate[:256], up[:256], down[:, :256 // 32 * 34], (Q8_0, Q8_0, Q8_0))  # warm torch's thread pool
         for _ in range(reps):
             t0 = time.perf_counter()
