@@ -289,6 +289,25 @@ def test_full_size_shapes_row_sample(dev):
             _check(y[rows.to(dev)][:, cols.to(dev)].cpu(), want)
 
 
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K])
+def test_vocabulary_sized_projection(dev, qt):
+    """The largest linear of the model: lm_head, 151936 x 4096, at decode.  A sample of output
+    columns is checked against the oracle run on exactly those weight rows; the row count is not a
+    multiple of 256 and the byte offsets of the last rows exceed 2^29."""
+    print(f"case lm_head qt={qt}", flush=True)
+    n, k = 151936, 4096
+    packed = synthetic.make_packed(qt, n, k, seed=5, device=dev)
+    g = torch.Generator().manual_seed(1)
+    cols = torch.cat([torch.randint(0, n, (60,), generator=g), torch.tensor([0, n - 1, n - 17, 75967])])
+    sub = packed[cols.to(dev)].cpu()
+    for m in (1, 5):
+        x = synthetic.make_activations(m, k, seed=m, device=dev)
+        y = ops.linear(x, packed, qt)
+        assert y.shape == (m, n)
+        _check(y[:, cols.to(dev)].cpu(), go.gguf_linear_forward(x.cpu(), sub, qt))
+    assert torch.isfinite(y.float()).all()
+
+
 def test_linear_errors(dev):
     packed = synthetic.make_packed(go.Q8_0, 8, 64).to(dev)
     with pytest.raises(ops.SnGgufError):
