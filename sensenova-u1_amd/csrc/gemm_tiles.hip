@@ -14,9 +14,10 @@
 // B operand (v_mfma_f32_32x32x16_bf16), so a lane ends up with runs of four consecutive output
 // columns of one activation row.
 //
-// Tiles are numbered so that the workgroups that land on one XCD (workgroup id modulo 8) cover
-// few activation row tiles times all column tiles: those activation tiles stay in that XCD's L2
-// while the (smaller) packed weight tiles stream through.
+// Tiles are numbered so that the workgroups that land on one XCD (workgroup id modulo 8) work on a
+// contiguous range of tiles, and within it on blocks of 4 row tiles x 8 column tiles at a time: the
+// 32 workgroups that run together on an XCD then share 4 activation tiles and 8 packed weight
+// tiles in that XCD's L2.
 #include "gemm_args.hpp"
 #include "sngguf_common.hpp"
 
@@ -108,7 +109,19 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     const int64_t per = total >> 3, rem = total & 7;
     const int64_t xcd = pid & 7, idx = pid >> 3;
     const int64_t tile = xcd * per + (xcd < rem ? xcd : rem) + idx;
-    const int64_t ty = tile / ntn, tn = tile - ty * ntn;
+    // The 32 workgroups that run at the same time on one XCD cover a block of 4 row tiles x 8 column
+    // tiles when the tile grid divides that way (4 activation tiles + 8 packed weight tiles pass
+    // through the XCD's L2 per block instead of 1 + 32), else 32 consecutive column tiles of one row.
+    int64_t ty, tn;
+    constexpr int BY = 4, BX = 8;
+    if ((ntn % BX) == 0 && ((t0 + t1) % BY) == 0) {
+        const int64_t blk = tile >> 5, within = tile & 31, bpr = ntn / BX;   // blocks per block row
+        ty = (blk / bpr) * BY + (within / BX);
+        tn = (blk % bpr) * BX + (within % BX);
+    } else {
+        ty = tile / ntn;
+        tn = tile - ty * ntn;
+    }
     int g;
     int64_t row_begin, row_end;
     if (ty < t0) {

@@ -140,9 +140,10 @@ def test_gemm_ragged_bias(dev, qt):
 @pytest.mark.parametrize("numerics", [0, 1])
 def test_gemm_q8_0_large_tile_kernel(dev, c_oracle, numerics):
     """M >= 384 with K % 64 == 0 takes the 256 x 256 tile kernel: ragged M / N, bias, one K step,
-    odd and even step counts."""
+    odd and even step counts, a tile grid that divides into 4 x 8 blocks (blocked tile order) and
+    grids that do not."""
     print(f"case gemm tiles numerics={numerics}", flush=True)
-    for m, n, k in [(2816, 2816, 64), (3000, 2904, 320), (3000, 2900, 192), (4100, 2050, 128), (8300, 1030, 64)]:
+    for m, n, k in [(2816, 2816, 64), (2048, 4096, 128), (3000, 2904, 320), (3000, 2900, 192), (4100, 2050, 128), (8300, 1030, 64)]:
         packed = synthetic.make_packed(go.Q8_0, n, k, seed=m + n + k)
         x = synthetic.make_activations(m, k, seed=m)
         bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
@@ -159,7 +160,7 @@ def test_gemm_q4_k_large_tile_kernel(dev, c_oracle, numerics):
     """Q4_K through the 256 x 256 tile kernel (M >= 384, at least 128 tiles): every chunk position of
     a super-block (K steps 0..3 and beyond), ragged M / N, both output paths, bias."""
     print(f"case gemm q4_k tiles numerics={numerics}", flush=True)
-    for m, n, k in [(3000, 2904, 256), (4100, 2050, 512), (3072, 3080, 1280)]:
+    for m, n, k in [(2048, 4096, 256), (3000, 2904, 256), (4100, 2050, 512), (3072, 3080, 1280)]:
         packed = synthetic.make_packed(go.Q4_K, n, k, seed=m + n + k)
         x = synthetic.make_activations(m, k, seed=m)
         bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
