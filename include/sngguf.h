@@ -26,7 +26,13 @@ extern "C" {
 /* ggml tensor type numbers (gguf.GGMLQuantizationType, the `quant_type` that
  * src/sensenova_u1/utils/gguf_loader.py:37-43 stores on each GGUFParameter). */
 enum {
+    SNGGUF_TYPE_Q4_0 = 2,  /* 32 elements / 18 bytes:  f16 d; u8 qs[16]                          */
+    SNGGUF_TYPE_Q4_1 = 3,  /* 32 elements / 20 bytes:  f16 d, m; u8 qs[16]                       */
+    SNGGUF_TYPE_Q5_0 = 6,  /* 32 elements / 22 bytes:  f16 d; u8 qh[4]; u8 qs[16]                */
+    SNGGUF_TYPE_Q5_1 = 7,  /* 32 elements / 24 bytes:  f16 d, m; u8 qh[4]; u8 qs[16]             */
     SNGGUF_TYPE_Q8_0 = 8,  /* 32 elements / 34 bytes:  f16 d; i8 qs[32]                         */
+    SNGGUF_TYPE_Q2_K = 10, /* 256 elements / 84 bytes:  u8 scales[16]; u8 qs[64]; f16 d, dmin    */
+    SNGGUF_TYPE_Q3_K = 11, /* 256 elements / 110 bytes: u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d */
     SNGGUF_TYPE_Q4_K = 12, /* 256 elements / 144 bytes: f16 d, dmin; u8 scales[12]; u8 qs[128]  */
     SNGGUF_TYPE_Q5_K = 13, /* 256 elements / 176 bytes: f16 d, dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] */
     SNGGUF_TYPE_Q6_K = 14  /* 256 elements / 210 bytes: u8 ql[128]; u8 qh[64]; i8 sc[16]; f16 d */

@@ -32,11 +32,14 @@ import subprocess
 import numpy as np
 import torch
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 2, 3, 6, 7, 8, 10, 11, 12, 13, 14
 QK_K = 256
 K_SCALE_SIZE = 12
 # gguf.GGML_QUANT_SIZES: type -> (elements per block, bytes per block)
-GGML_QUANT_SIZES = {Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
+GGML_QUANT_SIZES = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
+                    Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
+TYPE_NAMES = {Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q8_0", Q2_K: "Q2_K", Q3_K: "Q3_K",
+              Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
 
 NUM_GGML_FP32 = 0
 NUM_UPSTREAM_FP16 = 1
@@ -63,6 +66,92 @@ def dequantize_blocks_Q8_0(blocks, block_size, type_size, dtype=None):
     d = _to(d.contiguous().view(torch.float16), dtype)
     x = x.contiguous().view(torch.int8)
     return d * x
+
+
+def to_uint32(x: torch.Tensor) -> torch.Tensor:
+    """Four little-endian bytes per row -> one int32 column."""
+    x = x.contiguous().view(torch.uint8).to(torch.int32)
+    return (x[:, 0] | x[:, 1] << 8 | x[:, 2] << 16 | x[:, 3] << 24).unsqueeze(1)
+
+
+def _nibbles(qs: torch.Tensor, n_blocks: int, block_size: int) -> torch.Tensor:
+    """16 bytes -> 32 values: all low nibbles, then all high nibbles."""
+    ql = qs.reshape((n_blocks, -1, 1, block_size // 2)) >> torch.tensor([0, 4], dtype=torch.uint8).reshape((1, 1, 2, 1))
+    return (ql & 0x0F).reshape((n_blocks, -1))
+
+
+def _fifth_bits(qh: torch.Tensor, n_blocks: int) -> torch.Tensor:
+    qh = to_uint32(qh)
+    qh = qh.reshape((n_blocks, 1)) >> torch.arange(32, dtype=torch.int32).reshape((1, 32))
+    return (qh & 1).to(torch.uint8)
+
+
+def dequantize_blocks_Q4_0(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    d, qs = split_block_dims(blocks, 2)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    qs = _nibbles(qs, n_blocks, block_size).to(torch.int8) - 8
+    return d * qs
+
+
+def dequantize_blocks_Q4_1(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    d, m, qs = split_block_dims(blocks, 2, 2)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    m = _to(m.contiguous().view(torch.float16), dtype)
+    qs = _nibbles(qs, n_blocks, block_size)
+    return (d * qs) + m
+
+
+def dequantize_blocks_Q5_0(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    d, qh, qs = split_block_dims(blocks, 2, 4)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    qs = (_nibbles(qs, n_blocks, block_size) | (_fifth_bits(qh, n_blocks) << 4)).to(torch.int8) - 16
+    return d * qs
+
+
+def dequantize_blocks_Q5_1(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    d, m, qh, qs = split_block_dims(blocks, 2, 2, 4)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    m = _to(m.contiguous().view(torch.float16), dtype)
+    qs = _nibbles(qs, n_blocks, block_size) | (_fifth_bits(qh, n_blocks) << 4)
+    return (d * qs) + m
+
+
+def dequantize_blocks_Q2_K(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    scales, qs, d, dmin = split_block_dims(blocks, QK_K // 16, QK_K // 4, 2)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    dmin = _to(dmin.contiguous().view(torch.float16), dtype)
+    dl = (d * (scales & 0xF)).reshape((n_blocks, QK_K // 16, 1))
+    ml = (dmin * (scales >> 4)).reshape((n_blocks, QK_K // 16, 1))
+    shift = torch.tensor([0, 2, 4, 6], dtype=torch.uint8).reshape((1, 1, 4, 1))
+    qs = (qs.reshape((n_blocks, -1, 1, 32)) >> shift) & 3
+    qs = qs.reshape((n_blocks, QK_K // 16, 16))
+    qs = dl * qs - ml
+    return qs.reshape((n_blocks, -1))
+
+
+def dequantize_blocks_Q3_K(blocks, block_size, type_size, dtype=None):
+    n_blocks = blocks.shape[0]
+    hmask, qs, scales, d = split_block_dims(blocks, QK_K // 8, QK_K // 4, 12)
+    d = _to(d.contiguous().view(torch.float16), dtype)
+    lscales, hscales = scales[:, :8], scales[:, 8:]
+    lscales = lscales.reshape((n_blocks, 1, 8)) >> torch.tensor([0, 4], dtype=torch.uint8).reshape((1, 2, 1))
+    lscales = lscales.reshape((n_blocks, 16))
+    hscales = hscales.reshape((n_blocks, 1, 4)) >> torch.tensor([0, 2, 4, 6], dtype=torch.uint8).reshape((1, 4, 1))
+    hscales = hscales.reshape((n_blocks, 16))
+    scales = (lscales & 0x0F) | ((hscales & 0x03) << 4)
+    scales = scales.to(torch.int8) - 32
+    dl = (d * scales).reshape((n_blocks, 16, 1))
+    ql = qs.reshape((n_blocks, -1, 1, 32)) >> torch.tensor([0, 2, 4, 6], dtype=torch.uint8).reshape((1, 1, 4, 1))
+    qh = hmask.reshape((n_blocks, -1, 1, 32)) >> torch.arange(8, dtype=torch.uint8).reshape((1, 1, 8, 1))
+    ql = ql.reshape((n_blocks, 16, QK_K // 16)) & 3
+    qh = (qh.reshape((n_blocks, 16, QK_K // 16)) & 1) ^ 1
+    q = ql.to(torch.int8) - (qh << 2).to(torch.int8)
+    return (dl * q).reshape((n_blocks, QK_K))
 
 
 def get_scale_min(scales: torch.Tensor):
@@ -120,7 +209,9 @@ def dequantize_blocks_Q6_K(blocks, block_size, type_size, dtype=None):
     return (d * q).reshape((n_blocks, QK_K))
 
 
-dequantize_functions = {Q8_0: dequantize_blocks_Q8_0, Q4_K: dequantize_blocks_Q4_K, Q5_K: dequantize_blocks_Q5_K,
+dequantize_functions = {Q4_0: dequantize_blocks_Q4_0, Q4_1: dequantize_blocks_Q4_1, Q5_0: dequantize_blocks_Q5_0,
+                        Q5_1: dequantize_blocks_Q5_1, Q8_0: dequantize_blocks_Q8_0, Q2_K: dequantize_blocks_Q2_K,
+                        Q3_K: dequantize_blocks_Q3_K, Q4_K: dequantize_blocks_Q4_K, Q5_K: dequantize_blocks_Q5_K,
                         Q6_K: dequantize_blocks_Q6_K}
 
 
@@ -186,6 +277,95 @@ def pack_q8_0(d, qs) -> bytes:
     qs = np.asarray(qs, dtype=np.int8)
     assert qs.shape == (32,)
     return _f16_bytes(d) + qs.tobytes()
+
+
+def _pack_nibbles_32(q) -> bytes:
+    """ggml quantize_row_q4_0_ref packing: byte j holds element j (low) and element j + 16 (high)."""
+    return bytes((q[j] & 0x0F) | ((q[j + 16] & 0x0F) << 4) for j in range(16))
+
+
+def _pack_fifth_bits_32(q) -> bytes:
+    """ggml quantize_row_q5_0_ref: bit j of the 32-bit qh is bit 4 of element j."""
+    qh = 0
+    for j in range(32):
+        qh |= ((q[j] >> 4) & 1) << j
+    return int(qh).to_bytes(4, "little")
+
+
+def pack_q4_0(d, q) -> bytes:
+    """block_q4_0 {f16 d; u8 qs[16]} from 32 signed quants (-8..7), stored with offset 8."""
+    q = [int(v) + 8 for v in q]
+    assert len(q) == 32 and all(0 <= v < 16 for v in q)
+    return _f16_bytes(d) + _pack_nibbles_32(q)
+
+
+def pack_q4_1(d, m, q) -> bytes:
+    """block_q4_1 {f16 d; f16 m; u8 qs[16]} from 32 quants (0..15)."""
+    q = [int(v) for v in q]
+    assert len(q) == 32 and all(0 <= v < 16 for v in q)
+    return _f16_bytes(d) + _f16_bytes(m) + _pack_nibbles_32(q)
+
+
+def pack_q5_0(d, q) -> bytes:
+    """block_q5_0 {f16 d; u8 qh[4]; u8 qs[16]} from 32 signed quants (-16..15), stored with offset 16."""
+    q = [int(v) + 16 for v in q]
+    assert len(q) == 32 and all(0 <= v < 32 for v in q)
+    return _f16_bytes(d) + _pack_fifth_bits_32(q) + _pack_nibbles_32(q)
+
+
+def pack_q5_1(d, m, q) -> bytes:
+    """block_q5_1 {f16 d; f16 m; u8 qh[4]; u8 qs[16]} from 32 quants (0..31)."""
+    q = [int(v) for v in q]
+    assert len(q) == 32 and all(0 <= v < 32 for v in q)
+    return _f16_bytes(d) + _f16_bytes(m) + _pack_fifth_bits_32(q) + _pack_nibbles_32(q)
+
+
+def _pack_bit_pairs_256(q) -> bytes:
+    """ggml quantize_row_q2_K_ref / q3_K packing of the two low bits: per 128 elements, byte l holds
+    elements l, l + 32, l + 64, l + 96 at bits 0, 2, 4, 6."""
+    out = []
+    for j in range(0, 256, 128):
+        for l in range(32):
+            out.append((q[j + l] & 3) | ((q[j + l + 32] & 3) << 2) | ((q[j + l + 64] & 3) << 4) | ((q[j + l + 96] & 3) << 6))
+    return bytes(out)
+
+
+def pack_q2_k(d, dmin, sc, mn, q) -> bytes:
+    """block_q2_K {u8 scales[16]; u8 qs[64]; f16 d, dmin} from 16 scales, 16 mins (0..15), 256 quants (0..3)."""
+    sc = [int(v) for v in sc]
+    mn = [int(v) for v in mn]
+    q = [int(v) for v in q]
+    assert len(sc) == 16 and len(mn) == 16 and len(q) == 256
+    assert all(0 <= v < 16 for v in sc + mn) and all(0 <= v < 4 for v in q)
+    scales = bytes(sc[j] | (mn[j] << 4) for j in range(16))
+    return scales + _pack_bit_pairs_256(q) + _f16_bytes(d) + _f16_bytes(dmin)
+
+
+def pack_q3_k(d, sc, q) -> bytes:
+    """block_q3_K {u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d} from 16 signed scales (-32..31) and 256
+    signed quants (-4..3); stored as ggml's quantize_row_q3_K_ref does: scale + 32 split 4 + 2 bits, quant + 4
+    with bit 2 in hmask and bits 0..1 in qs."""
+    sc = [int(v) + 32 for v in sc]
+    q = [int(v) + 4 for v in q]
+    assert len(sc) == 16 and len(q) == 256
+    assert all(0 <= v < 64 for v in sc) and all(0 <= v < 8 for v in q)
+    scales = [0] * 12
+    for j in range(16):
+        l = sc[j]
+        if j < 8:
+            scales[j] = l & 0xF
+        else:
+            scales[j - 8] |= (l & 0xF) << 4
+        scales[8 + j % 4] |= (l >> 4) << (2 * (j // 4))
+    hmask = [0] * 32
+    m, hm = 0, 1
+    for j in range(256):
+        if q[j] > 3:
+            hmask[m] |= hm
+        m += 1
+        if m == 32:
+            m, hm = 0, hm << 1
+    return bytes(hmask) + _pack_bit_pairs_256([v & 3 for v in q]) + bytes(scales) + _f16_bytes(d)
 
 
 def pack_q4_k(d, dmin, sc, mn, q) -> bytes:

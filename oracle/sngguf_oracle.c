@@ -5,11 +5,11 @@
  *
  * What it restates.  The reference glue (src/sensenova_u1/utils/gguf_loader.py:17-85) hands
  * every quantized tensor to diffusers 0.37.1 (uv.lock:164-165), whose GGUFLinear.forward is
- *     w = dequantize_gguf_tensor(weight)      # dequantize_blocks_Q8_0 / _Q4_K / _Q6_K
+ *     w = dequantize_gguf_tensor(weight)      # dequantize_blocks_Q8_0 / _Q4_K / _Q6_K / ...
  *     w = w.to(compute_dtype)                 # bf16
  *     y = F.linear(x, w, bias)
- * and whose block decoders restate ggml's dequantize_row_q8_0 / q4_K / q6_K and
- * get_scale_min_k4.  Neither package's source is in the reference tree, so the functions
+ * and whose block decoders restate ggml's dequantize_row_q8_0 / q4_K / q6_K (and the other
+ * q4_0 ... q5_K formats) and get_scale_min_k4.  Neither package's source is in the reference tree, so the functions
  * below restate the published ggml block formats (numerics 0) and the upstream torch op
  * sequence with its fp16 intermediates (numerics 1).
  *
@@ -228,12 +228,175 @@ void sno_dequantize_row_q6_K(const uint8_t* src, float* y, int64_t k, int numeri
     }
 }
 
-int64_t sno_type_size(int qtype) { return qtype == 8 ? 34 : qtype == 12 ? 144 : qtype == 13 ? 176 : qtype == 14 ? 210 : 0; }
-int64_t sno_block_size(int qtype) { return qtype == 8 ? 32 : (qtype == 12 || qtype == 13 || qtype == 14) ? 256 : 0; }
+/* ---- legacy 32-element blocks --------------------------------------------------------- */
+
+/* block_q4_0 { f16 d; u8 qs[16] } (18 bytes), ggml dequantize_row_q4_0: element l is the low
+ * nibble of qs[l], element l+16 the high nibble; y = d * (q - 8).
+ * upstream dequantize_blocks_Q4_0: R(d * (q - 8)). */
+void sno_dequantize_row_q4_0(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / 32;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 18;
+        float d = sno_f16_to_f32(rd16(blk));
+        for (int l = 0; l < 16; l++) {
+            float v0 = d * (float)((int)(blk[2 + l] & 0x0F) - 8);
+            float v1 = d * (float)((int)(blk[2 + l] >> 4) - 8);
+            y[b * 32 + l] = numerics ? r16(v0) : v0;
+            y[b * 32 + l + 16] = numerics ? r16(v1) : v1;
+        }
+    }
+}
+
+/* block_q4_1 { f16 d; f16 m; u8 qs[16] } (20 bytes), ggml dequantize_row_q4_1: y = d * q + m.
+ * upstream dequantize_blocks_Q4_1: R(R(d * q) + m). */
+void sno_dequantize_row_q4_1(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / 32;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 20;
+        float d = sno_f16_to_f32(rd16(blk));
+        float m = sno_f16_to_f32(rd16(blk + 2));
+        for (int l = 0; l < 16; l++) {
+            float q0 = (float)(blk[4 + l] & 0x0F), q1 = (float)(blk[4 + l] >> 4);
+            y[b * 32 + l] = numerics ? r16(r16(d * q0) + m) : d * q0 + m;
+            y[b * 32 + l + 16] = numerics ? r16(r16(d * q1) + m) : d * q1 + m;
+        }
+    }
+}
+
+/* block_q5_0 { f16 d; u8 qh[4]; u8 qs[16] } (22 bytes), ggml dequantize_row_q5_0: bit e of the
+ * little-endian 32-bit qh is the fifth bit of element e; y = d * (q - 16).
+ * upstream dequantize_blocks_Q5_0: R(d * (q - 16)). */
+void sno_dequantize_row_q5_0(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / 32;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 22;
+        float d = sno_f16_to_f32(rd16(blk));
+        uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        for (int l = 0; l < 16; l++) {
+            int q0 = (int)((blk[6 + l] & 0x0F) | (((qh >> l) & 1u) << 4)) - 16;
+            int q1 = (int)((blk[6 + l] >> 4) | (((qh >> (l + 16)) & 1u) << 4)) - 16;
+            float v0 = d * (float)q0, v1 = d * (float)q1;
+            y[b * 32 + l] = numerics ? r16(v0) : v0;
+            y[b * 32 + l + 16] = numerics ? r16(v1) : v1;
+        }
+    }
+}
+
+/* block_q5_1 { f16 d; f16 m; u8 qh[4]; u8 qs[16] } (24 bytes), ggml dequantize_row_q5_1:
+ * y = d * q + m with the 5-bit q of Q5_0 (no offset).  upstream: R(R(d * q) + m). */
+void sno_dequantize_row_q5_1(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / 32;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 24;
+        float d = sno_f16_to_f32(rd16(blk));
+        float m = sno_f16_to_f32(rd16(blk + 2));
+        uint32_t qh = (uint32_t)blk[4] | ((uint32_t)blk[5] << 8) | ((uint32_t)blk[6] << 16) | ((uint32_t)blk[7] << 24);
+        for (int l = 0; l < 16; l++) {
+            float q0 = (float)((blk[8 + l] & 0x0F) | (((qh >> l) & 1u) << 4));
+            float q1 = (float)((blk[8 + l] >> 4) | (((qh >> (l + 16)) & 1u) << 4));
+            y[b * 32 + l] = numerics ? r16(r16(d * q0) + m) : d * q0 + m;
+            y[b * 32 + l + 16] = numerics ? r16(r16(d * q1) + m) : d * q1 + m;
+        }
+    }
+}
+
+/* ---- 2- and 3-bit super-blocks ---------------------------------------------------------- */
+
+/* block_q2_K { u8 scales[16]; u8 qs[64]; f16 d; f16 dmin } (84 bytes), ggml dequantize_row_q2_K:
+ * per 128-element half, bit pair j of qs[32*half + l] is element 32*j + l; 16-element group g
+ * has scale scales[g] & 15 and min scales[g] >> 4; y = d*sc*q - dmin*mn.
+ * upstream dequantize_blocks_Q2_K: DL = R(d*sc), ML = R(dmin*mn), y = R(R(DL*q) - ML). */
+void sno_dequantize_row_q2_K(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK_K;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 84;
+        const uint8_t* scales = blk;
+        const uint8_t* qs = blk + 16;
+        float d = sno_f16_to_f32(rd16(blk + 80));
+        float dmin = sno_f16_to_f32(rd16(blk + 82));
+        float* out = y + b * QK_K;
+        int is = 0;
+        for (int half = 0; half < 2; half++) {
+            for (int j = 0; j < 4; j++) {
+                for (int part = 0; part < 2; part++) {
+                    uint8_t sc = scales[is++];
+                    float dl = d * (float)(sc & 0x0F), ml = dmin * (float)(sc >> 4);
+                    if (numerics) { dl = r16(dl); ml = r16(ml); }
+                    for (int l = 0; l < 16; l++) {
+                        float q = (float)((qs[32 * half + 16 * part + l] >> (2 * j)) & 3);
+                        out[128 * half + 32 * j + 16 * part + l] = numerics ? r16(r16(dl * q) - ml) : dl * q - ml;
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* block_q3_K { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d } (110 bytes), ggml
+ * dequantize_row_q3_K: the 6-bit scale of 16-element group g has its low nibble in
+ * scales[g % 8] (upper nibble for g >= 8) and its two high bits in scales[8 + g % 4] at bit
+ * 2*(g/4), offset by -32; the quant is the bit pair as in Q2_K minus 4 unless bit
+ * (4*half + j) of hmask[l] is set; y = d*(sc-32)*q.
+ * upstream dequantize_blocks_Q3_K: DL = R(d*(sc-32)), y = R(DL*q). */
+void sno_dequantize_row_q3_K(const uint8_t* src, float* y, int64_t k, int numerics) {
+    int64_t nb = k / QK_K;
+    for (int64_t b = 0; b < nb; b++) {
+        const uint8_t* blk = src + b * 110;
+        const uint8_t* hm = blk;
+        const uint8_t* qs = blk + 32;
+        const uint8_t* sp = blk + 96;
+        float d = sno_f16_to_f32(rd16(blk + 108));
+        float* out = y + b * QK_K;
+        int sc[16];
+        for (int g = 0; g < 16; g++) {
+            int lo = g < 8 ? (sp[g] & 0x0F) : (sp[g - 8] >> 4);
+            int hi = (sp[8 + (g & 3)] >> (2 * (g >> 2))) & 3;
+            sc[g] = (lo | (hi << 4)) - 32;
+        }
+        int is = 0;
+        for (int half = 0; half < 2; half++) {
+            for (int j = 0; j < 4; j++) {
+                for (int part = 0; part < 2; part++) {
+                    float dl = d * (float)sc[is++];
+                    if (numerics) dl = r16(dl);
+                    for (int l = 0; l < 16; l++) {
+                        int ll = 16 * part + l;
+                        int q = (int)((qs[32 * half + ll] >> (2 * j)) & 3) - (((hm[ll] >> (4 * half + j)) & 1) ? 0 : 4);
+                        float v = dl * (float)q;
+                        out[128 * half + 32 * j + ll] = numerics ? r16(v) : v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+
+/* ggml type enum -> bytes / elements per block (0: not restated here) */
+int64_t sno_type_size(int qtype) {
+    switch (qtype) {
+    case 2: return 18; case 3: return 20; case 6: return 22; case 7: return 24; case 8: return 34;
+    case 10: return 84; case 11: return 110; case 12: return 144; case 13: return 176; case 14: return 210;
+    default: return 0;
+    }
+}
+int64_t sno_block_size(int qtype) {
+    switch (qtype) {
+    case 2: case 3: case 6: case 7: case 8: return 32;
+    case 10: case 11: case 12: case 13: case 14: return 256;
+    default: return 0;
+    }
+}
 
 static int dequant_row(const uint8_t* src, int qtype, float* y, int64_t k, int numerics) {
     switch (qtype) {
+    case 2: sno_dequantize_row_q4_0(src, y, k, numerics); return 0;
+    case 3: sno_dequantize_row_q4_1(src, y, k, numerics); return 0;
+    case 6: sno_dequantize_row_q5_0(src, y, k, numerics); return 0;
+    case 7: sno_dequantize_row_q5_1(src, y, k, numerics); return 0;
     case 8: sno_dequantize_row_q8_0(src, y, k, numerics); return 0;
+    case 10: sno_dequantize_row_q2_K(src, y, k, numerics); return 0;
+    case 11: sno_dequantize_row_q3_K(src, y, k, numerics); return 0;
     case 12: sno_dequantize_row_q4_K(src, y, k, numerics); return 0;
     case 13: sno_dequantize_row_q5_K(src, y, k, numerics); return 0;
     case 14: sno_dequantize_row_q6_K(src, y, k, numerics); return 0;

@@ -23,9 +23,7 @@ namespace {
 constexpr int64_t kMaxDim = (int64_t)1 << 31;  // kernels index rows / columns with 32-bit tile counters
 
 inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
-inline bool known_type(int t) {
-    return t == SNGGUF_TYPE_Q8_0 || t == SNGGUF_TYPE_Q4_K || t == SNGGUF_TYPE_Q5_K || t == SNGGUF_TYPE_Q6_K;
-}
+inline bool known_type(int t) { return sngguf_block_size(t) != 0; }
 inline bool known_numerics(int n) { return n == SNGGUF_NUM_GGML_FP32 || n == SNGGUF_NUM_UPSTREAM_FP16; }
 
 // Shape / pointer checks shared by the matmul entry points.
@@ -59,11 +57,29 @@ const char* sngguf_strerror(int code) {
 }
 
 int64_t sngguf_type_size(int qtype) {
-    return qtype == SNGGUF_TYPE_Q8_0 ? 34 : qtype == SNGGUF_TYPE_Q4_K ? 144 : qtype == SNGGUF_TYPE_Q5_K ? 176 : qtype == SNGGUF_TYPE_Q6_K ? 210 : 0;
+    switch (qtype) {
+    case SNGGUF_TYPE_Q4_0: return 18;
+    case SNGGUF_TYPE_Q4_1: return 20;
+    case SNGGUF_TYPE_Q5_0: return 22;
+    case SNGGUF_TYPE_Q5_1: return 24;
+    case SNGGUF_TYPE_Q8_0: return 34;
+    case SNGGUF_TYPE_Q2_K: return 84;
+    case SNGGUF_TYPE_Q3_K: return 110;
+    case SNGGUF_TYPE_Q4_K: return 144;
+    case SNGGUF_TYPE_Q5_K: return 176;
+    case SNGGUF_TYPE_Q6_K: return 210;
+    default: return 0;
+    }
 }
 
 int64_t sngguf_block_size(int qtype) {
-    return qtype == SNGGUF_TYPE_Q8_0 ? 32 : (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q5_K || qtype == SNGGUF_TYPE_Q6_K) ? 256 : 0;
+    switch (qtype) {
+    case SNGGUF_TYPE_Q4_0: case SNGGUF_TYPE_Q4_1: case SNGGUF_TYPE_Q5_0: case SNGGUF_TYPE_Q5_1: case SNGGUF_TYPE_Q8_0:
+        return 32;
+    case SNGGUF_TYPE_Q2_K: case SNGGUF_TYPE_Q3_K: case SNGGUF_TYPE_Q4_K: case SNGGUF_TYPE_Q5_K: case SNGGUF_TYPE_Q6_K:
+        return 256;
+    default: return 0;
+    }
 }
 
 int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
@@ -93,7 +109,7 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (!q_up) return SNGGUF_E_NULLPTR;
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
-    if (M > 16 || K % 64 != 0) return SNGGUF_E_BADSHAPE;
+    if (M > 16) return SNGGUF_E_BADSHAPE;
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
 }
 

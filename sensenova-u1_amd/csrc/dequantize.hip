@@ -66,13 +66,9 @@ static int launch_num(const uint8_t* q, int64_t rows, int64_t cols, void* out, i
 int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
                       hipStream_t stream) {
     const uint8_t* p = static_cast<const uint8_t*>(q);
-    switch (qtype) {
-    case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(p, rows, cols, out, out_dtype, numerics, stream);
-    case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(p, rows, cols, out, out_dtype, numerics, stream);
-    case SNGGUF_TYPE_Q5_K: return launch_num<SNGGUF_TYPE_Q5_K>(p, rows, cols, out, out_dtype, numerics, stream);
-    case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(p, rows, cols, out, out_dtype, numerics, stream);
-    default: return SNGGUF_E_BADTYPE;
-    }
+#define SNGGUF_CALL(QT) launch_num<QT>(p, rows, cols, out, out_dtype, numerics, stream)
+    SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
+#undef SNGGUF_CALL
 }
 
 }  // namespace sngguf

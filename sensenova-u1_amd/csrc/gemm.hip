@@ -219,13 +219,9 @@ static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t s
     const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
     const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0) || qtype == SNGGUF_TYPE_Q4_K;
     if (tile_type && a.M >= 384 && big_tiles >= 128) return launch_gemm_tiles(a, qtype, numerics, stream);
-    switch (qtype) {
-    case SNGGUF_TYPE_Q8_0: return launch_num<SNGGUF_TYPE_Q8_0>(a, numerics, stream);
-    case SNGGUF_TYPE_Q4_K: return launch_num<SNGGUF_TYPE_Q4_K>(a, numerics, stream);
-    case SNGGUF_TYPE_Q5_K: return launch_num<SNGGUF_TYPE_Q5_K>(a, numerics, stream);
-    case SNGGUF_TYPE_Q6_K: return launch_num<SNGGUF_TYPE_Q6_K>(a, numerics, stream);
-    default: return SNGGUF_E_BADTYPE;
-    }
+#define SNGGUF_CALL(QT) launch_num<QT>(a, numerics, stream)
+    SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
+#undef SNGGUF_CALL
 }
 
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,

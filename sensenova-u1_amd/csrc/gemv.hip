@@ -1,6 +1,7 @@
 // Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the path for Q8_0 rows that are not a
-// whole number of 256-element runs (the dispatcher at the end of this file sends Q8_0 with
-// K % 256 == 0 and all Q4_K / Q5_K / Q6_K shapes to the matrix-core kernels).
+// whole number of 256-element runs and for the formats without a matrix-core kernel (the
+// dispatcher at the end of this file sends Q8_0 with K % 256 == 0 and all Q4_K / Q5_K / Q6_K
+// shapes to the matrix-core kernels).
 //
 // K % 64 == 0: one wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate
 // matrix and row n of the up matrix); a lane takes 64 weight elements (68 packed bytes) per step,
@@ -132,43 +133,73 @@ __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x,
     }
 }
 
-// Q8_0 rows whose block count is odd are not a whole number of 64-element units (and their
-// rows are only 2-byte aligned): they take this plain path, one wavefront per row, eight
-// elements per lane and step through the shared 8-element decoder.
-template <int QT, int NUM>
-__global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q,
-                                                           int64_t N, int64_t K, const bf16_t* __restrict__ bias,
-                                                           bf16_t* __restrict__ y) {
+// Every other case - Q8_0 rows whose block count is odd (not a whole number of 64-element units,
+// rows only 2-byte aligned) and the formats without a kernel of their own (Q4_0, Q4_1, Q5_0,
+// Q5_1, Q2_K, Q3_K) - takes this plain path: one wavefront per row (GATED: row n of the gate and
+// of the up matrix), eight elements per lane and step through the shared 8-element decoder.
+template <int QT, int NUM, bool GATED>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
+                                                           const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                           const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+    constexpr int NW = GATED ? 2 : 1;
     const int lane = threadIdx.x & 63;
     const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N) return;
     const int64_t row_bytes = K / Fmt<QT>::bs * Fmt<QT>::ts;
-    const uint8_t* row = q + n * row_bytes;
-    float acc[16];
+    const uint8_t* rows[2] = {qa + n * row_bytes, GATED ? qb + n * row_bytes : nullptr};
+    float acc[NW][16];
 #pragma unroll
-    for (int m = 0; m < 16; m++) acc[m] = 0.f;
+    for (int t = 0; t < NW; t++)
+#pragma unroll
+        for (int m = 0; m < 16; m++) acc[t][m] = 0.f;
     for (int64_t e0 = (int64_t)lane * 8; e0 < K; e0 += 64 * 8) {
-        float w[8];
-        decode8<QT, NUM>(row, e0, w);
+        float w[NW][8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) w[i] = bf16_to_f32(f32_to_bf16(w[i]));
+        for (int t = 0; t < NW; t++) {
+            decode8<QT, NUM>(rows[t], e0, w[t]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) w[t][i] = bf16_to_f32(f32_to_bf16(w[t][i]));
+        }
         for (int m = 0; m < M; m++) {
-            const bf16_t* xr = x + (int64_t)m * K + e0;
-            float s = 0.f;
+            const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + e0);
+            float s[NW];
 #pragma unroll
-            for (int i = 0; i < 8; i++) s = fmaf(w[i], bf16_to_f32(xr[i]), s);
+            for (int t = 0; t < NW; t++) {
+                s[t] = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    s[t] = fmaf(w[t][2 * i], bf16lo_to_f32(xv[i]), s[t]);
+                    s[t] = fmaf(w[t][2 * i + 1], bf16hi_to_f32(xv[i]), s[t]);
+                }
+            }
 #pragma unroll
             for (int mm = 0; mm < 16; mm++)
-                if (mm == m) acc[mm] += s;
+                if (mm == m) {
+#pragma unroll
+                    for (int t = 0; t < NW; t++) acc[t][mm] += s[t];
+                }
         }
     }
     for (int m = 0; m < M; m++) {
-        float v = 0.f;
+        float v[NW];
 #pragma unroll
-        for (int mm = 0; mm < 16; mm++)
-            if (mm == m) v = acc[mm];
-        v = wave_sum(v);
-        if (lane == 0) y[(int64_t)m * N + n] = f32_to_bf16(v + (bias ? bf16_to_f32(bias[n]) : 0.f));
+        for (int t = 0; t < NW; t++) {
+            v[t] = 0.f;
+#pragma unroll
+            for (int mm = 0; mm < 16; mm++)
+                if (mm == m) v[t] = acc[t][mm];
+            v[t] = wave_sum(v[t]);
+        }
+        if (lane == 0) {
+            if constexpr (GATED) {
+                const float g = bf16_to_f32(f32_to_bf16(v[0]));
+                const float up = bf16_to_f32(f32_to_bf16(v[1]));
+                const float sg = bf16_to_f32(f32_to_bf16(g / (1.0f + expf(-g))));
+                y[(int64_t)m * N + n] = f32_to_bf16(sg * up);
+            } else {
+                y[(int64_t)m * N + n] = f32_to_bf16(v[0] + (bias ? bf16_to_f32(bias[n]) : 0.f));
+            }
+        }
     }
 }
 
@@ -193,14 +224,17 @@ static int launch_mt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 template <int QT, int NUM>
 static int launch_gated(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
                         const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
-    if (K % 64 != 0) {  // only Q8_0 with an odd block count
-        if (gated) return SNGGUF_E_BADSHAPE;
+    if (QT != SNGGUF_TYPE_Q8_0 || K % 64 != 0) {
         dim3 grid((unsigned)((N + 3) / 4)), block(256);
-        gemv_generic_kernel<QT, NUM><<<grid, block, 0, stream>>>(x, M, qa, N, K, bias, y);
+        if (gated) gemv_generic_kernel<QT, NUM, true><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y);
+        else gemv_generic_kernel<QT, NUM, false><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y);
         return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
     }
-    if (gated) return launch_mt<QT, NUM, true>(x, M, qa, qb, N, K, bias, y, stream);
-    return launch_mt<QT, NUM, false>(x, M, qa, qb, N, K, bias, y, stream);
+    if constexpr (QT == SNGGUF_TYPE_Q8_0) {
+        if (gated) return launch_mt<QT, NUM, true>(x, M, qa, qb, N, K, bias, y, stream);
+        return launch_mt<QT, NUM, false>(x, M, qa, qb, N, K, bias, y, stream);
+    }
+    return SNGGUF_E_BADTYPE;
 }
 
 template <int QT>
@@ -229,9 +263,11 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
     if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q5_K || qtype == SNGGUF_TYPE_Q6_K)
         return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
-    // Q8_0 rows that are not a whole number of 256-element runs
-    if (qtype == SNGGUF_TYPE_Q8_0) return launch_num<SNGGUF_TYPE_Q8_0>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream);
-    return SNGGUF_E_BADTYPE;
+    // Q8_0 rows that are not a whole number of 256-element runs, and the formats served by the
+    // generic kernel
+#define SNGGUF_CALL(QT) launch_num<QT>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream)
+    SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
+#undef SNGGUF_CALL
 }
 
 }  // namespace sngguf

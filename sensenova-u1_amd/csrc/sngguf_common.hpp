@@ -1,5 +1,5 @@
 // Shared device helpers of the gfx950 GGUF quantized-linear kernels: scalar format
-// conversions, the three block decoders and wavefront reductions.  Included by every .hip
+// conversions, the block decoders and wavefront reductions.  Included by every .hip
 // file of the library; nothing here touches the host runtime.
 #pragma once
 
@@ -23,7 +23,12 @@ constexpr int kWave = 64;
 // ---- scalar formats ---------------------------------------------------------------------
 
 __device__ __forceinline__ float f16_to_f32(uint16_t bits) { return (float)__builtin_bit_cast(_Float16, bits); }
-__device__ __forceinline__ uint16_t f32_to_f16(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+// The empty asm keeps the compiler from folding a preceding fp32 multiply into the conversion as
+// a mixed-precision fma with a +0 addend, which turns a product of -0 into +0.
+__device__ __forceinline__ uint16_t f32_to_f16(float v) {
+    asm volatile("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
 // One fp16 tensor-op rounding (v_cvt_f16_f32 is round-to-nearest-even with subnormals), widened again.
 __device__ __forceinline__ float round_f16(float v) { return (float)(_Float16)v; }
 __device__ __forceinline__ bf16_t f32_to_bf16(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
@@ -89,7 +94,13 @@ __device__ __forceinline__ uint32_t ld_u32(const uint8_t* p) { return *reinterpr
 // ---- format constants -----------------------------------------------------------------------
 
 template <int QT> struct Fmt;
+template <> struct Fmt<SNGGUF_TYPE_Q4_0> { static constexpr int bs = 32, ts = 18; };
+template <> struct Fmt<SNGGUF_TYPE_Q4_1> { static constexpr int bs = 32, ts = 20; };
+template <> struct Fmt<SNGGUF_TYPE_Q5_0> { static constexpr int bs = 32, ts = 22; };
+template <> struct Fmt<SNGGUF_TYPE_Q5_1> { static constexpr int bs = 32, ts = 24; };
 template <> struct Fmt<SNGGUF_TYPE_Q8_0> { static constexpr int bs = 32, ts = 34; };
+template <> struct Fmt<SNGGUF_TYPE_Q2_K> { static constexpr int bs = 256, ts = 84; };
+template <> struct Fmt<SNGGUF_TYPE_Q3_K> { static constexpr int bs = 256, ts = 110; };
 template <> struct Fmt<SNGGUF_TYPE_Q4_K> { static constexpr int bs = 256, ts = 144; };
 template <> struct Fmt<SNGGUF_TYPE_Q5_K> { static constexpr int bs = 256, ts = 176; };
 template <> struct Fmt<SNGGUF_TYPE_Q6_K> { static constexpr int bs = 256, ts = 210; };
@@ -107,6 +118,23 @@ __device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t
         mn = (b >> 4) | (((s1 >> (8 * i + 6)) & 3u) << 4);
     }
 }
+
+// Runs CALL(<type constant>) for the run-time quant type (CALL is a macro or a generic lambda-like
+// macro that returns); unknown types return SNGGUF_E_BADTYPE.
+#define SNGGUF_DISPATCH_TYPE(qtype, CALL)                       \
+    switch (qtype) {                                            \
+    case SNGGUF_TYPE_Q4_0: return CALL(SNGGUF_TYPE_Q4_0);       \
+    case SNGGUF_TYPE_Q4_1: return CALL(SNGGUF_TYPE_Q4_1);       \
+    case SNGGUF_TYPE_Q5_0: return CALL(SNGGUF_TYPE_Q5_0);       \
+    case SNGGUF_TYPE_Q5_1: return CALL(SNGGUF_TYPE_Q5_1);       \
+    case SNGGUF_TYPE_Q8_0: return CALL(SNGGUF_TYPE_Q8_0);       \
+    case SNGGUF_TYPE_Q2_K: return CALL(SNGGUF_TYPE_Q2_K);       \
+    case SNGGUF_TYPE_Q3_K: return CALL(SNGGUF_TYPE_Q3_K);       \
+    case SNGGUF_TYPE_Q4_K: return CALL(SNGGUF_TYPE_Q4_K);       \
+    case SNGGUF_TYPE_Q5_K: return CALL(SNGGUF_TYPE_Q5_K);       \
+    case SNGGUF_TYPE_Q6_K: return CALL(SNGGUF_TYPE_Q6_K);       \
+    default: return SNGGUF_E_BADTYPE;                           \
+    }
 
 // ---- 8-element decoders (standalone dequantize, GEMM tile fill) -------------------------------
 // decode8<QT,NUM>(row, e0, w): eight consecutive elements e0..e0+7 (e0 % 8 == 0) of a packed
@@ -126,6 +154,84 @@ __device__ __forceinline__ void decode8_q8_0(const uint8_t* __restrict__ row, in
         const uint32_t h = ld_u16(qs + 2 * i);
         w[2 * i] = A::widen(d * A::integer((int8_t)(h & 0xFF)));
         w[2 * i + 1] = A::widen(d * A::integer((int8_t)(h >> 8)));
+    }
+}
+
+// The four legacy formats: 32-element blocks, element l in the low nibble of qs[l], element
+// l + 16 in the high nibble; Q5_x add bit e of a 32-bit word as fifth bit of element e; the _0
+// formats subtract half the range, the _1 formats add a block minimum m.
+// HDR = bytes before qh/qs (2: d; 4: d, m); FIVE = has the fifth-bit word.
+template <int NUM, int TS, bool HAS_MIN, bool FIVE>
+__device__ __forceinline__ void decode8_legacy(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
+    const uint8_t* blk = row + (e0 >> 5) * TS;  // only 2-byte aligned in general
+    const int r = (int)(e0 & 31);
+    const int hi = r >> 4;
+    const int l0 = r & 15;
+    constexpr int kHdr = HAS_MIN ? 4 : 2;
+    const typename A::T d = A::scale(ld_u16(blk));
+    const uint32_t hbits = FIVE ? (ld_u32_a2(blk + kHdr) >> r) : 0u;
+    const uint8_t* qs = blk + kHdr + (FIVE ? 4 : 0) + l0;
+    const uint32_t q0 = ld_u32_a2(qs), q1 = ld_u32_a2(qs + 4);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t byte = ((i < 4 ? q0 : q1) >> (8 * (i & 3))) & 0xFFu;
+        int q = (int)(hi ? (byte >> 4) : (byte & 0x0Fu));
+        if constexpr (FIVE) q |= (int)(((hbits >> i) & 1u) << 4);
+        if constexpr (HAS_MIN) {
+            // fp32: d*q exact, one rounding in the sum; fp16: R(R(d*q) + m)
+            w[i] = A::widen(d * A::integer(q) + A::scale(ld_u16(blk + 2)));
+        } else {
+            w[i] = A::widen(d * A::integer(q - (FIVE ? 16 : 8)));
+        }
+    }
+}
+
+// Q2_K: { u8 scales[16]; u8 qs[64]; f16 d; f16 dmin }.  Per 128-element half, bit pair j of
+// qs[32 * half + l] is element 32 * j + l; group g = e / 16 has scale scales[g] & 15 and min
+// scales[g] >> 4.
+template <int NUM>
+__device__ __forceinline__ void decode8_q2_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
+    const uint8_t* blk = row + (e0 >> 8) * 84;
+    const int r = (int)(e0 & 255);
+    const int half = r >> 7, j = (r >> 5) & 3, l0 = r & 31;
+    const uint32_t sm = blk[r >> 4];
+    const uint32_t dd = ld_u32_a2(blk + 80);
+    const typename A::T DL = A::scale((uint16_t)(dd & 0xFFFF)) * A::integer((int)(sm & 15u));
+    const typename A::T ML = A::scale((uint16_t)(dd >> 16)) * A::integer((int)(sm >> 4));
+    const uint8_t* qs = blk + 16 + 32 * half + l0;
+    const uint32_t q0 = ld_u32_a2(qs) >> (2 * j), q1 = ld_u32_a2(qs + 4) >> (2 * j);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = (int)(((i < 4 ? q0 : q1) >> (8 * (i & 3))) & 3u);
+        w[i] = A::widen(DL * A::integer(q) - ML);
+    }
+}
+
+// Q3_K: { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d }.  Quant = bit pair as in Q2_K, minus 4
+// unless bit (4 * half + j) of hmask[l] is set; the 6-bit scale of group g has its low nibble in
+// scales[g % 8] (upper nibble for g >= 8), its high two bits in scales[8 + g % 4] at bit
+// 2 * (g / 4), and is offset by -32.
+template <int NUM>
+__device__ __forceinline__ void decode8_q3_k(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
+    typedef Num<NUM> A;
+    const uint8_t* blk = row + (e0 >> 8) * 110;  // 2-byte aligned
+    const int r = (int)(e0 & 255);
+    const int half = r >> 7, j = (r >> 5) & 3, l0 = r & 31;
+    const int g = r >> 4;
+    const uint32_t lo = g < 8 ? (blk[96 + g] & 15u) : ((uint32_t)blk[96 + g - 8] >> 4);
+    const uint32_t hi = ((uint32_t)blk[104 + (g & 3)] >> (2 * (g >> 2))) & 3u;
+    const typename A::T DL = A::scale(ld_u16(blk + 108)) * A::integer((int)(lo | (hi << 4)) - 32);
+    const uint8_t* qs = blk + 32 + 32 * half + l0;
+    const uint32_t q0 = ld_u32_a2(qs) >> (2 * j), q1 = ld_u32_a2(qs + 4) >> (2 * j);
+    const int hb = 4 * half + j;
+    const uint32_t h0 = ld_u32_a2(blk + l0) >> hb, h1 = ld_u32_a2(blk + l0 + 4) >> hb;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int sh = 8 * (i & 3);
+        const int q = (int)(((i < 4 ? q0 : q1) >> sh) & 3u) - ((((i < 4 ? h0 : h1) >> sh) & 1u) ? 0 : 4);
+        w[i] = A::widen(DL * A::integer(q));
     }
 }
 
@@ -208,9 +314,18 @@ __device__ __forceinline__ void decode8_q6_k(const uint8_t* __restrict__ row, in
 template <int QT, int NUM>
 __device__ __forceinline__ void decode8(const uint8_t* __restrict__ row, int64_t e0, float (&w)[8]) {
     if constexpr (QT == SNGGUF_TYPE_Q8_0) decode8_q8_0<NUM>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_0) decode8_legacy<NUM, 18, false, false>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_1) decode8_legacy<NUM, 20, true, false>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_0) decode8_legacy<NUM, 22, false, true>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_1) decode8_legacy<NUM, 24, true, true>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q2_K) decode8_q2_k<NUM>(row, e0, w);
+    else if constexpr (QT == SNGGUF_TYPE_Q3_K) decode8_q3_k<NUM>(row, e0, w);
     else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode8_q4_k<NUM>(row, e0, w);
     else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode8_q5_k<NUM>(row, e0, w);
-    else decode8_q6_k<NUM>(row, e0, w);
+    else {
+        static_assert(QT == SNGGUF_TYPE_Q6_K, "no decoder for this quant type");
+        decode8_q6_k<NUM>(row, e0, w);
+    }
 }
 
 // ---- Q8_0: one dword of quants -> four bf16 (shared by the GEMV and GEMM kernels) ---------------

@@ -22,7 +22,13 @@ from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType
 
 # quant types the HIP kernels decode
 SUPPORTED_GGUF_QUANT_TYPES = (
+    GGMLQuantizationType.Q4_0,
+    GGMLQuantizationType.Q4_1,
+    GGMLQuantizationType.Q5_0,
+    GGMLQuantizationType.Q5_1,
     GGMLQuantizationType.Q8_0,
+    GGMLQuantizationType.Q2_K,
+    GGMLQuantizationType.Q3_K,
     GGMLQuantizationType.Q4_K,
     GGMLQuantizationType.Q5_K,
     GGMLQuantizationType.Q6_K,

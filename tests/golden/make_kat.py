@@ -8,6 +8,12 @@ comments, so the file pins the oracle against the format definition itself.
     block_q4_K { f16 d; f16 dmin; u8 scales[12]; u8 qs[128]; }          144 bytes
     block_q5_K { f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]; } 176 bytes
     block_q6_K { u8 ql[128]; u8 qh[64]; int8 scales[16]; f16 d; }       210 bytes
+    block_q4_0 { f16 d; u8 qs[16]; }                                     18 bytes
+    block_q4_1 { f16 d; f16 m; u8 qs[16]; }                              20 bytes
+    block_q5_0 { f16 d; u8 qh[4]; u8 qs[16]; }                           22 bytes
+    block_q5_1 { f16 d; f16 m; u8 qh[4]; u8 qs[16]; }                    24 bytes
+    block_q2_K { u8 scales[16]; u8 qs[64]; f16 d; f16 dmin; }            84 bytes
+    block_q3_K { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d; }       110 bytes
 
 Run from this directory: ``python make_kat.py``.
 """
@@ -114,6 +120,65 @@ sc[9] = "fd"
 hexs = "".join(ql) + "".join(qh) + "".join(sc) + "0040"
 kats.append({"name": "q6_k quadrants, high bits, signed scale", "type": 14, "hex": hexs, "fill": 0.0,
              "expect": {"146": -186.0, "5": -64.0, "101": 32.0}, "how": "see make_kat.py"})
+
+# --- Q4_0: d = 2.0 ("0040"); value = d * (nibble - 8); byte l carries element l (low) and l + 16 (high).
+# Background nibble 8 (-> 0): bytes 0x88.  qs[3] = 0x1F: element 3 = 15 - 8 = 7 -> 14, element 19 = 1 - 8 = -7 -> -14.
+hexs = "0040" + "88" * 3 + "1f" + "88" * 12
+kats.append({"name": "q4_0 nibble order and offset", "type": 2, "hex": hexs, "fill": 0.0,
+             "expect": {"3": 14.0, "19": -14.0}, "how": "see make_kat.py"})
+
+# --- Q4_1: d = 0.5 ("0038"), m = -1.0 (f16 0xBC00, "00bc"); value = d * nibble + m.
+# Background nibble 0 -> -1.  qs[15] = 0x92: element 15 = 2 -> 0.0, element 31 = 9 -> 3.5.
+hexs = "0038" + "00bc" + "00" * 15 + "92"
+kats.append({"name": "q4_1 minimum is added", "type": 3, "hex": hexs, "fill": -1.0,
+             "expect": {"15": 0.0, "31": 3.5}, "how": "see make_kat.py"})
+
+# --- Q5_0: d = 1.0; value = d * ((nibble | fifth << 4) - 16), fifth bit of element e = bit e of the
+# little-endian 32-bit qh.  Background stored 16 (-> 0): nibbles 0, qh all ones.
+#   element 9: bit 9 (byte 1, bit 1) cleared -> qh bytes ff fd ff ff; low nibble of qs[9] = 3 -> 3 - 16 = -13
+#   element 30: bit 30 stays set; high nibble of qs[14] = 0xA -> (10 | 16) - 16 = 10
+qs = ["00"] * 16
+qs[9] = "03"
+qs[14] = "a0"
+hexs = "003c" + "fffdffff" + "".join(qs)
+kats.append({"name": "q5_0 fifth-bit word, bit order", "type": 6, "hex": hexs, "fill": 0.0,
+             "expect": {"9": -13.0, "30": 10.0}, "how": "see make_kat.py"})
+
+# --- Q5_1: d = 0.25 (f16 0x3400, "0034"), m = 1.0; value = d * (nibble | fifth << 4) + m.
+# Only bit 17 of qh set (byte 2 = 0x02); qs[1] = 0x70: element 1 = 0 -> 1.0, element 17 = 7 + 16 = 23 -> 6.75.
+hexs = "0034" + "003c" + "00000200" + "00" + "70" + "00" * 14
+kats.append({"name": "q5_1 fifth bit of a high-nibble element", "type": 7, "hex": hexs, "fill": 1.0,
+             "expect": {"17": 6.75}, "how": "see make_kat.py"})
+
+# --- Q2_K: d = 1.0, dmin = 0.5; scales[g] = scale | min << 4 for the 16-element group g; per 128-element half,
+# bit pair j of qs[32 * half + l] is element 128 * half + 32 * j + l; value = d * scale * q - dmin * min.
+# All scales 0x01 (scale 1, min 0) except scales[10] = 0x23 (scale 3, min 2): elements 160..175.
+# qs[32 + 5] = 0b01_00_11_10 = 0x4E (half 1, l = 5): element 133 = 2 -> 2; element 165 = 3 -> 3 * 3 - 1 = 8;
+# element 197 = 0; element 229 = 1 -> 1.  The rest of group 10 is 0 * 3 - 0.5 * 2 = -1.
+hexs = "01" * 10 + "23" + "01" * 5 + "00" * 37 + "4e" + "00" * 26 + "003c" + "0038"
+exp = {str(e): -1.0 for e in range(160, 176)}
+exp.update({"133": 2.0, "165": 8.0, "229": 1.0})
+kats.append({"name": "q2_k bit pairs, group scale and min", "type": 10, "hex": hexs, "fill": 0.0, "expect": exp,
+             "how": "see make_kat.py"})
+
+# --- Q3_K: d = 1.0; quant = bit pair (as Q2_K) minus 4 unless bit (4 * half + j) of hmask[l] is set;
+# value = d * (scale6 - 32) * quant.  Background: quant stored 4 (mask bit set, low bits 0) -> 0.
+# Scales: all 1 -> stored 33 = 0b10_0001: low nibble 1 (scales[0..7] = 0x11: low nibble for groups 0..7, high
+# nibble for groups 8..15), high bits 2 (scales[8..11] = 0b10101010 = 0xAA: byte k holds groups k, k+4, k+8,
+# k+12 at bits 0-1, 2-3, 4-5, 6-7).  Group 13 = -3 -> stored 29 = 0b01_1101: low nibble 0xD in the high nibble
+# of scales[5] (0xD1), high bits 1 at bits 6-7 of scales[9] (0b01101010 = 0x6A).
+#   element 210 (half 1, j = 2, l = 18, group 13): quant -4 -> stored 0: clear bit 6 of hmask[18] (0xBF) -> -3 * -4 = 12
+#   element 211 (l = 19): quant 3 -> stored 7: mask bit set, qs[32 + 19] bits 4-5 = 3 (0x30) -> -3 * 3 = -9
+#   element 7 (half 0, j = 0, group 0): quant -2 -> stored 2: clear bit 0 of hmask[7] (0xFE), qs[7] = 0x02 -> -2
+hm = ["ff"] * 32
+hm[7] = "fe"
+hm[18] = "bf"
+qs = ["00"] * 64
+qs[7] = "02"
+qs[51] = "30"
+hexs = "".join(hm) + "".join(qs) + "11" * 5 + "d1" + "11" * 2 + "aa" + "6a" + "aa" + "aa" + "003c"
+kats.append({"name": "q3_k mask bit, split scales", "type": 11, "hex": hexs, "fill": 0.0,
+             "expect": {"210": 12.0, "211": -9.0, "7": -2.0}, "how": "see make_kat.py"})
 
 with open("kat_blocks.json", "w") as f:
     json.dump(kats, f, indent=1)

@@ -31,7 +31,10 @@ def test_host_only_entry_points():
     assert (lib.sngguf_block_size(12), lib.sngguf_type_size(12)) == (256, 144)
     assert (lib.sngguf_block_size(14), lib.sngguf_type_size(14)) == (256, 210)
     assert (lib.sngguf_block_size(13), lib.sngguf_type_size(13)) == (256, 176)
-    assert lib.sngguf_block_size(11) == 0 and lib.sngguf_type_size(2) == 0
+    assert (lib.sngguf_block_size(11), lib.sngguf_type_size(11)) == (256, 110)
+    assert [lib.sngguf_type_size(t) for t in (2, 3, 6, 7, 10)] == [18, 20, 22, 24, 84]
+    assert [lib.sngguf_block_size(t) for t in (2, 3, 6, 7, 10)] == [32, 32, 32, 32, 256]
+    assert lib.sngguf_block_size(9) == 0 and lib.sngguf_type_size(16) == 0 and lib.sngguf_type_size(0) == 0
     assert lib.sngguf_grouped_workspace_bytes(1000) >= 4 * 1000 + 4
     assert lib.sngguf_strerror(0) == b"ok"
     for code in range(-6, 0):
@@ -45,7 +48,7 @@ def test_argument_validation_needs_no_device():
     p = ctypes.c_void_p((ctypes.addressof(buf) + 63) // 64 * 64)
     odd = ctypes.c_void_p(p.value + 2)
     E_TYPE, E_SHAPE, E_NULL, E_ALIGN = -1, -2, -3, -4
-    assert lib.sngguf_dequantize(p, 11, 1, 256, p, 0, 0, None) == E_TYPE        # Q3_K not implemented
+    assert lib.sngguf_dequantize(p, 16, 1, 256, p, 0, 0, None) == E_TYPE        # IQ2_XXS not implemented
     assert lib.sngguf_dequantize(p, 8, 1, 32, p, 7, 0, None) == E_TYPE          # bad out dtype
     assert lib.sngguf_dequantize(p, 8, 1, 32, p, 0, 5, None) == E_TYPE          # bad numerics
     assert lib.sngguf_dequantize(p, 8, 1, 33, p, 0, 0, None) == E_SHAPE         # cols % 32
@@ -60,6 +63,7 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_linear(p, 1, p, 8, 4, 64, None, odd, 1, None) == E_ALIGN
     assert lib.sngguf_linear(p, 0, p, 8, 4, 64, None, p, 1, None) == 0
     assert lib.sngguf_gate_up_silu(p, 17, p, p, 8, 4, 64, p, 1, None) == E_SHAPE  # decode only
+    assert lib.sngguf_linear(p, 1, p, 2, 4, 48, None, p, 1, None) == E_SHAPE    # Q4_0: K % 32
     assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL
     assert lib.sngguf_grouped_linear(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_NULL  # no workspace
     assert lib.sngguf_grouped_linear(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_SHAPE  # n_text > M

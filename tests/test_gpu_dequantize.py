@@ -7,7 +7,7 @@ from sensenova_u1_amd import ops, synthetic
 
 pytestmark = pytest.mark.gpu
 
-TYPES = [go.Q8_0, go.Q4_K, go.Q5_K, go.Q6_K]
+TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q8_0, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K]
 
 
 def _bits(t):
@@ -53,7 +53,8 @@ def test_dequantize_random_bytes_extremes(dev, c_oracle, qt):
     g = torch.Generator().manual_seed(99 + qt)
     packed = torch.randint(0, 256, (64, 1024 // bs * ts), dtype=torch.uint8, generator=g)
     blocks = packed.view(-1, ts)
-    for off in {go.Q8_0: [0], go.Q4_K: [0, 2], go.Q5_K: [0, 2], go.Q6_K: [208]}[qt]:
+    for off in {go.Q4_0: [0], go.Q4_1: [0, 2], go.Q5_0: [0], go.Q5_1: [0, 2], go.Q8_0: [0], go.Q2_K: [80, 82], go.Q3_K: [108],
+                go.Q4_K: [0, 2], go.Q5_K: [0, 2], go.Q6_K: [208]}[qt]:
         h = blocks[:, off:off + 2].contiguous().view(torch.int16)
         bad = (h & 0x7C00) == 0x7C00
         h[bad] = h[bad] & ~0x4000  # clear one exponent bit: finite, keeps sign and mantissa

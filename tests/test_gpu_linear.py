@@ -9,7 +9,7 @@ from sensenova_u1_amd import ops, synthetic
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-3          # rel-L2 bound on bf16 outputs
-TYPES = [go.Q8_0, go.Q4_K, go.Q5_K, go.Q6_K]
+TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q8_0, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K]
 
 
 def _check(got, want, tol=TOL):
@@ -233,7 +233,8 @@ def test_gate_up_silu(dev, c_oracle, qt, m):
     _check(got, c_oracle.silu_mul(g, u))
 
 
-@pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q4_K), (go.Q6_K, go.Q6_K), (go.Q4_K, go.Q6_K), (go.Q5_K, go.Q8_0)])
+@pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q4_K), (go.Q6_K, go.Q6_K), (go.Q4_K, go.Q6_K), (go.Q5_K, go.Q8_0),
+                                     (go.Q4_0, go.Q3_K), (go.Q5_1, go.Q2_K)])
 def test_grouped_linear_indicator(dev, qt_pair):
     print(f"case grouped indicator {qt_pair}", flush=True)
     qu, qg = qt_pair

@@ -89,14 +89,15 @@ def test_load_gguf_checkpoint_types_and_names(tmp_path):
 
 def test_unsupported_quant_type_raises_value_error(tmp_path):
     path = str(tmp_path / "u.gguf")
-    _make_file(path, extra=[("odd.weight", np.zeros((2, 110), dtype=np.uint8), int(GGMLQuantizationType.Q3_K))])
+    _make_file(path, extra=[("odd.weight", np.zeros((2, 36), dtype=np.uint8), int(GGMLQuantizationType.Q8_1))])
     with pytest.raises(ValueError, match="odd.weight has unsupported quant type") as exc:
         load_gguf_checkpoint(path)
     assert "Supported" in str(exc.value) and "Q8_0" in str(exc.value)
 
 
 @pytest.mark.parametrize("quant", [GGMLQuantizationType.Q8_0, GGMLQuantizationType.Q4_K, GGMLQuantizationType.Q5_K,
-                                   GGMLQuantizationType.Q6_K])
+                                   GGMLQuantizationType.Q6_K, GGMLQuantizationType.Q4_0, GGMLQuantizationType.Q5_1,
+                                   GGMLQuantizationType.Q3_K])
 def test_set_gguf2meta_model_replaces_and_places(tmp_path, quant):
     path = str(tmp_path / "m.gguf")
     ref, packed = _make_file(path, quant)

@@ -17,7 +17,7 @@ import torch
 from oracle import gguf_oracle as go
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = [go.Q8_0, go.Q4_K, go.Q5_K, go.Q6_K]
+TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q8_0, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K]
 
 
 def _blocks(raw: bytes) -> torch.Tensor:
@@ -203,6 +203,99 @@ def test_q6_k_random_round_trip_closed_form(c_oracle):
         assert np.array_equal(out.astype(np.float64), exact)
 
 
+# ---- Q4_0 / Q4_1 / Q5_0 / Q5_1 ------------------------------------------------------------------
+
+def test_legacy_blocks_one_hot_positions(c_oracle):
+    """One non-zero quant per block: pins the low-nibble / high-nibble element order (l, l + 16) and
+    the bit order of the 32-bit fifth-bit word."""
+    for pos in range(32):
+        q = [0] * 32
+        q[pos] = 5
+        out = _both(c_oracle, _blocks(go.pack_q4_0(0.5, q)), go.Q4_0)
+        want = torch.zeros(32)
+        want[pos] = 2.5
+        assert torch.equal(out, want), pos
+        out = _both(c_oracle, _blocks(go.pack_q4_1(0.5, 0.0, q)), go.Q4_1)
+        assert torch.equal(out, want), pos
+        for v in (-16, -11, 11):        # fifth bit alone (stored 0), nibble only (stored 5), nibble + fifth bit (stored 27)
+            q[pos] = v
+            out = _both(c_oracle, _blocks(go.pack_q5_0(0.5, q)), go.Q5_0)
+            want[pos] = 0.5 * v
+            assert torch.equal(out, want), (pos, v)
+        q = [0] * 32
+        for v in (16, 21, 5):
+            q[pos] = v
+            out = _both(c_oracle, _blocks(go.pack_q5_1(0.5, 0.0, q)), go.Q5_1)
+            want[pos] = 0.5 * v
+            assert torch.equal(out, want), (pos, v)
+
+
+def test_legacy_blocks_closed_form(c_oracle):
+    """Offsets (-8 / -16 against + m) and the sign of the minimum: exact fp64 closed form, one rounding."""
+    rng = np.random.default_rng(7)
+    for _ in range(50):
+        d = np.float16(abs(rng.standard_normal()) * 0.01)
+        m = np.float16(rng.standard_normal() * 0.01)
+        q4, q5 = rng.integers(0, 16, 32), rng.integers(0, 32, 32)
+        out = _both(c_oracle, _blocks(go.pack_q4_0(d, q4 - 8)), go.Q4_0).numpy()
+        assert np.array_equal(out.astype(np.float64), np.float64(d) * (q4 - 8))
+        out = _both(c_oracle, _blocks(go.pack_q5_0(d, q5 - 16)), go.Q5_0).numpy()
+        assert np.array_equal(out.astype(np.float64), np.float64(d) * (q5 - 16))
+        out = _both(c_oracle, _blocks(go.pack_q4_1(d, m, q4)), go.Q4_1).numpy()
+        assert np.array_equal(out, (np.float64(d) * q4 + np.float64(m)).astype(np.float32))
+        out = _both(c_oracle, _blocks(go.pack_q5_1(d, m, q5)), go.Q5_1).numpy()
+        assert np.array_equal(out, (np.float64(d) * q5 + np.float64(m)).astype(np.float32))
+
+
+# ---- Q2_K / Q3_K ------------------------------------------------------------------------------
+
+def test_q2_k_one_hot_and_closed_form(c_oracle):
+    sc, mn = [1] * 16, [0] * 16
+    for pos in list(range(0, 256, 7)) + [15, 16, 31, 32, 127, 128, 255]:
+        q = [0] * 256
+        q[pos] = 3
+        out = _both(c_oracle, _blocks(go.pack_q2_k(1.0, 0.0, sc, mn, q)), go.Q2_K)
+        want = torch.zeros(256)
+        want[pos] = 3.0
+        assert torch.equal(out, want), pos
+    sc = [1, 15, 2, 14, 3, 13, 4, 12, 5, 11, 6, 10, 7, 9, 8, 0]
+    mn = [15, 0, 14, 1, 13, 2, 12, 3, 11, 4, 10, 5, 9, 6, 8, 7]
+    q = [(5 * i + 1) % 4 for i in range(256)]
+    out = _both(c_oracle, _blocks(go.pack_q2_k(2.0, 0.5, sc, mn, q)), go.Q2_K).numpy()
+    want = np.array([2.0 * sc[i // 16] * q[i] - 0.5 * mn[i // 16] for i in range(256)], dtype=np.float32)
+    assert np.array_equal(out, want)
+    rng = np.random.default_rng(8)
+    for _ in range(50):
+        sc, mn, q = rng.integers(0, 16, 16), rng.integers(0, 16, 16), rng.integers(0, 4, 256)
+        d, dmin = np.float16(abs(rng.standard_normal()) * 0.01), np.float16(abs(rng.standard_normal()) * 0.01)
+        out = _both(c_oracle, _blocks(go.pack_q2_k(d, dmin, sc, mn, q)), go.Q2_K).numpy()
+        exact = np.float64(d) * sc.repeat(16) * q - np.float64(dmin) * mn.repeat(16)
+        assert np.array_equal(out, exact.astype(np.float32))
+
+
+def test_q3_k_one_hot_and_closed_form(c_oracle):
+    sc = [1] * 16
+    for pos in list(range(0, 256, 7)) + [15, 16, 31, 32, 127, 128, 255]:
+        for v in (3, -4, -1, 1):     # stored 7 (mask bit + both low bits), 0 (nothing set), 3, 5
+            q = [0] * 256            # 0 is stored as 4: mask bit set, low bits clear
+            q[pos] = v
+            out = _both(c_oracle, _blocks(go.pack_q3_k(1.0, sc, q)), go.Q3_K)
+            want = torch.zeros(256)
+            want[pos] = float(v)
+            assert torch.equal(out, want), (pos, v)
+    sc = [-32, 31, 1, -1, 15, -16, 16, -17, 7, -8, 21, -22, 3, -29, 30, -5]    # every low / high bit pattern
+    q = [(5 * i + 2) % 8 - 4 for i in range(256)]
+    out = _both(c_oracle, _blocks(go.pack_q3_k(0.25, sc, q)), go.Q3_K).numpy()
+    want = np.array([0.25 * sc[i // 16] * q[i] for i in range(256)], dtype=np.float32)
+    assert np.array_equal(out, want)
+    rng = np.random.default_rng(9)
+    for _ in range(50):
+        sc, q = rng.integers(-32, 32, 16), rng.integers(-4, 4, 256)
+        d = np.float16(abs(rng.standard_normal()) * 0.01)
+        out = _both(c_oracle, _blocks(go.pack_q3_k(d, sc, q)), go.Q3_K).numpy()
+        assert np.array_equal(out.astype(np.float64), np.float64(d) * sc.repeat(16) * q)
+
+
 # ---- hand-written known-answer blocks ---------------------------------------------------------
 
 def test_known_answer_blocks(c_oracle):
@@ -210,7 +303,7 @@ def test_known_answer_blocks(c_oracle):
     (hex bytes) with expected values worked out on paper; see the file's "how" fields."""
     with open(os.path.join(HERE, "golden", "kat_blocks.json")) as f:
         kats = json.load(f)
-    assert len(kats) >= 7
+    assert len(kats) >= 13
     for kat in kats:
         packed = _blocks(bytes.fromhex(kat["hex"]))
         qt = kat["type"]
