@@ -1,7 +1,7 @@
 // Fused dequant-GEMV for decode (M <= 16) on the vector ALU: the path for Q8_0 rows that are not a
-// whole number of 256-element runs and for the formats without a matrix-core kernel (the
-// dispatcher at the end of this file sends Q8_0 with K % 256 == 0 and all Q4_K / Q5_K / Q6_K
-// shapes to the matrix-core kernels).
+// whole number of 256-element runs and for the other 32-element formats when K % 256 != 0 (the
+// dispatcher at the end of this file sends everything with K % 256 == 0 to the matrix-core
+// kernels).
 //
 // K % 64 == 0: one wavefront owns two weight rows (or, for the SiLU-gated pair, row n of the gate
 // matrix and row n of the up matrix); a lane takes 64 weight elements (68 packed bytes) per step,
@@ -134,8 +134,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x,
 }
 
 // Every other case - Q8_0 rows whose block count is odd (not a whole number of 64-element units,
-// rows only 2-byte aligned) and the formats without a kernel of their own (Q4_0, Q4_1, Q5_0,
-// Q5_1, Q2_K, Q3_K) - takes this plain path: one wavefront per row (GATED: row n of the gate and
+// rows only 2-byte aligned) and Q4_0 / Q4_1 / Q5_0 / Q5_1 rows that are not a whole number of
+// 256-element runs - takes this plain path: one wavefront per row (GATED: row n of the gate and
 // of the up matrix), eight elements per lane and step through the shared 8-element decoder.
 template <int QT, int NUM, bool GATED>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
@@ -261,10 +261,9 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     bf16_t* yp = static_cast<bf16_t*>(y);
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
-    if (qtype == SNGGUF_TYPE_Q4_K || qtype == SNGGUF_TYPE_Q5_K || qtype == SNGGUF_TYPE_Q6_K)
+    if (qtype != SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
-    // Q8_0 rows that are not a whole number of 256-element runs, and the formats served by the
-    // generic kernel
+    // rows that are not a whole number of 256-element runs
 #define SNGGUF_CALL(QT) launch_num<QT>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream)
     SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
 #undef SNGGUF_CALL

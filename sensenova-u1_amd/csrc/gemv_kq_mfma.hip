@@ -1,4 +1,6 @@
-// Q4_K / Q5_K / Q6_K decode GEMV on the matrix cores (1 <= M <= 16, K % 256 == 0).
+// Decode GEMV on the matrix cores for every format but Q8_0 (1 <= M <= 16, K % 256 == 0): the
+// K-quants Q2_K .. Q6_K, one 256-element super-block per step, and the 32-element formats Q4_0,
+// Q4_1, Q5_0, Q5_1, eight blocks per step.
 //
 // Same shape as the Q8_0 kernel: a workgroup owns R * 16 weight rows (for the SiLU-gated pair the
 // same rows of the gate and of the up matrix, on separate wavefronts), its wavefronts split K by
@@ -8,7 +10,9 @@
 //     along a row, one super-block ahead, and dropped into the wavefront's private LDS slab.  Q4_K
 //     and Q5_K super-blocks (144 / 176 bytes) are 16-byte aligned; Q6_K super-blocks (210 bytes) are only 2-byte
 //     aligned and are fetched as 13 unaligned 16-byte pieces plus the 2-byte scale, which never
-//     touches a byte outside the super-block and puts every field at an aligned LDS address;
+//     touches a byte outside the super-block and puts every field at an aligned LDS address; Q2_K
+//     (84 bytes) and Q3_K (110 bytes) take their last piece from the last 16 bytes of the
+//     super-block, so it overlaps the piece before it in memory but not in the slab;
 //   * lane (r = lane % 16, g = lane / 16) decodes, for each 32-element sub-block j, elements
 //     8 g .. 8 g + 7 of row r to bf16 (rounding chain by numerics mode) as the A operand of
 //     v_mfma_f32_16x16x32_bf16; the B operand is x[m = lane % 16][256 s + 32 j + 8 g ..].  With R = 2
@@ -80,19 +84,162 @@ __device__ __forceinline__ void kq_dword_bf16(half4_t ident, uint32_t v, float z
     }
 }
 
+// Slab<QT>: how the `ts` bytes that hold 256 elements of one row travel to the wavefront's LDS slab.
+// `pieces` 16-byte loads per row; piece p comes from byte 16 p of the run, except that the last one
+// comes from byte `last_src` (formats whose run is not a multiple of 16 bytes end with a piece that
+// overlaps its predecessor in memory); piece p lands at byte 16 p of the row's `stride`-byte slot.
+// `align` is what the format guarantees for the address of a run when the matrix is 16-byte aligned.
+// Strides are chosen so that 16 rows start in 16 different groups of four LDS banks.
 template <int QT> struct Slab;
-// Q4_K: 9 pieces per row and super-block, rows back to back (144 = 9 * 16)
+template <> struct Slab<SNGGUF_TYPE_Q4_0> {  // 8 blocks of 18 bytes
+    static constexpr int ts = 144, pieces = 9, last_src = 128, stride = 144, align = 16;
+};
+template <> struct Slab<SNGGUF_TYPE_Q4_1> {  // 8 blocks of 20 bytes
+    static constexpr int ts = 160, pieces = 10, last_src = 144, stride = 176, align = 16;
+};
+template <> struct Slab<SNGGUF_TYPE_Q5_0> {  // 8 blocks of 22 bytes
+    static constexpr int ts = 176, pieces = 11, last_src = 160, stride = 176, align = 16;
+};
+template <> struct Slab<SNGGUF_TYPE_Q5_1> {  // 8 blocks of 24 bytes
+    static constexpr int ts = 192, pieces = 12, last_src = 176, stride = 208, align = 16;
+};
+// Q2_K: bytes 0..79 (scales, quants) as five pieces, bytes 68..83 as the sixth: d, dmin land at slab bytes 92, 94
+template <> struct Slab<SNGGUF_TYPE_Q2_K> {
+    static constexpr int ts = 84, pieces = 6, last_src = 68, stride = 112, align = 4;
+};
+// Q3_K: bytes 0..95 (mask, quants) as six pieces, bytes 94..109 as the seventh: the 12 scale bytes land at slab
+// bytes 98..109, d at 110
+template <> struct Slab<SNGGUF_TYPE_Q3_K> {
+    static constexpr int ts = 110, pieces = 7, last_src = 94, stride = 112, align = 2;
+};
 template <> struct Slab<SNGGUF_TYPE_Q4_K> {
-    static constexpr int ts = 144, pieces = 9, stride = 144;
+    static constexpr int ts = 144, pieces = 9, last_src = 128, stride = 144, align = 16;
 };
-// Q5_K: 11 pieces per row and super-block (176 = 11 * 16); 44-dword rows fall on distinct bank groups
 template <> struct Slab<SNGGUF_TYPE_Q5_K> {
-    static constexpr int ts = 176, pieces = 11, stride = 176;
+    static constexpr int ts = 176, pieces = 11, last_src = 160, stride = 176, align = 16;
 };
-// Q6_K: 13 pieces (208 bytes) + the fp16 scale at byte 208; 240-byte rows fall on distinct banks
+// Q6_K: 13 pieces (208 bytes) + the fp16 scale at byte 208, fetched on its own
 template <> struct Slab<SNGGUF_TYPE_Q6_K> {
-    static constexpr int ts = 210, pieces = 13, stride = 240;
+    static constexpr int ts = 210, pieces = 13, last_src = 192, stride = 240, align = 2;
 };
+
+template <int ALIGN>
+__device__ __forceinline__ u32x4_t ld_piece(const uint8_t* p) {
+    if constexpr (ALIGN >= 16) return *reinterpret_cast<const u32x4_t*>(p);
+    else if constexpr (ALIGN >= 4) return ld_u128_a4(p);
+    else return ld_u128_a2(p);
+}
+
+// Eight bytes from slab address p, which is a multiple of 4 (ALIGNED) or 2 more than one.
+template <bool ALIGNED>
+__device__ __forceinline__ u32x2_t lds_u64(const uint8_t* p) {
+    if constexpr (ALIGNED) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(p);
+        return u32x2_t{w[0], w[1]};
+    } else {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(p - 2);
+        const uint32_t w0 = w[0], w1 = w[1], w2 = w[2];
+        return u32x2_t{__builtin_amdgcn_alignbit(w1, w0, 16), __builtin_amdgcn_alignbit(w2, w1, 16)};
+    }
+}
+template <bool ALIGNED>
+__device__ __forceinline__ uint32_t lds_u32(const uint8_t* p) {
+    if constexpr (ALIGNED) {
+        return *reinterpret_cast<const uint32_t*>(p);
+    } else {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(p - 2);
+        return __builtin_amdgcn_alignbit(w[1], w[0], 16);
+    }
+}
+
+// Q4_0 / Q4_1 / Q5_0 / Q5_1: sub-block jj of the half is block 4 HALF + jj of the eight in the slab
+// row.  TS block bytes; HAS_MIN: f16 m after d, value d q + m, else d (q - 8 or 16); FIVE: 32-bit
+// fifth-bit word before the quants.  Lane group g covers elements 8 g .. 8 g + 7: bytes
+// 8 (g % 2) .. of qs, low nibbles for g < 2, high nibbles otherwise; fifth bits = byte g of qh.
+template <int NUM, int B, int TS, bool HAS_MIN, bool FIVE>
+__device__ __forceinline__ u32x4_t legacy_block(half4_t ident, const uint8_t* row, int g) {
+    typedef Num<NUM> A;
+    constexpr int kHdr = HAS_MIN ? 4 : 2;
+    constexpr int kQs = kHdr + (FIVE ? 4 : 0);
+    constexpr float kZero = HAS_MIN ? 0.f : (FIVE ? 16.f : 8.f);
+    const uint8_t* blk = row + B * TS;
+    const typename A::T d = A::scale(*reinterpret_cast<const uint16_t*>(blk));
+    typename A::T DM = d;
+    if constexpr (HAS_MIN) DM = -A::scale(*reinterpret_cast<const uint16_t*>(blk + 2));
+    const int sh = 4 * (g >> 1);
+    const u32x2_t qs = lds_u64<((B * TS + kQs) & 3) == 0>(blk + kQs + 8 * (g & 1));
+    uint32_t v0 = (qs[0] >> sh) & 0x0F0F0F0Fu, v1 = (qs[1] >> sh) & 0x0F0F0F0Fu;
+    if constexpr (FIVE) {
+        const uint32_t bits = lds_u32<((B * TS + kHdr) & 3) == 0>(blk + kHdr) >> (8 * g);
+        // bits 0..3 -> bit 4 of bytes 0..3
+        v0 |= (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+        v1 |= ((((bits >> 4) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+    }
+    uint32_t a0, a1, a2, a3;
+    kq_dword_bf16<NUM, HAS_MIN>(ident, v0, kZero, d, DM, a0, a1);
+    kq_dword_bf16<NUM, HAS_MIN>(ident, v1, kZero, d, DM, a2, a3);
+    return u32x4_t{a0, a1, a2, a3};
+}
+template <int NUM, int HALF, int TS, bool HAS_MIN, bool FIVE, typename Emit>
+__device__ __forceinline__ void decode_legacy(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    emit(0, legacy_block<NUM, 4 * HALF + 0, TS, HAS_MIN, FIVE>(ident, row, g));
+    emit(1, legacy_block<NUM, 4 * HALF + 1, TS, HAS_MIN, FIVE>(ident, row, g));
+    emit(2, legacy_block<NUM, 4 * HALF + 2, TS, HAS_MIN, FIVE>(ident, row, g));
+    emit(3, legacy_block<NUM, 4 * HALF + 3, TS, HAS_MIN, FIVE>(ident, row, g));
+}
+
+// Q2_K: element 128 h + 32 j + l is bit pair j of qs[32 h + l]; its 16-element group
+// 8 h + 2 j + l / 16 has scale (low nibble) and min (high nibble) in one byte.
+template <int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_q2_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    typedef Num<NUM> A;
+    constexpr int h = HALF;
+    const u32x2_t sm = *reinterpret_cast<const u32x2_t*>(row + 8 * h);  // groups 8 h .. 8 h + 7
+    const uint32_t dd = *reinterpret_cast<const uint32_t*>(row + 92);
+    const typename A::T d = A::scale((uint16_t)(dd & 0xFFFF)), dmin = A::scale((uint16_t)(dd >> 16));
+    const u32x2_t qs = *reinterpret_cast<const u32x2_t*>(row + 16 + 32 * h + 8 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t byte = (sm[j >> 1] >> (8 * (2 * (j & 1) + (g >> 1)))) & 0xFFu;
+        const typename A::T D = d * A::integer((int)(byte & 15u)), DM = dmin * A::integer((int)(byte >> 4));
+        uint32_t a0, a1, a2, a3;
+        kq_dword_bf16<NUM, true>(ident, (qs[0] >> (2 * j)) & 0x03030303u, 0.f, D, DM, a0, a1);
+        kq_dword_bf16<NUM, true>(ident, (qs[1] >> (2 * j)) & 0x03030303u, 0.f, D, DM, a2, a3);
+        emit(j, u32x4_t{a0, a1, a2, a3});
+    }
+}
+
+// Q3_K: stored quant (0..7) = bit pair as in Q2_K | mask bit (4 h + j of hmask[l]) << 2, value
+// stored - 4; 6-bit group scales split over the 12 scale bytes, value stored - 32.
+template <int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_q3_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    typedef Num<NUM> A;
+    constexpr int h = HALF;
+    const u32x4_t t = *reinterpret_cast<const u32x4_t*>(row + 96);  // source bytes 94..109
+    const uint32_t s0 = __builtin_amdgcn_alignbit(t[1], t[0], 16);  // scale bytes 0..3
+    const uint32_t s1 = __builtin_amdgcn_alignbit(t[2], t[1], 16);  // 4..7
+    const uint32_t s2 = __builtin_amdgcn_alignbit(t[3], t[2], 16);  // 8..11
+    const typename A::T d = A::scale((uint16_t)(t[3] >> 16));
+    const u32x2_t hm = *reinterpret_cast<const u32x2_t*>(row + 8 * g);
+    const u32x2_t qs = *reinterpret_cast<const u32x2_t*>(row + 32 + 32 * h + 8 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        // group 8 h + tt, tt = 2 j + g / 2: low nibble in byte tt (upper nibble for h = 1), high bits in
+        // byte 8 + tt % 4 at bit 2 (2 h + tt / 4)
+        const int t3 = (2 * (j & 1) + (g >> 1));  // tt % 4
+        const uint32_t lo = (((j < 2 ? s0 : s1) >> (8 * t3)) >> (4 * h)) & 15u;
+        const uint32_t hi = (((s2 >> (8 * t3)) & 0xFFu) >> (2 * (2 * h + (j >> 1)))) & 3u;
+        const typename A::T D = d * A::integer((int)(lo | (hi << 4)) - 32);
+        uint32_t a[4];
+#pragma unroll
+        for (int w = 0; w < 2; w++) {
+            const uint32_t v = ((qs[w] >> (2 * j)) & 0x03030303u) | (((hm[w] >> (4 * h + j)) & 0x01010101u) << 2);
+            kq_dword_bf16<NUM, false>(ident, v, 4.f, D, D, a[2 * w], a[2 * w + 1]);
+        }
+        emit(j, u32x4_t{a[0], a[1], a[2], a[3]});
+    }
+}
+
 
 // The four A operands of half a super-block (sub-blocks 4 HALF .. 4 HALF + 3) of one row, fed to
 // `emit(jj, a)` with jj = 0..3.  `row` points at the row's super-block in the slab; g = lane / 16.
@@ -178,6 +325,23 @@ __device__ __forceinline__ void decode_q6_k(half4_t ident, const uint8_t* row, i
     }
 }
 
+// One half (sub-blocks 4 HALF .. 4 HALF + 3) of a slab row -> four A operands through `emit(jj, a)`.
+template <int QT, int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_half(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    if constexpr (QT == SNGGUF_TYPE_Q4_0) decode_legacy<NUM, HALF, 18, false, false>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_1) decode_legacy<NUM, HALF, 20, true, false>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_0) decode_legacy<NUM, HALF, 22, false, true>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_1) decode_legacy<NUM, HALF, 24, true, true>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q2_K) decode_q2_k<NUM, HALF>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q3_K) decode_q3_k<NUM, HALF>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode_q4_k<NUM, HALF>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode_q5_k<NUM, HALF>(ident, row, g, emit);
+    else {
+        static_assert(QT == SNGGUF_TYPE_Q6_K, "no matrix-core decoder for this quant type");
+        decode_q6_k<NUM, HALF>(ident, row, g, emit);
+    }
+}
+
 template <int QT, int NUM, int R, bool GATED, int WMAX>
 __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
@@ -212,7 +376,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
         const int fr = ok ? f / S::pieces : 0, fp = ok ? f % S::pieces : 0;
         int64_t n = n0 + fr;
         if (n >= N) n = N - 1;  // rows past the end are decoded from the last row and never stored
-        off[i] = (uint32_t)((n - n0) * row_bytes + 16 * fp);
+        off[i] = (uint32_t)((n - n0) * row_bytes + (fp == S::pieces - 1 ? S::last_src : 16 * fp));
         dst[i] = (uint32_t)(fr * S::stride + 16 * fp);
     }
     const bool tail_lane = lane + 64 * (kLoads - 1) < kPieces;
@@ -234,8 +398,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     auto fetch = [&](int s) {
         const uint8_t* p = base + (int64_t)s * S::ts;
 #pragma unroll
-        for (int i = 0; i < kLoads - 1; i++) pre[i] = kQ6 ? ld_u128_a2(p + off[i]) : *reinterpret_cast<const u32x4_t*>(p + off[i]);
-        if (tail_lane) pre[kLoads - 1] = kQ6 ? ld_u128_a2(p + off[kLoads - 1]) : *reinterpret_cast<const u32x4_t*>(p + off[kLoads - 1]);
+        for (int i = 0; i < kLoads - 1; i++) pre[i] = ld_piece<S::align>(p + off[i]);
+        if (tail_lane) pre[kLoads - 1] = ld_piece<S::align>(p + off[kLoads - 1]);
         if constexpr (kQ6) {
             if (lane < kRows) pre_d = ld_u16(p + doff);
         }
@@ -270,9 +434,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                 acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                                   __builtin_bit_cast(bf16x8_t, xa[jj]), acc[rg], 0, 0, 0);
             };
-            if constexpr (kQ6) decode_q6_k<NUM, 0>(ident, row, g, emit);
-            else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode_q5_k<NUM, 0>(ident, row, g, emit);
-            else decode_q4_k<NUM, 0>(ident, row, g, emit);
+            decode_half<QT, NUM, 0>(ident, row, g, emit);
         }
         if (s + 1 < s1) load_x(s + 1, 0, xa);
 #pragma unroll
@@ -282,9 +444,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                 acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                                   __builtin_bit_cast(bf16x8_t, xb[jj]), acc[rg], 0, 0, 0);
             };
-            if constexpr (kQ6) decode_q6_k<NUM, 1>(ident, row, g, emit);
-            else if constexpr (QT == SNGGUF_TYPE_Q5_K) decode_q5_k<NUM, 1>(ident, row, g, emit);
-            else decode_q4_k<NUM, 1>(ident, row, g, emit);
+            decode_half<QT, NUM, 1>(ident, row, g, emit);
         }
     };
     if (s0 < s1) {
@@ -381,7 +541,7 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
 
 }  // namespace
 
-// Q4_K, Q5_K or Q6_K, 1 <= M <= 16, K % 256 == 0, 16-byte aligned x and q (checked by the caller).
+// Any format but Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned x and q (checked by the caller).
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
@@ -389,14 +549,23 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
     bf16_t* yp = static_cast<bf16_t*>(y);
-#define SNGGUF_CASE(QT, NUM) \
-    if (qtype == QT && numerics == NUM) return launch_qt<QT, NUM>(xp, (int)M, a, b, N, K, bp, yp, gated, stream)
-    SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_GGML_FP32);
-    SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_UPSTREAM_FP16);
-    SNGGUF_CASE(SNGGUF_TYPE_Q5_K, SNGGUF_NUM_GGML_FP32);
-    SNGGUF_CASE(SNGGUF_TYPE_Q5_K, SNGGUF_NUM_UPSTREAM_FP16);
-    SNGGUF_CASE(SNGGUF_TYPE_Q6_K, SNGGUF_NUM_GGML_FP32);
-    SNGGUF_CASE(SNGGUF_TYPE_Q6_K, SNGGUF_NUM_UPSTREAM_FP16);
+#define SNGGUF_CASE(QT)                                                                                          \
+    if (qtype == QT) {                                                                                           \
+        if (numerics == SNGGUF_NUM_GGML_FP32)                                                                    \
+            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);          \
+        if (numerics == SNGGUF_NUM_UPSTREAM_FP16)                                                                \
+            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);      \
+        return SNGGUF_E_BADTYPE;                                                                                 \
+    }
+    SNGGUF_CASE(SNGGUF_TYPE_Q4_0)
+    SNGGUF_CASE(SNGGUF_TYPE_Q4_1)
+    SNGGUF_CASE(SNGGUF_TYPE_Q5_0)
+    SNGGUF_CASE(SNGGUF_TYPE_Q5_1)
+    SNGGUF_CASE(SNGGUF_TYPE_Q2_K)
+    SNGGUF_CASE(SNGGUF_TYPE_Q3_K)
+    SNGGUF_CASE(SNGGUF_TYPE_Q4_K)
+    SNGGUF_CASE(SNGGUF_TYPE_Q5_K)
+    SNGGUF_CASE(SNGGUF_TYPE_Q6_K)
 #undef SNGGUF_CASE
     return SNGGUF_E_BADTYPE;
 }

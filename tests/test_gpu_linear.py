@@ -48,7 +48,7 @@ def test_gemv_shapes_bias_ragged(dev, c_oracle, qt):
         _check(got, c_oracle.linear(x, packed, qt, bias))
 
 
-@pytest.mark.parametrize("qt", [go.Q4_K, go.Q5_K, go.Q6_K])
+@pytest.mark.parametrize("qt", [t for t in TYPES if t != go.Q8_0])
 @pytest.mark.parametrize("numerics", [0, 1])
 def test_gemv_k_quants_two_row_groups(dev, c_oracle, qt, numerics):
     """N >= 32768 puts two 16-row groups on one wavefront: ragged N (last group half empty, last
@@ -68,6 +68,25 @@ def test_gemv_k_quants_two_row_groups(dev, c_oracle, qt, numerics):
     u = go.gguf_linear_forward(x, up, qt, numerics=numerics)
     got = ops.gate_up_silu(x.to(dev), gate.to(dev), up.to(dev), qt, numerics).cpu()
     _check(got, c_oracle.silu_mul(g, u))
+
+
+@pytest.mark.parametrize("qt", [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1])
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_gemv_32_element_formats_ragged_k(dev, c_oracle, qt, numerics):
+    """K a multiple of 32 but not of 256 (the vector-ALU path; rows only 2-byte aligned for the 18- and
+    22-byte blocks), plain with bias and SiLU-gated."""
+    print(f"case gemv ragged K qt={qt} numerics={numerics}", flush=True)
+    for n, k, m in [(37, 32, 1), (130, 96, 16), (9, 4128, 5)]:
+        packed = synthetic.make_packed(qt, n, k, seed=n + k)
+        x = synthetic.make_activations(m, k, seed=k + 1)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16)
+        got = ops.linear(x.to(dev), packed.to(dev), qt, bias.to(dev), numerics).cpu()
+        _check(got, c_oracle.linear(x, packed, qt, bias, numerics))
+        up = synthetic.make_packed(qt, n, k, seed=n + k + 1)
+        g = go.gguf_linear_forward(x, packed, qt, numerics=numerics)
+        u = go.gguf_linear_forward(x, up, qt, numerics=numerics)
+        got = ops.gate_up_silu(x.to(dev), packed.to(dev), up.to(dev), qt, numerics).cpu()
+        _check(got, c_oracle.silu_mul(g, u))
 
 
 def test_gemv_q8_0_odd_block_count(dev):
