@@ -68,7 +68,9 @@ enum {
     SNGGUF_E_NULLPTR = -3,   /* a required pointer is NULL                                    */
     SNGGUF_E_ALIGN = -4,     /* a pointer violates the alignment stated for it                */
     SNGGUF_E_LAUNCH = -5,    /* the HIP runtime refused the launch (hipGetLastError != 0)     */
-    SNGGUF_E_NODEVICE = -6   /* no usable gfx950 device / code object                         */
+    SNGGUF_E_NODEVICE = -6,  /* no usable gfx950 device / code object                         */
+    SNGGUF_E_IO = -7,        /* a file could not be opened or mapped                          */
+    SNGGUF_E_FORMAT = -8     /* not a GGUF file, truncated, corrupt, or a tensor type of unknown size */
 };
 
 /* Library version (major*10000 + minor*100 + patch) and error text. */
@@ -141,6 +143,55 @@ int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, in
                           const void* q_und, int qtype_und, const void* q_gen, int qtype_gen,
                           int64_t N, int64_t K, const void* bias_und, const void* bias_gen,
                           void* y, void* workspace, int numerics, void* stream);
+
+/*
+ * ---- GGUF container reader (host only, no GPU call) -----------------------------------
+ * What the reference gets from gguf.GGUFReader at
+ * src/sensenova_u1/utils/gguf_loader.py:29-44: open the file, walk `reader.tensors`, read each
+ * tensor's name, ggml type and shape, and copy its bytes out of the file mapping (`:42`).
+ * The file is mapped read-only; header, metadata and tensor infos (GGUF v2 / v3) are parsed
+ * with a bounds check on every read, so a truncated or corrupt file gives SNGGUF_E_FORMAT,
+ * never a fault.  `data` / `value` pointers and strings stay valid until sngguf_file_close.
+ */
+typedef struct sngguf_file sngguf_file;
+
+typedef struct sngguf_tensor_info {
+    const char* name;     /* the state-dict key, NUL-terminated                              */
+    int32_t ggml_type;    /* GGMLQuantizationType number                                     */
+    int32_t n_dims;       /* 0..4                                                            */
+    int64_t dims[4];      /* ggml order: dims[0] is the row length (in_features); unused = 1 */
+    int64_t n_elements;
+    int64_t n_bytes;      /* n_elements / block * type_size                                  */
+    int64_t file_offset;  /* of the payload, from the start of the file                      */
+    const void* data;     /* the payload inside the read-only mapping                        */
+} sngguf_tensor_info;
+
+typedef struct sngguf_metadata_info {
+    const char* key;
+    int32_t value_type;   /* GGUF value type: 0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool,
+                             8 string, 9 array, 10 u64, 11 i64, 12 f64                        */
+    int32_t item_type;    /* arrays: value type of the items; otherwise -1                   */
+    int64_t count;        /* arrays: number of items; strings: byte length; scalars: 1       */
+    const void* value;    /* the encoded value as it stands in the file (little endian;
+                             strings and arrays start with their length words)               */
+    int64_t value_bytes;  /* encoded length of the value                                     */
+} sngguf_metadata_info;
+
+/* Opens, maps and parses `path`.  On failure *out is NULL, the return value is negative and
+ * `err` (if not NULL, `err_len` bytes) receives a NUL-terminated message. */
+int sngguf_file_open(const char* path, sngguf_file** out, char* err, int64_t err_len);
+void sngguf_file_close(sngguf_file* f);
+int sngguf_file_version(const sngguf_file* f);
+int64_t sngguf_file_alignment(const sngguf_file* f);   /* general.alignment, default 32 */
+int64_t sngguf_file_tensor_count(const sngguf_file* f);
+int sngguf_file_tensor(const sngguf_file* f, int64_t index, sngguf_tensor_info* out);
+int64_t sngguf_file_metadata_count(const sngguf_file* f);
+int sngguf_file_metadata(const sngguf_file* f, int64_t index, sngguf_metadata_info* out);
+/* Copies the payloads of `count` tensors (file order numbers in `indices`) to dst[i], each of at
+ * least n_bytes, with up to `threads` threads working on 8 MiB pieces: the copy at
+ * gguf_loader.py:42, into buffers the caller chose (pinned host memory, for instance). */
+int sngguf_file_read_tensors(const sngguf_file* f, const int64_t* indices, void* const* dst,
+                             int64_t count, int threads);
 
 #ifdef __cplusplus
 }

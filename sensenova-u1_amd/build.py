@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libsngguf.so")
-SOURCES = ["api.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemm.hip", "gemm_tiles.hip"]
+SOURCES = ["api.cpp", "gguf_reader.cpp", "dequantize.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemm.hip", "gemm_tiles.hip"]
 
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIP_FLAGS = [
@@ -62,7 +62,7 @@ def build_library(force: bool = True, extra_flags: list[str] | None = None, jobs
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda so: _compile(so[0], so[1], extra_flags or []), zip(SOURCES, objs)))
     tmp = LIB_PATH + ".tmp"
-    res = subprocess.run([_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", tmp, *objs],
+    res = subprocess.run([_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-pthread", "-o", tmp, *objs],
                          capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")

@@ -52,6 +52,8 @@ const char* sngguf_strerror(int code) {
     case SNGGUF_E_ALIGN: return "pointer is not aligned as required";
     case SNGGUF_E_LAUNCH: return "HIP kernel launch failed";
     case SNGGUF_E_NODEVICE: return "no usable gfx950 device";
+    case SNGGUF_E_IO: return "file could not be opened or mapped";
+    case SNGGUF_E_FORMAT: return "not a GGUF file, or truncated / corrupt";
     default: return "unknown error";
     }
 }

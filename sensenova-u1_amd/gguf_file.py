@@ -5,7 +5,9 @@ The reference parses files with the third-party ``gguf`` package
 ``.tensor_type`` and ``.data``).  This module provides those three attributes, the
 ``GGMLQuantizationType`` numbering and ``GGML_QUANT_SIZES`` from the public GGUF
 specification, so that the loader needs no external package; the writer exists so that tests
-and tools can produce files.
+and tools can produce files.  ``NativeGGUFReader`` gives the same view through the C++ reader
+of libsngguf.so (``sngguf_file_*``) and is what the checkpoint loader uses; ``GGUFReader`` is
+the pure-Python counterpart.
 
 Layout (little endian): magic ``GGUF``, u32 version, u64 tensor count, u64 metadata count,
 metadata key/values, tensor infos (name, u32 n_dims, u64 dims fastest-first, u32 type, u64
@@ -13,7 +15,9 @@ offset), padding to ``general.alignment`` (default 32), tensor data.
 """
 from __future__ import annotations
 
+import ctypes
 import mmap
+import os
 import struct
 from enum import IntEnum
 from typing import Any, Iterable
@@ -235,6 +239,131 @@ class GGUFReader:
 
     def __exit__(self, *exc):
         self.close()
+
+
+class _TensorInfo(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("ggml_type", ctypes.c_int32), ("n_dims", ctypes.c_int32),
+                ("dims", ctypes.c_int64 * 4), ("n_elements", ctypes.c_int64), ("n_bytes", ctypes.c_int64),
+                ("file_offset", ctypes.c_int64), ("data", ctypes.c_void_p)]
+
+
+class _MetadataInfo(ctypes.Structure):
+    _fields_ = [("key", ctypes.c_char_p), ("value_type", ctypes.c_int32), ("item_type", ctypes.c_int32),
+                ("count", ctypes.c_int64), ("value", ctypes.c_void_p), ("value_bytes", ctypes.c_int64)]
+
+
+def _decode_value(buf: bytes, pos: int, vtype: int):
+    """One encoded GGUF metadata value at ``buf[pos:]`` -> (python value, next position)."""
+    vtype = GGUFValueType(vtype)
+    if vtype == GGUFValueType.STRING:
+        (n,) = struct.unpack_from("<Q", buf, pos)
+        return buf[pos + 8:pos + 8 + n].decode("utf-8", errors="replace"), pos + 8 + n
+    if vtype == GGUFValueType.ARRAY:
+        item_type, count = struct.unpack_from("<IQ", buf, pos)
+        pos += 12
+        items = []
+        for _ in range(count):
+            v, pos = _decode_value(buf, pos, item_type)
+            items.append(v)
+        return items, pos
+    fmt = _SCALAR_FMT[vtype]
+    (v,) = struct.unpack_from(fmt, buf, pos)
+    return v, pos + struct.calcsize(fmt)
+
+
+class NativeGGUFReader:
+    """The same view of a file as ``GGUFReader`` (``version``, ``alignment``, ``fields``, ``tensors``
+    with numpy views into the mapping), parsed and mapped by the C++ reader inside libsngguf.so.
+    ``read_into`` copies payloads to caller-chosen host buffers with several threads."""
+
+    def __init__(self, path: str):
+        from . import ops
+        self._lib = ops.load_library()
+        handle = ctypes.c_void_p()
+        err = ctypes.create_string_buffer(1024)
+        rc = self._lib.sngguf_file_open(os.fsencode(path), ctypes.byref(handle), err, len(err))
+        if rc != 0:
+            msg = err.value.decode("utf-8", errors="replace")
+            if rc == -7:
+                raise OSError(msg)
+            raise ValueError(msg if msg.startswith(path) else f"{path}: {msg}")
+        self._handle = handle
+        self.version = self._lib.sngguf_file_version(handle)
+        self.alignment = self._lib.sngguf_file_alignment(handle)
+        self.fields: dict[str, Any] = {}
+        info = _MetadataInfo()
+        for i in range(self._lib.sngguf_file_metadata_count(handle)):
+            self._lib.sngguf_file_metadata(handle, i, ctypes.byref(info))
+            raw = ctypes.string_at(info.value, info.value_bytes)
+            self.fields[info.key.decode("utf-8", errors="replace")] = _decode_value(raw, 0, info.value_type)[0]
+        self.tensors: list[ReaderTensor] = []
+        tinfo = _TensorInfo()
+        for i in range(self._lib.sngguf_file_tensor_count(handle)):
+            self._lib.sngguf_file_tensor(handle, i, ctypes.byref(tinfo))
+            name = tinfo.name.decode("utf-8", errors="replace")
+            try:
+                qtype = GGMLQuantizationType(tinfo.ggml_type)
+            except ValueError as exc:
+                self.close()
+                raise ValueError(f"{path}: tensor {name} has unknown ggml type {tinfo.ggml_type}") from exc
+            block, tsize = GGML_QUANT_SIZES[qtype]
+            dims = [int(tinfo.dims[d]) for d in range(tinfo.n_dims)]
+            np_dims = list(reversed(dims)) if dims else [1]
+            if tinfo.n_bytes:
+                flat = np.ctypeslib.as_array(ctypes.cast(tinfo.data, ctypes.POINTER(ctypes.c_uint8)), shape=(tinfo.n_bytes,))
+            else:
+                flat = np.empty((0,), dtype=np.uint8)
+            flat.flags.writeable = False
+            if qtype in _PLAIN_DTYPES:
+                arr = flat.view(_PLAIN_DTYPES[qtype]).reshape(np_dims)
+            else:
+                np_dims[-1] = np_dims[-1] // block * tsize
+                arr = flat.reshape(np_dims)
+            self.tensors.append(ReaderTensor(name, qtype, dims, int(tinfo.n_elements), int(tinfo.n_bytes),
+                                             int(tinfo.file_offset), arr))
+
+    def read_into(self, indices, buffers, threads: int = 8) -> None:
+        """Copy the payloads of tensors ``indices`` (positions in ``tensors``) into ``buffers``:
+        objects with the buffer protocol or ``data_ptr()`` (torch tensors), each at least as large."""
+        n = len(indices)
+        idx = (ctypes.c_int64 * n)(*indices)
+        dst = (ctypes.c_void_p * n)()
+        for i, (t, b) in enumerate(zip(indices, buffers)):
+            need = self.tensors[t].n_bytes
+            if hasattr(b, "data_ptr"):
+                have, ptr = b.numel() * b.element_size(), b.data_ptr()
+                if not b.is_contiguous() or b.device.type != "cpu":
+                    raise ValueError("read_into needs contiguous host tensors")
+            else:
+                view = np.asarray(b)
+                if not view.flags.c_contiguous or not view.flags.writeable:
+                    raise ValueError("read_into needs contiguous writable buffers")
+                have, ptr = view.nbytes, view.ctypes.data
+            if have < need:
+                raise ValueError(f"buffer for tensor {self.tensors[t].name} holds {have} bytes, needs {need}")
+            dst[i] = ptr
+        rc = self._lib.sngguf_file_read_tensors(self._handle, idx, dst, n, int(threads))
+        if rc != 0:
+            raise RuntimeError(f"sngguf_file_read_tensors failed: {rc}")
+
+    def close(self) -> None:
+        """Unmaps the file: arrays in ``tensors`` must not be used afterwards."""
+        self.tensors = []
+        if getattr(self, "_handle", None):
+            self._lib.sngguf_file_close(self._handle)
+            self._handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class GGUFWriter:

@@ -15,7 +15,7 @@ import gc
 import torch
 from torch import nn
 
-from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader
+from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, NativeGGUFReader
 from .quantized_linear import (
     SUPPORTED_GGUF_QUANT_TYPES,
     GGUFLinear,
@@ -25,26 +25,38 @@ from .quantized_linear import (
 )
 
 
-def load_gguf_checkpoint(gguf_checkpoint_path: str) -> dict:
+_TORCH_PLAIN = {GGMLQuantizationType.F32: torch.float32, GGMLQuantizationType.F16: torch.float16}
+
+
+def load_gguf_checkpoint(gguf_checkpoint_path: str, pin_memory: bool = False, threads: int = 8) -> dict:
     """Parse a .gguf file into a state-dict-compatible mapping.
 
     F32 / F16 tensors come back as plain torch tensors; every other type must be one the HIP
     kernels decode and is wrapped in ``GGUFParameter`` (packed bytes, copied out of the file
     mapping).  Tensor names are used verbatim: GGUF names are the model's state-dict keys.
+
+    The file is parsed by the library's C++ reader and all payloads are copied in one
+    multi-threaded pass into freshly allocated host tensors - page-locked ones with
+    ``pin_memory=True``, ready for asynchronous upload.
     """
-    reader = GGUFReader(gguf_checkpoint_path)
+    reader = NativeGGUFReader(gguf_checkpoint_path)
     parsed: dict = {}
     try:
+        kinds = []
         for tensor in reader.tensors:
-            name = tensor.name
             quant_type = tensor.tensor_type
-            is_quant = quant_type not in (GGMLQuantizationType.F32, GGMLQuantizationType.F16)
+            is_quant = quant_type not in _TORCH_PLAIN
             if is_quant and quant_type not in SUPPORTED_GGUF_QUANT_TYPES:
                 supported = "\n".join(str(t) for t in SUPPORTED_GGUF_QUANT_TYPES)
-                raise ValueError(f"{name} has unsupported quant type {quant_type!s}.\nSupported:\n{supported}")
-            weights = torch.from_numpy(tensor.data.copy())
-            parsed[name] = GGUFParameter(weights, quant_type=quant_type) if is_quant else weights
-            del tensor, weights
+                raise ValueError(f"{tensor.name} has unsupported quant type {quant_type!s}.\nSupported:\n{supported}")
+            kinds.append(is_quant)
+        buffers = []
+        for tensor, is_quant in zip(reader.tensors, kinds):
+            dtype = torch.uint8 if is_quant else _TORCH_PLAIN[tensor.tensor_type]
+            buffers.append(torch.empty(tuple(tensor.data.shape), dtype=dtype, pin_memory=pin_memory))
+        reader.read_into(list(range(len(buffers))), buffers, threads=threads)
+        for tensor, is_quant, weights in zip(reader.tensors, kinds, buffers):
+            parsed[tensor.name] = GGUFParameter(weights, quant_type=tensor.tensor_type) if is_quant else weights
     finally:
         reader.close()
         del reader

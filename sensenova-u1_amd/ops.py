@@ -33,6 +33,8 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
     "sngguf_linear", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
+    "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
 
 _lib = None
@@ -72,6 +74,26 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_grouped_workspace_bytes.restype = i64
     lib.sngguf_grouped_linear.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, ci, vp]
     lib.sngguf_grouped_linear.restype = ci
+    # host-only GGUF container reader
+    cp = ctypes.c_char_p
+    lib.sngguf_file_open.argtypes = [cp, ctypes.POINTER(vp), cp, i64]
+    lib.sngguf_file_open.restype = ci
+    lib.sngguf_file_close.argtypes = [vp]
+    lib.sngguf_file_close.restype = None
+    lib.sngguf_file_version.argtypes = [vp]
+    lib.sngguf_file_version.restype = ci
+    lib.sngguf_file_alignment.argtypes = [vp]
+    lib.sngguf_file_alignment.restype = i64
+    lib.sngguf_file_tensor_count.argtypes = [vp]
+    lib.sngguf_file_tensor_count.restype = i64
+    lib.sngguf_file_tensor.argtypes = [vp, i64, vp]
+    lib.sngguf_file_tensor.restype = ci
+    lib.sngguf_file_metadata_count.argtypes = [vp]
+    lib.sngguf_file_metadata_count.restype = i64
+    lib.sngguf_file_metadata.argtypes = [vp, i64, vp]
+    lib.sngguf_file_metadata.restype = ci
+    lib.sngguf_file_read_tensors.argtypes = [vp, ctypes.POINTER(i64), ctypes.POINTER(vp), i64, ci]
+    lib.sngguf_file_read_tensors.restype = ci
     _lib = lib
     return lib
 
