@@ -243,6 +243,23 @@ def main() -> None:
         tflops = flops / (wall / gs * 1e-3) / 1e12
         _, ev_gate = run_region(gate_only, gs * 2, args.gemm_warmup)
         gate_ms = ev_gate / (gs * 2)
+
+        # the module's default for M > 16 (GGUFLinear.gemm_policy "auto"): one dequantize launch to a transient
+        # bf16 weight, then the device's dense GEMM (hipBLASLt through torch.matmul)
+        wtmp = torch.empty(INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
+
+        def two_pass(x, packed, n, k, y):
+            w = wtmp[:n * k].view(n, k)
+            ops.dequantize_into(packed, Q8_0, w, num)
+            torch.matmul(x, w.t(), out=y)
+
+        def tower_two_pass(i):
+            ws = tower[i % 2]
+            for j, (_, n, k) in enumerate(shapes):
+                two_pass(xs[k], ws[j], n, k, ys[n])
+
+        wall2, _ = run_region(tower_two_pass, gs, args.gemm_warmup)
+        _, ev_gate2 = run_region(lambda i: two_pass(xs[HIDDEN], tower[i % 2][4], INTER, HIDDEN, ys[INTER]), gs * 2, args.gemm_warmup)
         gate_tflops = 2.0 * m * INTER * HIDDEN / (gate_ms * 1e-3) / 1e12
         result["gemm"] = {
             "workload": "configs[2]: Q8_0 generation-tower projections over M=4096 image tokens "
@@ -265,8 +282,17 @@ def main() -> None:
                 "flop_per_launch": 2.0 * m * INTER * HIDDEN,
                 "avg_launch_us": round(gate_ms * 1e3, 2),
             },
+            "two_pass": {
+                "what": "same tower as sngguf dequantize (packed -> bf16, transient) + dense bf16 GEMM of the device "
+                        "library: what GGUFLinear does for M > 16 by default",
+                "value": round(flops / (wall2 / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                "ms_per_step": round(wall2 / gs, 4),
+                "pct_of_bf16_mfma_peak": round(100 * flops / (wall2 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+                "gate_us": round(ev_gate2 / (gs * 2) * 1e3, 2),
+                "gate_tflops": round(2.0 * m * INTER * HIDDEN / (ev_gate2 / (gs * 2) * 1e-3) / 1e12, 2),
+            },
         }
-        del tower, xs, ys
+        del tower, xs, ys, wtmp
 
     # ---- standalone dequantize (the reference's dequantize_gguf_tensor): packed [12288, 4096] -> fp16 -----------
     if not args.no_extra:
@@ -350,13 +376,29 @@ def main() -> None:
         wall, ev = run_region(layer_step, gs, max(2, args.gemm_warmup // 2))
         flops = sum(2.0 * m * n * k for _, n, k in shapes)
         tflops = flops / (wall / gs * 1e-3) / 1e12
+        wtmp = torch.empty(INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
+
+        def layer_two_pass(i):
+            for j, (_, n, k) in enumerate(shapes):
+                for packed, lo, hi in ((und[j], 0, n_text), (gen[j], n_text, m)):
+                    w = wtmp[:n * k].view(n, k)
+                    ops.dequantize_into(packed, Q8_0, w, num)
+                    torch.matmul(xs[k][lo:hi], w.t(), out=ys[n][lo:hi])
+
+        wall2, _ = run_region(layer_two_pass, gs, max(2, args.gemm_warmup // 2))
         result["grouped_layer"] = {
             "workload": "configs[4], one of the 36 layers: 512 text rows -> understanding weights, 4096 image rows -> "
                         "generation weights, 7 Q8_0 linears through the modality-grouped launcher (contiguous split)",
             "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall / gs, 4),
             "flop_per_layer": flops, "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+            "two_pass": {
+                "what": "per group: sngguf dequantize to a transient bf16 weight + dense bf16 GEMM into the group's rows "
+                        "(modality.grouped_linear with n_text, default policy)",
+                "value": round(flops / (wall2 / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall2 / gs, 4),
+                "pct_of_bf16_mfma_peak": round(100 * flops / (wall2 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            },
         }
-        del und, gen, xs, ys
+        del und, gen, xs, ys, wtmp
 
     # ---- CPU baseline: the oracle's port of GGUFLinear.forward_native on the host cores -----------
     if not args.no_cpu_baseline:

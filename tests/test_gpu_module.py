@@ -65,10 +65,51 @@ def test_grouped_modules(tmp_path, dev):
                                      8, torch.from_numpy(packed["layers.1.q_proj_mot_gen.weight"]), 8)
     assert go.rel_l2(got.cpu().reshape(60, H), want) <= TOL
     # the reference's production cases: all text -> understanding weights only, all image -> generation only
+    # (bit for bit when both sides run the library's fused kernels)
+    layer.q_proj.gemm_policy = layer.q_proj_mot_gen.gemm_policy = "fused"
     all_und = grouped_linear(x.to(dev), torch.zeros(2, 30, dtype=torch.bool, device=dev), layer.q_proj, layer.q_proj_mot_gen)
     assert torch.equal(all_und, layer.q_proj(x.to(dev)))
     all_gen = grouped_linear(x.to(dev), None, layer.q_proj, layer.q_proj_mot_gen, n_text=0)
     assert torch.equal(all_gen, layer.q_proj_mot_gen(x.to(dev)))
+    # contiguous [text | image] layout under both policies: fused kernel, and weight pass + dense GEMM per group
+    split = torch.arange(60) >= 22
+    want = go.grouped_linear_forward(x.reshape(60, H), split, torch.from_numpy(packed["layers.1.q_proj.weight"]),
+                                     8, torch.from_numpy(packed["layers.1.q_proj_mot_gen.weight"]), 8)
+    for policy in ("fused", "auto"):
+        layer.q_proj.gemm_policy = layer.q_proj_mot_gen.gemm_policy = policy
+        for n_text in (22, 0, 60, 5, 50):
+            got = grouped_linear(x.to(dev), None, layer.q_proj, layer.q_proj_mot_gen, n_text=n_text)
+            ind = (torch.arange(60) >= n_text)
+            want = go.grouped_linear_forward(x.reshape(60, H), ind, torch.from_numpy(packed["layers.1.q_proj.weight"]),
+                                             8, torch.from_numpy(packed["layers.1.q_proj_mot_gen.weight"]), 8)
+            assert got.shape == (2, 30, H) and go.rel_l2(got.cpu().reshape(60, H), want) <= TOL, (policy, n_text)
+
+
+@pytest.mark.parametrize("quant", [8, 12, 2, 11])
+def test_gemm_policies_agree_with_the_oracle(tmp_path, dev, quant):
+    """More than 16 rows: "fused" (library GEMM kernels) and "auto" / "two_pass" (bf16 weight pass + dense
+    GEMM) both reproduce the oracle; with and without bias; 3-d inputs keep their leading dims."""
+    print(f"case module gemm policies quant={quant}", flush=True)
+    model, packed = _load(tmp_path, dev, quant)
+    for name in ("layers.0.mlp.down_proj", "timestep_embedder"):
+        mod = model.get_submodule(name)
+        assert mod.gemm_policy == "auto"
+        for m in (17, 300):
+            x = synthetic.make_activations(2 * m, mod.in_features, seed=m)
+            want = go.gguf_linear_forward(x, torch.from_numpy(packed[name + ".weight"]), quant,
+                                          mod.bias.cpu() if mod.bias is not None else None)
+            outs = {}
+            for policy in ("auto", "two_pass", "fused"):
+                mod.gemm_policy = policy
+                got = mod(x.to(dev).reshape(2, m, -1))
+                assert got.shape == (2, m, mod.out_features) and got.dtype == torch.bfloat16
+                assert go.rel_l2(got.cpu().reshape(2 * m, -1), want) <= TOL, (name, m, policy)
+                outs[policy] = got
+            assert torch.equal(outs["auto"], outs["two_pass"])
+        mod.gemm_policy = "sometimes"
+        with pytest.raises(ValueError):
+            mod(x.to(dev))
+        mod.gemm_policy = "auto"
 
 
 def test_weight_data_rebinding_between_forwards(dev):
