@@ -101,7 +101,9 @@ int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N,
     const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (M <= 16) return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, y, numerics, false, s);
+    // decode-shaped work (weights streamed and decoded once): up to 16 rows always, up to 64 rows when the
+    // rows are whole 256-element runs
+    if (M <= 16 || (M <= 64 && K % 256 == 0)) return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, y, numerics, false, s);
     return sngguf::launch_gemm(x, M, q, qtype, N, K, bias, y, numerics, s);
 }
 

@@ -138,8 +138,10 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 
     // ---- LDS: two stages of (activation tile, weight tile) + one raw-weight slab per wavefront ------------
     // A tile is 256 rows of 64 bf16 (128 bytes, no padding); the eight 16-byte chunks of a row are
-    // stored at chunk ^ (row % 8), which keeps fragment reads and row-wise writes off each
-    // other's banks.
+    // stored at chunk ^ ((row / 2) % 8): two consecutive rows cover all 64 banks, so sixteen
+    // consecutive rows at one logical chunk fall into sixteen different 16-byte bank groups and both
+    // the fragment reads and the row-wise writes run without conflicts (swizzling by row % 8 leaves
+    // rows r and r + 8 on the same banks and halves the ds_read_b128 rate).
     bf16_t* xs[2] = {reinterpret_cast<bf16_t*>(lds), reinterpret_cast<bf16_t*>(lds + 2 * kTileBytes)};
     bf16_t* ws[2] = {reinterpret_cast<bf16_t*>(lds + kTileBytes), reinterpret_cast<bf16_t*>(lds + 3 * kTileBytes)};
     uint32_t* raw = reinterpret_cast<uint32_t*>(lds + 4 * kTileBytes) + wave * kRawDwords;
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     // (global_load_lds_dwordx4: lane l of a wavefront writes LDS bytes [16 l, +16) after a uniform
     // base, so one instruction fills eight consecutive 128-byte tile rows).  Instruction i of
     // wavefront w covers rows 64 i + 8 w .. + 7; the lane that fills physical chunk p of row r
-    // fetches logical chunk p ^ (r % 8), i.e. the swizzle is applied on the global side.
+    // fetches logical chunk p ^ ((r / 2) % 8), i.e. the swizzle is applied on the global side.
     // Rows past the end of the group re-read the group's last row: they only feed output rows
     // that are never stored.
     const bf16_t* xsrc[4];
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         int64_t rr = row_begin + (tid >> 3) + 64 * i;
         if (rr >= row_end) rr = row_end - 1;
         const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-        xsrc[i] = a.x + gr * a.K + 8 * ((tid & 7) ^ ((tid >> 3) & 7));
+        xsrc[i] = a.x + gr * a.K + 8 * ((tid & 7) ^ ((tid >> 4) & 7));
     }
     const int xrow0 = 8 * wave;  // first tile row this wavefront fills with instruction 0 (+ 64 i)
     // weights: wavefront w decodes elements 32 `wblk` .. + 31 (wblk = w / 4) of the K step for rows
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         goff[i] = kQ4K ? (uint32_t)((n - nb0) * row_bytes + 16 * fj) : (uint32_t)((n - nb0) * row_bytes + 32 * wblk + 12 * fj);
     }
     const uint8_t* __restrict__ wbase = q + nb0 * row_bytes;
-    const int wsw = wrow_l & 7;
+    const int wsw = (wrow_l >> 1) & 7;
     // v_perm_b32 selectors (bytes 0-3 = second operand, 4-7 = first operand)
     const uint32_t sel_q = wblk ? 0x07060504u : 0x05040302u;  // quant dword: next dword as is / 2 bytes off
     const uint32_t sel_d = wblk ? 0x03020302u : 0x01000100u;  // block scale copied into both halves
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     // fragment reads: row (lane % 32) of a 32-row tile, logical chunk 2 ks + lane / 32
     int foff[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) foff[ks] = (lane & 31) * 64 + 8 * ((2 * ks + (lane >> 5)) ^ (lane & 7));
+    for (int ks = 0; ks < 4; ks++) foff[ks] = (lane & 31) * 64 + 8 * ((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7));
 
     f32x16_t acc[4][2];  // [column tile i][row tile j]
 #pragma unroll

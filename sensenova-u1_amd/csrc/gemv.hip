@@ -251,7 +251,8 @@ int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, void* y, int numerics, bool gated, hipStream_t stream);
 
-// M in 1..16, N >= 1, K a positive multiple of the block size (checked by the caller).
+// M in 1..16 (up to 64 when K % 256 == 0 and not gated), N >= 1, K a positive multiple of the block
+// size (checked by the caller).
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                 const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
@@ -259,6 +260,10 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
     bf16_t* yp = static_cast<bf16_t*>(y);
+    if (M > 16) {
+        if (K % 256 != 0 || M > 64 || gated) return SNGGUF_E_BADSHAPE;
+        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
+    }
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
         return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
     if (qtype != SNGGUF_TYPE_Q8_0 && K % 256 == 0)

@@ -1,6 +1,8 @@
-// Decode GEMV on the matrix cores for every format but Q8_0 (1 <= M <= 16, K % 256 == 0): the
-// K-quants Q2_K .. Q6_K, one 256-element super-block per step, and the 32-element formats Q4_0,
-// Q4_1, Q5_0, Q5_1, eight blocks per step.
+// Decode GEMV on the matrix cores (K % 256 == 0): the K-quants Q2_K .. Q6_K, one 256-element
+// super-block per step, and the 32-element formats Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, eight blocks per
+// step.  Up to 16 activation rows are one matrix operand; 17 .. 64 rows use MT = 2 .. 4 operands per
+// decoded weight fragment, so the weights are still fetched and decoded once.  (Q8_0 with at most
+// 16 rows has faster kernels of its own.)
 //
 // Same shape as the Q8_0 kernel: a workgroup owns R * 16 weight rows (for the SiLU-gated pair the
 // same rows of the gate and of the up matrix, on separate wavefronts), its wavefronts split K by
@@ -100,6 +102,9 @@ template <> struct Slab<SNGGUF_TYPE_Q4_1> {  // 8 blocks of 20 bytes
 template <> struct Slab<SNGGUF_TYPE_Q5_0> {  // 8 blocks of 22 bytes
     static constexpr int ts = 176, pieces = 11, last_src = 160, stride = 176, align = 16;
 };
+template <> struct Slab<SNGGUF_TYPE_Q8_0> {  // 8 blocks of 34 bytes
+    static constexpr int ts = 272, pieces = 17, last_src = 256, stride = 272, align = 16;
+};
 template <> struct Slab<SNGGUF_TYPE_Q5_1> {  // 8 blocks of 24 bytes
     static constexpr int ts = 192, pieces = 12, last_src = 176, stride = 208, align = 16;
 };
@@ -186,6 +191,25 @@ __device__ __forceinline__ void decode_legacy(half4_t ident, const uint8_t* row,
     emit(1, legacy_block<NUM, 4 * HALF + 1, TS, HAS_MIN, FIVE>(ident, row, g));
     emit(2, legacy_block<NUM, 4 * HALF + 2, TS, HAS_MIN, FIVE>(ident, row, g));
     emit(3, legacy_block<NUM, 4 * HALF + 3, TS, HAS_MIN, FIVE>(ident, row, g));
+}
+
+// Q8_0: block b at byte 34 b of the slab row: f16 d, then 32 int8 quants (2 bytes off a dword for even b)
+template <int NUM, int B>
+__device__ __forceinline__ u32x4_t q8_0_block(const uint8_t* row, int g) {
+    const uint8_t* blk = row + B * 34;
+    const uint16_t d = *reinterpret_cast<const uint16_t*>(blk);
+    const u32x2_t qs = lds_u64<(B & 1) == 1>(blk + 2 + 8 * g);
+    uint32_t a0, a1, a2, a3;
+    q8_dword_bf16<NUM>(d, qs[0], a0, a1);
+    q8_dword_bf16<NUM>(d, qs[1], a2, a3);
+    return u32x4_t{a0, a1, a2, a3};
+}
+template <int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_q8_0(const uint8_t* row, int g, Emit&& emit) {
+    emit(0, q8_0_block<NUM, 4 * HALF + 0>(row, g));
+    emit(1, q8_0_block<NUM, 4 * HALF + 1>(row, g));
+    emit(2, q8_0_block<NUM, 4 * HALF + 2>(row, g));
+    emit(3, q8_0_block<NUM, 4 * HALF + 3>(row, g));
 }
 
 // Q2_K: element 128 h + 32 j + l is bit pair j of qs[32 h + l]; its 16-element group
@@ -332,6 +356,7 @@ __device__ __forceinline__ void decode_half(half4_t ident, const uint8_t* row, i
     else if constexpr (QT == SNGGUF_TYPE_Q4_1) decode_legacy<NUM, HALF, 20, true, false>(ident, row, g, emit);
     else if constexpr (QT == SNGGUF_TYPE_Q5_0) decode_legacy<NUM, HALF, 22, false, true>(ident, row, g, emit);
     else if constexpr (QT == SNGGUF_TYPE_Q5_1) decode_legacy<NUM, HALF, 24, true, true>(ident, row, g, emit);
+    else if constexpr (QT == SNGGUF_TYPE_Q8_0) decode_q8_0<NUM, HALF>(row, g, emit);
     else if constexpr (QT == SNGGUF_TYPE_Q2_K) decode_q2_k<NUM, HALF>(ident, row, g, emit);
     else if constexpr (QT == SNGGUF_TYPE_Q3_K) decode_q3_k<NUM, HALF>(ident, row, g, emit);
     else if constexpr (QT == SNGGUF_TYPE_Q4_K) decode_q4_k<NUM, HALF>(ident, row, g, emit);
@@ -342,7 +367,7 @@ __device__ __forceinline__ void decode_half(half4_t ident, const uint8_t* row, i
     }
 }
 
-template <int QT, int NUM, int R, bool GATED, int WMAX>
+template <int QT, int NUM, int R, bool GATED, int WMAX, int MT>
 __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
@@ -390,9 +415,11 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     const uint8_t* __restrict__ base = q + n0 * row_bytes;
     uint8_t* slab = lds + wave * kSlab;
 
-    f32x4_t acc[R];
+    f32x4_t acc[R][MT];
 #pragma unroll
-    for (int rg = 0; rg < R; rg++) acc[rg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rg = 0; rg < R; rg++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[rg][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     u32x4_t pre[kLoads];
     uint16_t pre_d = 0;
     auto fetch = [&](int s) {
@@ -404,20 +431,24 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
             if (lane < kRows) pre_d = ld_u16(p + doff);
         }
     };
-    // Lane (r, g) supplies B-operand column r.  Columns >= M are never stored, so those lanes
-    // re-read the last activation row instead of being masked.
-    const bool has_x = r < M;
-    const bf16_t* xrow = x + (int64_t)(has_x ? r : M - 1) * K + 8 * g;
+    // Lane (r, g) supplies column r of B operand t, i.e. activation row 16 t + r.  Rows >= M are never
+    // stored, so those lanes re-read the last activation row instead of being masked.
+    const bf16_t* xrow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) xrow[t] = x + (int64_t)(16 * t + r < M ? 16 * t + r : M - 1) * K + 8 * g;
 
     // Activations are buffered by half super-blocks (four fragments): `xa` holds the first half of
     // the current super-block on entry; the second half is requested into `xb` before the first is
     // used, and the first half of the next super-block into `xa` before the second is used, so each
     // request has half a step of decode work to cover its latency.
-    auto load_x = [&](int s, int half, u32x4_t (&dstx)[4]) {
+    auto load_x = [&](int s, int half, u32x4_t (&dstx)[MT][4]) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) dstx[j] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)s * 8 + 4 * half + j) * 32);
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                dstx[t][j] = *reinterpret_cast<const u32x4_t*>(xrow[t] + ((int64_t)s * 8 + 4 * half + j) * 32);
     };
-    u32x4_t xa[4], xb[4];
+    u32x4_t xa[MT][4], xb[MT][4];
     auto step = [&](int s) {
 #pragma unroll
         for (int i = 0; i < kLoads - 1; i++) *reinterpret_cast<u32x4_t*>(slab + dst[i]) = pre[i];
@@ -431,8 +462,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
         for (int rg = 0; rg < R; rg++) {
             const uint8_t* row = slab + (16 * rg + r) * S::stride;
             auto emit = [&](int jj, const u32x4_t& a) {
-                acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                                  __builtin_bit_cast(bf16x8_t, xa[jj]), acc[rg], 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                    acc[rg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xa[t][jj]), acc[rg][t], 0, 0, 0);
             };
             decode_half<QT, NUM, 0>(ident, row, g, emit);
         }
@@ -441,8 +474,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
         for (int rg = 0; rg < R; rg++) {
             const uint8_t* row = slab + (16 * rg + r) * S::stride;
             auto emit = [&](int jj, const u32x4_t& a) {
-                acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                                  __builtin_bit_cast(bf16x8_t, xb[jj]), acc[rg], 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                    acc[rg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xb[t][jj]), acc[rg][t], 0, 0, 0);
             };
             decode_half<QT, NUM, 1>(ident, row, g, emit);
         }
@@ -455,46 +490,52 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
 
     // ---- add the wavefronts' partial sums (the slabs are dead: reuse them) -------------------------
     __syncthreads();
-    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][R][64]
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][R][MT][64]
 #pragma unroll
-    for (int rg = 0; rg < R; rg++) red[(wave * R + rg) * 64 + lane] = acc[rg];
+    for (int rg = 0; rg < R; rg++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) red[((wave * R + rg) * MT + t) * 64 + lane] = acc[rg][t];
     __syncthreads();
-    if (wave != 0 || !has_x) return;
-    // D[i][j]: j = lane % 16 is the activation row, register v holds weight row 4 * (lane / 16) + v
-    const int m = r;
+    if (wave != 0) return;
+    // D[i][j]: j = lane % 16 is the activation row (of operand t), register v holds weight row 4 * (lane / 16) + v
 #pragma unroll
-    for (int rg = 0; rg < R; rg++) {
-        f32x4_t sum = red[rg * 64 + lane];
-        for (int w = 1; w < W; w++) {
-            const f32x4_t t = red[(w * R + rg) * 64 + lane];
-            sum[0] += t[0]; sum[1] += t[1]; sum[2] += t[2]; sum[3] += t[3];
-        }
-        const int64_t n = n0 + 16 * rg + 4 * g;
-        float o[4];
-        if constexpr (GATED) {
-            f32x4_t up = red[(W * R + rg) * 64 + lane];
+    for (int t = 0; t < MT; t++) {
+        const int m = 16 * t + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int rg = 0; rg < R; rg++) {
+            f32x4_t sum = red[(rg * MT + t) * 64 + lane];
             for (int w = 1; w < W; w++) {
-                const f32x4_t t = red[((W + w) * R + rg) * 64 + lane];
-                up[0] += t[0]; up[1] += t[1]; up[2] += t[2]; up[3] += t[3];
+                const f32x4_t p = red[((w * R + rg) * MT + t) * 64 + lane];
+                sum[0] += p[0]; sum[1] += p[1]; sum[2] += p[2]; sum[3] += p[3];
             }
+            const int64_t n = n0 + 16 * rg + 4 * g;
+            float o[4];
+            if constexpr (GATED) {
+                f32x4_t up = red[((W * R + rg) * MT + t) * 64 + lane];
+                for (int w = 1; w < W; w++) {
+                    const f32x4_t p = red[(((W + w) * R + rg) * MT + t) * 64 + lane];
+                    up[0] += p[0]; up[1] += p[1]; up[2] += p[2]; up[3] += p[3];
+                }
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float gt = bf16_to_f32(f32_to_bf16(sum[v]));
-                const float ut = bf16_to_f32(f32_to_bf16(up[v]));
-                const float sl = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
-                o[v] = sl * ut;
+                for (int v = 0; v < 4; v++) {
+                    const float gt = bf16_to_f32(f32_to_bf16(sum[v]));
+                    const float ut = bf16_to_f32(f32_to_bf16(up[v]));
+                    const float sl = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+                    o[v] = sl * ut;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
             }
-        } else {
+            bf16_t* yr = y + (int64_t)m * N + n;
+            if (n + 3 < N && (N & 3) == 0) {
+                *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+            } else {
 #pragma unroll
-            for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
-        }
-        bf16_t* yr = y + (int64_t)m * N + n;
-        if (n + 3 < N && (N & 3) == 0) {
-            *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
-        } else {
-#pragma unroll
-            for (int v = 0; v < 4; v++)
-                if (n + v < N) yr[v] = f32_to_bf16(o[v]);
+                for (int v = 0; v < 4; v++)
+                    if (n + v < N) yr[v] = f32_to_bf16(o[v]);
+            }
         }
     }
 }
@@ -504,6 +545,7 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
              bf16_t* y, bool gated, hipStream_t stream) {
     const int64_t groups = (N + 16 * R - 1) / (16 * R);
     const int nsb = (int)(K >> 8);
+    const int mt = (M + 15) / 16;
     // wavefronts per row group: enough that the launch fills the chip (about 12 per compute unit),
     // at least one super-block each, at most 8 per workgroup
     const int64_t per_group = gated ? 2 : 1;
@@ -514,16 +556,27 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     if (w > cap) w = cap;
     const int waves = (int)(gated ? 2 * w : w);
     const size_t slab = (size_t)waves * 16 * R * Slab<QT>::stride;
-    const size_t red = (size_t)waves * R * 64 * sizeof(f32x4_t);
+    const size_t red = (size_t)waves * R * mt * 64 * sizeof(f32x4_t);
     const size_t lds_bytes = slab > red ? slab : red;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
-#define SNGGUF_LAUNCH(G, WM) gemv_kq_mfma_kernel<QT, NUM, R, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y)
-    if (gated) {
-        if (waves <= 4) SNGGUF_LAUNCH(true, 4);
-        else SNGGUF_LAUNCH(true, 8);
+#define SNGGUF_LAUNCH(G, WM, MT_) \
+    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y)
+    if (mt > 1) {
+        // more than 16 activation rows: plain projections with one row group per wavefront only
+        if constexpr (R == 1) {
+            if (gated || mt > 4) return SNGGUF_E_BADSHAPE;
+            if (mt == 2) SNGGUF_LAUNCH(false, 8, 2);
+            else if (mt == 3) SNGGUF_LAUNCH(false, 8, 3);
+            else SNGGUF_LAUNCH(false, 8, 4);
+        } else {
+            return SNGGUF_E_BADSHAPE;
+        }
+    } else if (gated) {
+        if (waves <= 4) SNGGUF_LAUNCH(true, 4, 1);
+        else SNGGUF_LAUNCH(true, 8, 1);
     } else {
-        if (waves <= 4) SNGGUF_LAUNCH(false, 4);
-        else SNGGUF_LAUNCH(false, 8);
+        if (waves <= 4) SNGGUF_LAUNCH(false, 4, 1);
+        else SNGGUF_LAUNCH(false, 8, 1);
     }
 #undef SNGGUF_LAUNCH
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
@@ -535,13 +588,13 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
     // Two row groups per wavefront only when one per wavefront would already give far more
     // wavefronts than the chip holds (a vocabulary-sized projection): otherwise more, smaller
     // workgroups spread more evenly over the 256 compute units.
-    if (N >= 32768) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, y, gated, stream);
+    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, y, gated, stream);
     return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, y, gated, stream);
 }
 
 }  // namespace
 
-// Any format but Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned x and q (checked by the caller).
+// 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
@@ -561,6 +614,7 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
     SNGGUF_CASE(SNGGUF_TYPE_Q4_1)
     SNGGUF_CASE(SNGGUF_TYPE_Q5_0)
     SNGGUF_CASE(SNGGUF_TYPE_Q5_1)
+    SNGGUF_CASE(SNGGUF_TYPE_Q8_0)
     SNGGUF_CASE(SNGGUF_TYPE_Q2_K)
     SNGGUF_CASE(SNGGUF_TYPE_Q3_K)
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K)

@@ -31,7 +31,7 @@ def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[t
 
     ``image_gen_indicators`` is a bool tensor over the leading dims.  When the layout is known
     to be ``[text rows | image rows]`` pass ``image_gen_indicators=None`` and ``n_text`` instead:
-    no row map is built and both groups stream contiguous rows.  In that form, with more than 16
+    no row map is built and both groups stream contiguous rows.  In that form, with more than 64
     rows and unless ``proj.gemm_policy`` is ``"fused"``, each group goes through its module's
     forward (bf16 weight pass + dense GEMM, see ``GGUFLinear``) and writes its slice of the result.
     """
@@ -45,12 +45,12 @@ def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[t
             raise ValueError("give either image_gen_indicators or n_text")
         ind, split = None, int(n_text)
         x2d = hidden_states.reshape(-1, hidden_states.shape[-1])
-        if x2d.shape[0] > 16 and proj.gemm_policy != "fused" and hidden_states.dtype == torch.bfloat16:
+        if x2d.shape[0] > 64 and proj.gemm_policy != "fused" and hidden_states.dtype == torch.bfloat16:
             if not 0 <= split <= x2d.shape[0]:
                 raise ValueError(f"n_text={split} is outside 0..{x2d.shape[0]}")
             out = torch.empty((x2d.shape[0], proj.out_features), dtype=torch.bfloat16, device=hidden_states.device)
             for mod, lo, hi in ((proj, 0, split), (proj_mot_gen, split, x2d.shape[0])):
-                if hi - lo > 16:
+                if hi - lo > 64:
                     mod.two_pass_into(x2d[lo:hi], out[lo:hi])
                 elif hi > lo:
                     out[lo:hi] = mod(x2d[lo:hi])

@@ -127,12 +127,13 @@ class GGUFLinear(nn.Linear):
     """``nn.Linear`` whose weight is a :class:`GGUFParameter`.
 
     ``forward`` computes ``F.linear(x, dequantize(weight).to(compute_dtype), bias)`` with the
-    reference's rounding chain.  With bf16 activations and at most 16 rows (decode) it is one fused
-    dequant-GEMV launch.  With more rows ``gemm_policy`` decides:
+    reference's rounding chain.  With bf16 activations and at most 16 rows (decode) - at most 64 rows
+    when ``in_features`` is a multiple of 256 - it is one fused dequant-GEMV launch that streams and
+    decodes the weights once.  With more rows ``gemm_policy`` decides:
 
     * ``"two_pass"`` (what ``"auto"`` picks): one HIP dequantize launch writes the bf16 weight
       (2 * N * K bytes of transient memory) and the device's dense GEMM consumes it.  Measured on
-      MI355X this is the faster route for every M > 16: the weight pass costs about 30 us for a
+      MI355X this is the faster route from there on: the weight pass costs about 30 us for a
       12288 x 4096 matrix and the dense GEMM then runs at 1.5 PFLOP/s.
     * ``"fused"``: the fused dequant-GEMM kernels of the library (``sngguf_linear``), which need
       no transient memory.
@@ -141,7 +142,7 @@ class GGUFLinear(nn.Linear):
     """
 
     numerics: int = ops.NUM_UPSTREAM_FP16
-    gemm_policy: str = "auto"     # "auto" | "two_pass" | "fused", for inputs of more than 16 rows
+    gemm_policy: str = "auto"     # "auto" | "two_pass" | "fused", for inputs beyond the fused GEMV's row limit
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False,
                  compute_dtype: Optional[torch.dtype] = None, device=None) -> None:
@@ -161,7 +162,7 @@ class GGUFLinear(nn.Linear):
             raise RuntimeError(f"GGUFLinear: input dtype {inputs.dtype} does not match compute dtype {compute_dtype}")
         if compute_dtype == torch.bfloat16:
             rows = inputs.numel() // self.in_features if inputs.numel() else 0
-            if rows <= 16 or self.gemm_policy == "fused":
+            if rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused":
                 return ops.linear(inputs, self.weight, qtype, self.bias, self.numerics)
             if self.gemm_policy not in ("auto", "two_pass"):
                 raise ValueError(f"GGUFLinear.gemm_policy is {self.gemm_policy!r}; expected 'auto', 'two_pass' or 'fused'")

@@ -89,6 +89,25 @@ def test_gemv_32_element_formats_ragged_k(dev, c_oracle, qt, numerics):
         _check(got, c_oracle.silu_mul(g, u))
 
 
+@pytest.mark.parametrize("qt", TYPES)
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_gemv_17_to_64_rows(dev, c_oracle, qt, numerics):
+    """17 .. 64 activation rows with K % 256 == 0 stay on the decode kernel (2 .. 4 matrix operands per
+    decoded weight fragment): every operand count, partly filled last operand, ragged N, bias, one and
+    several super-blocks per wavefront."""
+    print(f"case gemv 17..64 rows qt={qt} numerics={numerics}", flush=True)
+    for n, k, m in [(192, 4096, 17), (131, 768, 32), (37, 256, 33), (64, 1024, 48), (20, 512, 49), (192, 2048, 64)]:
+        packed = synthetic.make_packed(qt, n, k, seed=n + k + m)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16)
+        got = ops.linear(x.to(dev), packed.to(dev), qt, bias.to(dev), numerics).cpu()
+        err = _check(got, go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics))
+        other = go.gguf_linear_forward(x, packed, qt, bias, numerics=1 - numerics)
+        assert err <= go.rel_l2(got, other) + 1e-6
+    rows = torch.tensor([0, 15, 16, 47, 63])
+    _check(got[rows], c_oracle.linear(x[rows], packed, qt, bias, numerics))
+
+
 def test_gemv_q8_0_odd_block_count(dev):
     """K = 32 * odd: rows are 2-byte aligned and not a whole number of 64-element units."""
     print("case gemv odd blocks", flush=True)
