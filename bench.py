@@ -219,6 +219,55 @@ def main() -> None:
                            "down_us": round(dn * 1e3, 3)}
     result["decode_other_M"] = decode
 
+    # ---- all seven linears of one decoder layer at M = 1: separate q / k / v launches against one launch over the
+    # row-wise stacked q|k|v weight (modality.FusedProjections); gate/up fused with SiLU in both ---------------------
+    if not args.no_extra:
+        nl = 6
+        attn = [(synthetic.make_packed(Q8_0, HIDDEN, HIDDEN, seed=9000 + 4 * i, device=dev),
+                 synthetic.make_packed(Q8_0, KV, HIDDEN, seed=9001 + 4 * i, device=dev),
+                 synthetic.make_packed(Q8_0, KV, HIDDEN, seed=9002 + 4 * i, device=dev),
+                 synthetic.make_packed(Q8_0, HIDDEN, HIDDEN, seed=9003 + 4 * i, device=dev)) for i in range(nl)]
+        qkv = [torch.cat(a[:3], dim=0) for a in attn]
+        x1 = synthetic.make_activations(1, HIDDEN, seed=11, device=dev)
+        yq = torch.empty((1, HIDDEN), dtype=torch.bfloat16, device=dev)
+        yk = torch.empty((1, KV), dtype=torch.bfloat16, device=dev)
+        yv = torch.empty((1, KV), dtype=torch.bfloat16, device=dev)
+        yqkv = torch.empty((1, HIDDEN + 2 * KV), dtype=torch.bfloat16, device=dev)
+        yo = torch.empty((1, HIDDEN), dtype=torch.bfloat16, device=dev)
+        h1 = torch.empty((1, INTER), dtype=torch.bfloat16, device=dev)
+
+        def layer_rest(i):
+            gate, up, down = layers[i % len(layers)]
+            ops.linear_into(yq, attn[i % nl][3], Q8_0, None, yo, num)
+            ops.gate_up_silu_into(yo, gate, up, Q8_0, h1, num)
+            ops.linear_into(h1, down, Q8_0, None, yq, num)
+
+        def layer_separate(i):
+            q, k, v, _ = attn[i % nl]
+            ops.linear_into(x1, q, Q8_0, None, yq, num)
+            ops.linear_into(x1, k, Q8_0, None, yk, num)
+            ops.linear_into(x1, v, Q8_0, None, yv, num)
+            layer_rest(i)
+
+        def layer_stacked(i):
+            ops.linear_into(x1, qkv[i % nl], Q8_0, None, yqkv, num)
+            layer_rest(i)
+
+        k3 = max(64, K // 4)
+        lbytes = (2 * linear_bytes(1, HIDDEN, HIDDEN) + 2 * linear_bytes(1, KV, HIDDEN) + mlp_bytes(1))
+        wall_a, _ = run_region(layer_separate, k3, min(W, 16))
+        wall_b, _ = run_region(layer_stacked, k3, min(W, 16))
+        result["decode_layer"] = {
+            "workload": "the 7 Q8_0 linears of one decoder layer at M=1 (q,o 4096^2; k,v 4096->1024; gate/up fused with SiLU; "
+                        "down), linears only",
+            "bytes_per_layer": lbytes,
+            "separate_qkv": {"launches": 6, "us_per_layer": round(wall_a / k3 * 1e3, 2),
+                             "value": round(lbytes / (wall_a / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"},
+            "stacked_qkv": {"launches": 4, "us_per_layer": round(wall_b / k3 * 1e3, 2),
+                            "value": round(lbytes / (wall_b / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"},
+        }
+        del attn, qkv
+
     # ---- M = 4096 generation-tower projections on the MFMA GEMM ----------------------------------
     if not args.no_gemm:
         m = 4096

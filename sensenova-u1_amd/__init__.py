@@ -1,8 +1,8 @@
 """MI355X (gfx950) GGUF quantized-linear path for SenseNova-U1: drop-in ``GGUFLinear`` module and
 GGUF loader over hand-written HIP kernels (libsngguf.so, C ABI in include/sngguf.h)."""
-from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader, GGUFWriter
+from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader, GGUFWriter, NativeGGUFReader
 from .gguf_loader import count_gguf_linear, load_gguf_checkpoint, match_state_dict, set_gguf2meta_model
-from .modality import find_mot_pairs, gated_mlp, grouped_linear
+from .modality import FusedProjections, find_mot_pairs, gated_mlp, grouped_linear
 from .quantized_linear import (
     SUPPORTED_GGUF_QUANT_TYPES,
     GGUFLinear,
@@ -14,5 +14,5 @@ __all__ = [
     "GGML_QUANT_SIZES", "GGMLQuantizationType", "GGUFReader", "GGUFWriter",
     "load_gguf_checkpoint", "set_gguf2meta_model", "match_state_dict", "count_gguf_linear",
     "GGUFLinear", "GGUFParameter", "SUPPORTED_GGUF_QUANT_TYPES", "dequantize_gguf_tensor",
-    "grouped_linear", "find_mot_pairs", "gated_mlp",
+    "grouped_linear", "find_mot_pairs", "gated_mlp", "FusedProjections", "NativeGGUFReader",
 ]

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import gguf_oracle as go
-from sensenova_u1_amd import (GGUFLinear, GGUFParameter, gated_mlp, grouped_linear, load_gguf_checkpoint,
+from sensenova_u1_amd import (FusedProjections, GGUFLinear, GGUFParameter, gated_mlp, grouped_linear, load_gguf_checkpoint,
                               set_gguf2meta_model, synthetic)
 from tests.test_loader import H, I, TinyModel, _make_file
 
@@ -110,6 +110,34 @@ def test_gemm_policies_agree_with_the_oracle(tmp_path, dev, quant):
         with pytest.raises(ValueError):
             mod(x.to(dev))
         mod.gemm_policy = "auto"
+
+
+@pytest.mark.parametrize("quant", [8, 12, 3])
+def test_fused_qkv_projections(tmp_path, dev, quant):
+    """Projections that read the same hidden states (q / k / v in the model; here the four H-input projections the
+    test model has) stacked row-wise into one launch: each output equals its own projection's oracle result, at
+    decode and above 64 rows; sources can be released afterwards."""
+    print(f"case module fused qkv quant={quant}", flush=True)
+    model, packed = _load(tmp_path, dev, quant)
+    layer = model.layers[0]
+    names = ("q_proj", "q_proj_mot_gen", "mlp.gate_proj", "mlp.up_proj")
+    fused = FusedProjections([layer.get_submodule(n) for n in names])
+    assert fused.fused.out_features == sum(layer.get_submodule(n).out_features for n in names)
+    for m in (1, 7, 16, 40, 100):
+        x = synthetic.make_activations(m, H, seed=50 + m)
+        outs = fused(x.to(dev))
+        assert len(outs) == 4
+        for n, got in zip(names, outs):
+            want = go.gguf_linear_forward(x, torch.from_numpy(packed[f"layers.0.{n}.weight"]), quant)
+            assert got.shape == (m, layer.get_submodule(n).out_features)
+            assert go.rel_l2(got.cpu(), want) <= TOL, (n, m)
+    released = FusedProjections([layer.get_submodule(n) for n in names], release_sources=True)
+    assert all(layer.get_submodule(n).weight.numel() == 0 for n in names)
+    x = synthetic.make_activations(3, H, seed=9)
+    for a, b in zip(fused(x.to(dev)), released(x.to(dev))):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        FusedProjections([model.layers[1].q_proj, model.layers[1].mlp.down_proj])    # different in_features
 
 
 def test_weight_data_rebinding_between_forwards(dev):
