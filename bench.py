@@ -236,35 +236,49 @@ def main() -> None:
         yo = torch.empty((1, HIDDEN), dtype=torch.bfloat16, device=dev)
         h1 = torch.empty((1, INTER), dtype=torch.bfloat16, device=dev)
 
-        def layer_rest(i):
+        res = synthetic.make_activations(1, HIDDEN, seed=12, device=dev)
+        hid = torch.empty((1, HIDDEN), dtype=torch.bfloat16, device=dev)
+
+        def layer_rest(i, fused_residual):
             gate, up, down = layers[i % len(layers)]
-            ops.linear_into(yq, attn[i % nl][3], Q8_0, None, yo, num)
-            ops.gate_up_silu_into(yo, gate, up, Q8_0, h1, num)
-            ops.linear_into(h1, down, Q8_0, None, yq, num)
+            if fused_residual:
+                ops.linear_residual_into(yq, attn[i % nl][3], Q8_0, None, res, hid, num)
+                ops.gate_up_silu_into(hid, gate, up, Q8_0, h1, num)
+                ops.linear_residual_into(h1, down, Q8_0, None, hid, yo, num)
+            else:
+                ops.linear_into(yq, attn[i % nl][3], Q8_0, None, yo, num)
+                torch.add(res, yo, out=hid)
+                ops.gate_up_silu_into(hid, gate, up, Q8_0, h1, num)
+                ops.linear_into(h1, down, Q8_0, None, yo, num)
+                torch.add(hid, yo, out=yq)
 
         def layer_separate(i):
             q, k, v, _ = attn[i % nl]
             ops.linear_into(x1, q, Q8_0, None, yq, num)
             ops.linear_into(x1, k, Q8_0, None, yk, num)
             ops.linear_into(x1, v, Q8_0, None, yv, num)
-            layer_rest(i)
+            layer_rest(i, False)
 
         def layer_stacked(i):
             ops.linear_into(x1, qkv[i % nl], Q8_0, None, yqkv, num)
-            layer_rest(i)
+            layer_rest(i, False)
+
+        def layer_stacked_residual(i):
+            ops.linear_into(x1, qkv[i % nl], Q8_0, None, yqkv, num)
+            layer_rest(i, True)
 
         k3 = max(64, K // 4)
         lbytes = (2 * linear_bytes(1, HIDDEN, HIDDEN) + 2 * linear_bytes(1, KV, HIDDEN) + mlp_bytes(1))
-        wall_a, _ = run_region(layer_separate, k3, min(W, 16))
-        wall_b, _ = run_region(layer_stacked, k3, min(W, 16))
+        legs = {}
+        for name, fn, launches in (("separate", layer_separate, "6 linears + 2 adds"), ("stacked_qkv", layer_stacked, "4 linears + 2 adds"),
+                                   ("stacked_qkv_fused_residual", layer_stacked_residual, "4 linears")):
+            wall_l, _ = run_region(fn, k3, min(W, 16))
+            legs[name] = {"launches": launches, "us_per_layer": round(wall_l / k3 * 1e3, 2),
+                          "value": round(lbytes / (wall_l / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"}
         result["decode_layer"] = {
             "workload": "the 7 Q8_0 linears of one decoder layer at M=1 (q,o 4096^2; k,v 4096->1024; gate/up fused with SiLU; "
-                        "down), linears only",
-            "bytes_per_layer": lbytes,
-            "separate_qkv": {"launches": 6, "us_per_layer": round(wall_a / k3 * 1e3, 2),
-                             "value": round(lbytes / (wall_a / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"},
-            "stacked_qkv": {"launches": 4, "us_per_layer": round(wall_b / k3 * 1e3, 2),
-                            "value": round(lbytes / (wall_b / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"},
+                        "down) and its two residual adds; no attention, no norms",
+            "bytes_per_layer": lbytes, **legs,
         }
         del attn, qkv
 

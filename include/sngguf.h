@@ -114,6 +114,17 @@ int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N,
                   const void* bias, void* y, int numerics, void* stream);
 
 /*
+ * residual + linear: y[M][N] = bf16(residual[M][N] + bf16(x . W^T + bias)) - the decoder layer's
+ * `hidden_states = residual + o_proj(attn)` and `residual + mlp(...)`
+ * (src/sensenova_u1/models/neo_unify/modeling_qwen3.py:934,940,973,979) with the add folded into the
+ * projection's epilogue, rounding after the projection and after the add as the two separate bf16
+ * tensor operations do.  residual: bf16 [M][N], 16-byte aligned, must not overlap y.  Everything
+ * else as sngguf_linear.
+ */
+int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
+                           const void* bias, const void* residual, void* y, int numerics, void* stream);
+
+/*
  * SiLU-gated pair for the decode MLP: h[M][N] = silu(x.Wg^T) * (x.Wu^T), with both
  * projections rounded to bf16 first, silu evaluated in fp32 on the rounded gate and rounded
  * to bf16, and the product rounded to bf16 - the rounding chain of

@@ -9,8 +9,9 @@ namespace sngguf {
 int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
                       hipStream_t stream);
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                const void* bias, void* y, int numerics, bool gated, hipStream_t stream);
-int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
+                const void* residual, void* y,
                 int numerics, hipStream_t stream);
 int64_t grouped_workspace_bytes(int64_t M);
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
@@ -96,15 +97,32 @@ int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
     return sngguf::launch_dequantize(q, qtype, rows, cols, out, out_dtype, numerics, static_cast<hipStream_t>(stream));
 }
 
-int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
-                  int numerics, void* stream) {
+namespace {
+
+int linear_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
+                const void* residual, void* y, int numerics, void* stream) {
     const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (residual && !aligned(residual, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // decode-shaped work (weights streamed and decoded once): up to 16 rows always, up to 64 rows when the
     // rows are whole 256-element runs
-    if (M <= 16 || (M <= 64 && K % 256 == 0)) return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, y, numerics, false, s);
-    return sngguf::launch_gemm(x, M, q, qtype, N, K, bias, y, numerics, s);
+    if (M <= 16 || (M <= 64 && K % 256 == 0))
+        return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, residual, y, numerics, false, s);
+    return sngguf::launch_gemm(x, M, q, qtype, N, K, bias, residual, y, numerics, s);
+}
+
+}  // namespace
+
+int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                  int numerics, void* stream) {
+    return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
+}
+
+int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
+                           const void* residual, void* y, int numerics, void* stream) {
+    if (!residual && M > 0 && N > 0) return SNGGUF_E_NULLPTR;
+    return linear_impl(x, M, q, qtype, N, K, bias, residual, y, numerics, stream);
 }
 
 int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype, int64_t N, int64_t K,
@@ -114,7 +132,7 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (!q_up) return SNGGUF_E_NULLPTR;
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
     if (M > 16) return SNGGUF_E_BADSHAPE;
-    return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+    return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
 }
 
 int64_t sngguf_grouped_workspace_bytes(int64_t M) { return sngguf::grouped_workspace_bytes(M); }

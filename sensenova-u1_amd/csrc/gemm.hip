@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const float b = (bias && n + e < a.N) ? bf16_to_f32(bias[n + e]) : 0.f;
-                    o[e] = acc[i][j][4 * vg + e] + b;
+                    o[e] = n + e < a.N ? add_residual(acc[i][j][4 * vg + e] + b, a.residual, gr * a.N + n + e) : 0.f;
                 }
                 if (n + 3 < a.N && (a.N & 3) == 0) {
                     u32x2_t pk = {pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
@@ -224,7 +224,8 @@ static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t s
 #undef SNGGUF_CALL
 }
 
-int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
+                const void* residual, void* y,
                 int numerics, hipStream_t stream) {
     GemmArgs a{};
     a.x = static_cast<const bf16_t*>(x);
@@ -233,6 +234,7 @@ int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, i
     a.rowmap = nullptr; a.n0_dev = nullptr; a.n0 = M;
     a.q[0] = a.q[1] = static_cast<const uint8_t*>(q);
     a.bias[0] = a.bias[1] = static_cast<const bf16_t*>(bias);
+    a.residual = static_cast<const bf16_t*>(residual);
     a.group_mask = 1;
     return launch_type(a, qtype, numerics, stream);
 }
@@ -250,6 +252,7 @@ int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int6
     a.q[1] = static_cast<const uint8_t*>(q_gen);
     a.bias[0] = static_cast<const bf16_t*>(bias_und);
     a.bias[1] = static_cast<const bf16_t*>(bias_gen);
+    a.residual = nullptr;
     if (indicator) {
         int32_t* ws = static_cast<int32_t*>(workspace);
         partition_rows_kernel<<<1, 1024, 0, stream>>>(indicator, M, ws);

@@ -17,6 +17,7 @@ struct GemmArgs {
     int64_t n0;
     const uint8_t* q[2];
     const bf16_t* bias[2];
+    const bf16_t* residual; // [M][N] added to the rounded projection output (same rows as y), or NULL
     int group_mask;         // bit g: rows of group g are computed by this launch
 };
 

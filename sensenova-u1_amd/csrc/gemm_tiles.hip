@@ -395,7 +395,15 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
             const int64_t rr = row_begin + ml;
             if (rr >= row_end) break;
             const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-            *reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n) = *reinterpret_cast<const u32x4_t*>(lds + ml * kYRow + 16 * (tid & 31));
+            u32x4_t o = *reinterpret_cast<const u32x4_t*>(lds + ml * kYRow + 16 * (tid & 31));
+            if (a.residual) {
+                // the staged values are the rounded projection outputs: add the residual row and round again
+                const u32x4_t rs = *reinterpret_cast<const u32x4_t*>(a.residual + gr * a.N + n);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    o[e] = pack_bf16(bf16lo_to_f32(rs[e]) + bf16lo_to_f32(o[e]), bf16hi_to_f32(rs[e]) + bf16hi_to_f32(o[e]));
+            }
+            *reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n) = o;
         }
         return;
     }
@@ -417,8 +425,11 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
                 if (rr >= row_end || n >= a.N) continue;
                 const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
                 bf16_t* yp = a.y + gr * a.N + n;
-                const float o0 = acc[i][j][4 * vg] + b[0], o1 = acc[i][j][4 * vg + 1] + b[1];
-                const float o2 = acc[i][j][4 * vg + 2] + b[2], o3 = acc[i][j][4 * vg + 3] + b[3];
+                const int64_t yi = gr * a.N + n;
+                const float o0 = add_residual(acc[i][j][4 * vg] + b[0], a.residual, yi);
+                const float o1 = n + 1 < a.N ? add_residual(acc[i][j][4 * vg + 1] + b[1], a.residual, yi + 1) : 0.f;
+                const float o2 = n + 2 < a.N ? add_residual(acc[i][j][4 * vg + 2] + b[2], a.residual, yi + 2) : 0.f;
+                const float o3 = n + 3 < a.N ? add_residual(acc[i][j][4 * vg + 3] + b[3], a.residual, yi + 3) : 0.f;
                 if (fast) {
                     *reinterpret_cast<u32x2_t*>(yp) = u32x2_t{pack_bf16(o0, o1), pack_bf16(o2, o3)};
                 } else {

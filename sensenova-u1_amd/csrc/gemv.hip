@@ -60,7 +60,7 @@ __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
 template <int QT, int NUM, int MT, bool GATED>
 __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
                                                    const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                   const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                   const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     const int lane = threadIdx.x & 63;
     const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int64_t n_pairs = GATED ? N : (N + 1) / 2;
@@ -122,10 +122,10 @@ __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x,
                     y[(int64_t)m * N + pair] = f32_to_bf16(s * up);
                 } else {
                     const float ba = bias ? bf16_to_f32(bias[na]) : 0.f;
-                    y[(int64_t)m * N + na] = f32_to_bf16(sa + ba);
+                    y[(int64_t)m * N + na] = f32_to_bf16(add_residual(sa + ba, residual, (int64_t)m * N + na));
                     if (nb != na) {
                         const float bb = bias ? bf16_to_f32(bias[nb]) : 0.f;
-                        y[(int64_t)m * N + nb] = f32_to_bf16(sb + bb);
+                        y[(int64_t)m * N + nb] = f32_to_bf16(add_residual(sb + bb, residual, (int64_t)m * N + nb));
                     }
                 }
             }
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ x,
 template <int QT, int NUM, bool GATED>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
                                                            const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                           const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                           const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     constexpr int NW = GATED ? 2 : 1;
     const int lane = threadIdx.x & 63;
     const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restr
                 const float sg = bf16_to_f32(f32_to_bf16(g / (1.0f + expf(-g))));
                 y[(int64_t)m * N + n] = f32_to_bf16(sg * up);
             } else {
-                y[(int64_t)m * N + n] = f32_to_bf16(v[0] + (bias ? bf16_to_f32(bias[n]) : 0.f));
+                y[(int64_t)m * N + n] = f32_to_bf16(add_residual(v[0] + (bias ? bf16_to_f32(bias[n]) : 0.f), residual, (int64_t)m * N + n));
             }
         }
     }
@@ -207,11 +207,11 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const bf16_t* __restr
 
 template <int QT, int NUM, bool GATED>
 static int launch_mt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                     const bf16_t* bias, bf16_t* y, hipStream_t stream) {
+                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, hipStream_t stream) {
     const int64_t n_pairs = GATED ? N : (N + 1) / 2;
     dim3 grid((unsigned)((n_pairs + 3) / 4)), block(256);
 #define SNGGUF_GEMV_CASE(MT) \
-    gemv_kernel<QT, NUM, MT, GATED><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y)
+    gemv_kernel<QT, NUM, MT, GATED><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, residual, y)
     if (M == 1) SNGGUF_GEMV_CASE(1);
     else if (M == 2) SNGGUF_GEMV_CASE(2);
     else if (M <= 4) SNGGUF_GEMV_CASE(4);
@@ -223,53 +223,54 @@ static int launch_mt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 
 template <int QT, int NUM>
 static int launch_gated(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                        const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+                        const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     if (QT != SNGGUF_TYPE_Q8_0 || K % 64 != 0) {
         dim3 grid((unsigned)((N + 3) / 4)), block(256);
-        if (gated) gemv_generic_kernel<QT, NUM, true><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y);
-        else gemv_generic_kernel<QT, NUM, false><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, y);
+        if (gated) gemv_generic_kernel<QT, NUM, true><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, residual, y);
+        else gemv_generic_kernel<QT, NUM, false><<<grid, block, 0, stream>>>(x, M, qa, qb, N, K, bias, residual, y);
         return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
     }
     if constexpr (QT == SNGGUF_TYPE_Q8_0) {
-        if (gated) return launch_mt<QT, NUM, true>(x, M, qa, qb, N, K, bias, y, stream);
-        return launch_mt<QT, NUM, false>(x, M, qa, qb, N, K, bias, y, stream);
+        if (gated) return launch_mt<QT, NUM, true>(x, M, qa, qb, N, K, bias, residual, y, stream);
+        return launch_mt<QT, NUM, false>(x, M, qa, qb, N, K, bias, residual, y, stream);
     }
     return SNGGUF_E_BADTYPE;
 }
 
 template <int QT>
 static int launch_num(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                      const bf16_t* bias, bf16_t* y, int numerics, bool gated, hipStream_t stream) {
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_gated<QT, SNGGUF_NUM_GGML_FP32>(x, M, qa, qb, N, K, bias, y, gated, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_gated<QT, SNGGUF_NUM_UPSTREAM_FP16>(x, M, qa, qb, N, K, bias, y, gated, stream);
+                      const bf16_t* bias, const bf16_t* residual, bf16_t* y, int numerics, bool gated, hipStream_t stream) {
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_gated<QT, SNGGUF_NUM_GGML_FP32>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_gated<QT, SNGGUF_NUM_UPSTREAM_FP16>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
     return SNGGUF_E_BADTYPE;
 }
 
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
-                        void* y, int numerics, bool gated, hipStream_t stream);
+                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
 
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                        const void* bias, void* y, int numerics, bool gated, hipStream_t stream);
+                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
 
 // M in 1..16 (up to 64 when K % 256 == 0 and not gated), N >= 1, K a positive multiple of the block
 // size (checked by the caller).
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
+                const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
+    const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
     if (M > 16) {
         if (K % 256 != 0 || M > 64 || gated) return SNGGUF_E_BADSHAPE;
-        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
+        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, residual, y, numerics, gated, stream);
     }
     if (qtype == SNGGUF_TYPE_Q8_0 && K % 256 == 0)
-        return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, y, numerics, gated, stream);
+        return launch_gemv_q8_mfma(x, M, qa, qb, N, K, bias, residual, y, numerics, gated, stream);
     if (qtype != SNGGUF_TYPE_Q8_0 && K % 256 == 0)
-        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, y, numerics, gated, stream);
+        return launch_gemv_kq_mfma(x, M, qa, qb, qtype, N, K, bias, residual, y, numerics, gated, stream);
     // rows that are not a whole number of 256-element runs
-#define SNGGUF_CALL(QT) launch_num<QT>(xp, (int)M, a, b, N, K, bp, yp, numerics, gated, stream)
+#define SNGGUF_CALL(QT) launch_num<QT>(xp, (int)M, a, b, N, K, bp, rp, yp, numerics, gated, stream)
     SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
 #undef SNGGUF_CALL
 }

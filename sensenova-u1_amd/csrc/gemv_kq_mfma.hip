@@ -371,7 +371,7 @@ template <int QT, int NUM, int R, bool GATED, int WMAX, int MT>
 __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                                 const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     typedef Slab<QT> S;
     constexpr int kRows = 16 * R;
     constexpr int kPieces = kRows * S::pieces;
@@ -526,7 +526,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                 }
             } else {
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
+                for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
             }
             bf16_t* yr = y + (int64_t)m * N + n;
             if (n + 3 < N && (N & 3) == 0) {
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
 
 template <int QT, int NUM, int R>
 int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-             bf16_t* y, bool gated, hipStream_t stream) {
+             const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     const int64_t groups = (N + 16 * R - 1) / (16 * R);
     const int nsb = (int)(K >> 8);
     const int mt = (M + 15) / 16;
@@ -560,7 +560,7 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     const size_t lds_bytes = slab > red ? slab : red;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
 #define SNGGUF_LAUNCH(G, WM, MT_) \
-    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y)
+    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y)
     if (mt > 1) {
         // more than 16 activation rows: plain projections with one row group per wavefront only
         if constexpr (R == 1) {
@@ -584,30 +584,31 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
 
 template <int QT, int NUM>
 int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-              bf16_t* y, bool gated, hipStream_t stream) {
+              const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     // Two row groups per wavefront only when one per wavefront would already give far more
     // wavefronts than the chip holds (a vocabulary-sized projection): otherwise more, smaller
     // workgroups spread more evenly over the 256 compute units.
-    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, y, gated, stream);
-    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, y, gated, stream);
+    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
+    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
 }
 
 }  // namespace
 
 // 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                        const void* bias, void* y, int numerics, bool gated, hipStream_t stream) {
+                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
+    const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
 #define SNGGUF_CASE(QT)                                                                                          \
     if (qtype == QT) {                                                                                           \
         if (numerics == SNGGUF_NUM_GGML_FP32)                                                                    \
-            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);          \
+            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);          \
         if (numerics == SNGGUF_NUM_UPSTREAM_FP16)                                                                \
-            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);      \
+            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);      \
         return SNGGUF_E_BADTYPE;                                                                                 \
     }
     SNGGUF_CASE(SNGGUF_TYPE_Q4_0)

@@ -26,7 +26,7 @@ template <int NUM, int CB, bool GATED, int WMAX>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                             const uint8_t* __restrict__ qa,
                                                             const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                            const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                            const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
     constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
     constexpr int kPieces = 16 * kRowPieces;      // per slab
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
         }
     } else {
 #pragma unroll
-        for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
+        for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
     }
     bf16_t* yr = y + (int64_t)m * N + n;
     if (n + 3 < N && (N & 3) == 0) {
@@ -185,7 +185,7 @@ template <int NUM, bool GATED, int WMAX, bool XLDS>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                                 const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         }
     } else {
 #pragma unroll
-        for (int v = 0; v < 4; v++) o[v] = sum[v] + ((bias && n + v < N) ? bf16_to_f32(bias[n + v]) : 0.f);
+        for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
     }
     bf16_t* yr = y + (int64_t)m * N + n;
     if (n + 3 < N && (N & 3) == 0) {
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 
 template <int NUM>
 static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                       const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+                       const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int spans = (int)(K >> 11);
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
@@ -406,7 +406,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL>), \
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
-        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y); \
+        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y); \
     } while (0)
 #define SNGGUF_LAUNCH(G, WM) \
     do { \
@@ -439,7 +439,7 @@ static int pick_k_split(int64_t groups, int steps, bool gated) {
 
 template <int NUM, int CB>
 static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                     const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int steps = (int)(K / (32 * CB));
     const int w = pick_k_split(groups, steps, gated);
@@ -447,7 +447,7 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     const size_t lds_bytes = (size_t)waves * 16 * CB * 34;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     // WMAX only sets the register budget the compiler may assume for the workgroup size
-#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, y)
+#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y)
     if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
@@ -461,26 +461,27 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 
 template <int NUM>
 static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                     const bf16_t* bias, bf16_t* y, bool gated, hipStream_t stream) {
+                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
     // The line-aligned variant needs whole 2048-element spans per wavefront; with few row groups
     // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
     // every 256 elements) is the better fit.
     const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
     if (K % 2048 == 0 && span_waves >= 2048)
-        return launch_span<NUM>(x, M, qa, qb, N, K, bias, y, gated, stream);
-    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, y, gated, stream);
+        return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
+    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
 }
 
 // Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
-                        void* y, int numerics, bool gated, hipStream_t stream) {
+                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
+    const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, yp, gated, stream);
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
     return SNGGUF_E_BADTYPE;
 }
 

@@ -44,6 +44,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// Value of one output element before its final rounding: v = accumulator + bias; with a residual
+// tensor, residual + bf16(v) - the two roundings of `residual + linear(x)` evaluated as two bf16
+// tensor operations.  idx = m * N + n; only read when `residual` is given.
+__device__ __forceinline__ float add_residual(float v, const bf16_t* residual, int64_t idx) {
+    return residual ? bf16_to_f32(residual[idx]) + bf16_to_f32(f32_to_bf16(v)) : v;
+}
+
 // Arithmetic of the block decode.  Num<SNGGUF_NUM_GGML_FP32> works in fp32, where every product
 // of the three formats is exact.  Num<SNGGUF_NUM_UPSTREAM_FP16> works in native fp16
 // (v_mul_f16 / v_sub_f16, round-to-nearest-even, subnormals and signed zeros kept): each

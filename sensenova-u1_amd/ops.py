@@ -32,7 +32,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
-    "sngguf_linear", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_linear", "sngguf_linear_residual", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -68,6 +68,8 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_dequantize.restype = ci
     lib.sngguf_linear.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, ci, vp]
     lib.sngguf_linear.restype = ci
+    lib.sngguf_linear_residual.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, ci, vp]
+    lib.sngguf_linear_residual.restype = ci
     lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu.restype = ci
     lib.sngguf_grouped_workspace_bytes.argtypes = [i64]
@@ -169,6 +171,17 @@ def linear_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: 
     _check(rc, "sngguf_linear")
 
 
+def linear_residual_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],
+                         residual2d: torch.Tensor, y2d: torch.Tensor, numerics: int) -> None:
+    """y2d[M, N] = residual2d + (x2d @ W^T + bias), rounded to bf16 after the projection and after the add."""
+    dev = x2d.device
+    n, k = y2d.shape[1], x2d.shape[1]
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_linear_residual(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
+                                                   _ptr(residual2d), _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_linear_residual")
+
+
 def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int, h2d: torch.Tensor,
                       numerics: int) -> None:
     dev = x2d.device
@@ -215,6 +228,7 @@ def _bias_bf16(bias: Optional[torch.Tensor], n: int, what: str) -> Optional[torc
 _torch_lib = torch.library.Library("sn_gguf", "DEF")
 _torch_lib.define("dequantize(Tensor packed, int quant_type, ScalarType out_dtype, int numerics) -> Tensor")
 _torch_lib.define("linear(Tensor x, Tensor packed, int quant_type, Tensor? bias, int numerics) -> Tensor")
+_torch_lib.define("linear_residual(Tensor x, Tensor packed, int quant_type, Tensor? bias, Tensor residual, int numerics) -> Tensor")
 _torch_lib.define("gate_up_silu(Tensor x, Tensor gate, Tensor up, int quant_type, int numerics) -> Tensor")
 _torch_lib.define(
     "grouped_linear(Tensor x, Tensor? indicator, int n_text, Tensor packed_und, int quant_type_und, "
@@ -236,6 +250,20 @@ def _linear_hip(x, packed, quant_type, bias, numerics):
     y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
     if y.numel():
         linear_into(x2d, p, quant_type, _bias_bf16(bias, n, "linear"), y.view(-1, n), numerics)
+    return y
+
+
+def _linear_residual_hip(x, packed, quant_type, bias, residual, numerics):
+    _require_device(x, packed, bias, residual)
+    p, n, k = _packed_2d(packed, quant_type)
+    x2d = _as_bf16_rows(x, k, "linear_residual")
+    if residual.dtype != torch.bfloat16 or tuple(residual.shape) != (*x.shape[:-1], n):
+        raise SnGgufError(f"linear_residual: residual must be bf16 of shape {(*x.shape[:-1], n)}")
+    r2d = residual.reshape(-1, n)
+    r2d = r2d if r2d.is_contiguous() else r2d.contiguous()
+    y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
+    if y.numel():
+        linear_residual_into(x2d, p, quant_type, _bias_bf16(bias, n, "linear_residual"), r2d, y.view(-1, n), numerics)
     return y
 
 
@@ -279,7 +307,8 @@ def _no_cpu(*args, **kwargs):
     raise SnGgufError("sn_gguf ops have no CPU implementation: move the tensors to the MI355X (HIP) device")
 
 
-for _name, _fn in (("dequantize", _dequantize_hip), ("linear", _linear_hip), ("gate_up_silu", _gate_up_silu_hip),
+for _name, _fn in (("dequantize", _dequantize_hip), ("linear", _linear_hip), ("linear_residual", _linear_residual_hip),
+                   ("gate_up_silu", _gate_up_silu_hip),
                    ("grouped_linear", _grouped_linear_hip)):
     _torch_lib.impl(_name, _fn, "CUDA")  # torch's dispatch key for HIP devices
     _torch_lib.impl(_name, _no_cpu, "CPU")
@@ -298,6 +327,10 @@ def _linear_meta(x, packed, quant_type, bias, numerics):
     return x.new_empty((*x.shape[:-1], packed.shape[0]), dtype=torch.bfloat16)
 
 
+def _linear_residual_meta(x, packed, quant_type, bias, residual, numerics):
+    return x.new_empty((*x.shape[:-1], packed.shape[0]), dtype=torch.bfloat16)
+
+
 def _gate_up_silu_meta(x, gate, up, quant_type, numerics):
     return x.new_empty((*x.shape[:-1], gate.shape[0]), dtype=torch.bfloat16)
 
@@ -308,6 +341,7 @@ def _grouped_linear_meta(x, indicator, n_text, packed_und, qt_und, packed_gen, q
 
 _torch_lib.impl("dequantize", _dequantize_meta, "Meta")
 _torch_lib.impl("linear", _linear_meta, "Meta")
+_torch_lib.impl("linear_residual", _linear_residual_meta, "Meta")
 _torch_lib.impl("gate_up_silu", _gate_up_silu_meta, "Meta")
 _torch_lib.impl("grouped_linear", _grouped_linear_meta, "Meta")
 
@@ -329,6 +363,12 @@ def dequantize(packed: torch.Tensor, quant_type: int, out_dtype: torch.dtype = t
 def linear(x: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor] = None,
            numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
     return torch.ops.sn_gguf.linear(x, _plain(packed), int(quant_type), _plain(bias), int(numerics))
+
+
+def linear_residual(x: torch.Tensor, packed: torch.Tensor, quant_type: int, residual: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None, numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    """``residual + linear(x)`` in one launch (bf16 rounding after the projection and after the add)."""
+    return torch.ops.sn_gguf.linear_residual(x, _plain(packed), int(quant_type), _plain(bias), residual, int(numerics))
 
 
 def gate_up_silu(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int,

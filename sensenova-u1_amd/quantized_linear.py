@@ -174,6 +174,17 @@ class GGUFLinear(nn.Linear):
         bias = self.bias.to(compute_dtype) if self.bias is not None else None
         return torch.nn.functional.linear(inputs, weight, bias)
 
+    def forward_residual(self, inputs: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        """``residual + self(inputs)`` (the decoder layer's ``hidden_states = residual + o_proj(...)`` /
+        ``residual + mlp(...)``, modeling_qwen3.py:934,940).  For bf16 inputs within the fused kernels' row
+        range the add happens in the projection's epilogue; otherwise it is the plain sum."""
+        rows = inputs.numel() // self.in_features if inputs.numel() else 0
+        fused_rows = rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused"
+        if inputs.dtype == torch.bfloat16 and (self.compute_dtype or inputs.dtype) == torch.bfloat16 and fused_rows \
+                and residual.dtype == torch.bfloat16:
+            return ops.linear_residual(inputs, self.weight, self._weight_type(), residual, self.bias, self.numerics)
+        return residual + self(inputs)
+
     def two_pass_into(self, x2d: torch.Tensor, out2d: torch.Tensor) -> None:
         """``out2d[M, N] = x2d[M, K] @ W^T (+ bias)`` for bf16 rows: one dequantize launch to a transient
         bf16 weight, then the dense GEMM writing straight into ``out2d`` (contiguous rows)."""

@@ -62,6 +62,9 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_linear(None, 1, p, 8, 4, 64, None, p, 1, None) == E_NULL
     assert lib.sngguf_linear(p, 1, p, 8, 4, 64, None, odd, 1, None) == E_ALIGN
     assert lib.sngguf_linear(p, 0, p, 8, 4, 64, None, p, 1, None) == 0
+    assert lib.sngguf_linear_residual(p, 1, p, 8, 4, 64, None, None, p, 1, None) == E_NULL   # residual is required
+    assert lib.sngguf_linear_residual(p, 1, p, 8, 4, 64, None, odd, p, 1, None) == E_ALIGN
+    assert lib.sngguf_linear_residual(p, 0, p, 8, 4, 64, None, None, p, 1, None) == 0
     assert lib.sngguf_gate_up_silu(p, 17, p, p, 8, 4, 64, p, 1, None) == E_SHAPE  # decode only
     assert lib.sngguf_linear(p, 1, p, 2, 4, 48, None, p, 1, None) == E_SHAPE    # Q4_0: K % 32
     assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL

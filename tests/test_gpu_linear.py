@@ -348,6 +348,33 @@ def test_vocabulary_sized_projection(dev, qt):
     assert torch.isfinite(y.float()).all()
 
 
+@pytest.mark.parametrize("qt", TYPES)
+def test_linear_residual(dev, qt):
+    """residual + linear in one launch equals the two bf16 tensor operations, bit for bit against the library's own
+    plain linear followed by torch's add (same kernel, same accumulation order), and within tolerance of the oracle:
+    every kernel family (decode kernels, 17..64 rows, 128- and 256-tile GEMM, ragged N, odd K)."""
+    print(f"case linear residual qt={qt}", flush=True)
+    bs = go.GGML_QUANT_SIZES[qt][0]
+    shapes = [(1, 192, 4096), (5, 37, 512), (16, 130, 768), (40, 64, 1024), (100, 131, 512), (513, 260, 256)]
+    if bs == 32:
+        shapes += [(3, 50, 96), (70, 33, 160)]
+    if qt in (go.Q8_0, go.Q4_K):
+        shapes += [(2048, 4096, 256)]
+    for m, n, k in shapes:
+        packed = synthetic.make_packed(qt, n, k, seed=m + n + k).to(dev)
+        x = synthetic.make_activations(m, k, seed=m).to(dev)
+        res = synthetic.make_activations(m, n, seed=n).to(dev)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16).to(dev)
+        for b in (None, bias):
+            got = ops.linear_residual(x, packed, qt, res, b)
+            plain = ops.linear(x, packed, qt, b)
+            assert torch.equal(got, res + plain), (m, n, k, b is not None)
+        want = res.cpu() + go.gguf_linear_forward(x.cpu(), packed.cpu(), qt, bias.cpu())
+        _check(got.cpu(), want)
+    with pytest.raises(ops.SnGgufError):
+        ops.linear_residual(x, packed, qt, res[:, :-1].contiguous())
+
+
 def test_linear_errors(dev):
     packed = synthetic.make_packed(go.Q8_0, 8, 64).to(dev)
     with pytest.raises(ops.SnGgufError):
