@@ -28,7 +28,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LDS_LD];
     __shared__ __attribute__((aligned(16))) bf16_t ws[BN * LDS_LD];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wavefront index is the same in all lanes: holding it in a scalar register keeps every address derived
+    // from it (LDS slabs, tile rows) in scalar arithmetic
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- which rows does this tile cover --------------------------------------------------
@@ -218,7 +221,9 @@ static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t s
     // everything else: the 128 x 128 kernel below
     const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
     const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0) || qtype == SNGGUF_TYPE_Q4_K;
-    if (tile_type && a.M >= 384 && big_tiles >= 128) return launch_gemm_tiles(a, qtype, numerics, stream);
+    // (the large-tile kernel addresses activations with 32-bit byte offsets)
+    const bool x_fits = a.M * a.K < ((int64_t)1 << 31);
+    if (tile_type && x_fits && a.M >= 384 && big_tiles >= 128) return launch_gemm_tiles(a, qtype, numerics, stream);
 #define SNGGUF_CALL(QT) launch_num<QT>(a, numerics, stream)
     SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
 #undef SNGGUF_CALL

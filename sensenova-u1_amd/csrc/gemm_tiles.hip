@@ -89,12 +89,23 @@ __device__ __forceinline__ void q4k_dword_bf16(uint32_t D_bits, uint32_t DM_bits
     }
 }
 
+// A pointer that is the same in all lanes, pinned to scalar registers: the loop optimiser cannot fold it into
+// per-lane 64-bit induction variables, and the request uses the scalar-base + 32-bit-offset address form.
+__device__ __forceinline__ const uint8_t* scalar_ptr(const void* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
+}
+
 template <int QT, int NUM>
 __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     constexpr bool kQ4K = QT == SNGGUF_TYPE_Q4_K;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wavefront index is the same in all lanes: holding it in a scalar register keeps every address derived
+    // from it (LDS slabs, tile rows) in scalar arithmetic
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 wavefronts: rows wm * 64, columns wn * 128
 
     // ---- tile of this workgroup ---------------------------------------------------------------------
@@ -154,13 +165,16 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     // fetches logical chunk p ^ ((r / 2) % 8), i.e. the swizzle is applied on the global side.
     // Rows past the end of the group re-read the group's last row: they only feed output rows
     // that are never stored.
-    const bf16_t* xsrc[4];
+    // Sources are kept as 32-bit byte offsets from a.x (the launcher routes problems with 2 M K >= 2^32 bytes to
+    // the 128-tile kernel): with the K-step part of the address in scalar registers a request needs no vector
+    // arithmetic.
+    uint32_t xoff[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         int64_t rr = row_begin + (tid >> 3) + 64 * i;
         if (rr >= row_end) rr = row_end - 1;
         const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-        xsrc[i] = a.x + gr * a.K + 8 * ((tid & 7) ^ ((tid >> 4) & 7));
+        xoff[i] = (uint32_t)(2 * (gr * a.K + 8 * ((tid & 7) ^ ((tid >> 4) & 7))));
     }
     const int xrow0 = 8 * wave;  // first tile row this wavefront fills with instruction 0 (+ 64 i)
     // weights: wavefront w decodes elements 32 `wblk` .. + 31 (wblk = w / 4) of the K step for rows
@@ -210,14 +224,14 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 #define SNGGUF_FETCH_W(kb, I0, I1)                                                                           \
     do {                                                                                                     \
         if constexpr (kQ4K) {                                                                                \
-            const uint8_t* ph_ = wbase + (int64_t)((kb) >> 2) * 144;                                         \
+            const uint8_t* ph_ = scalar_ptr(wbase + (int64_t)((kb) >> 2) * 144);                             \
             const uint8_t* pq_ = ph_ + 32 * ((kb) & 3);                                                      \
             _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
                 __builtin_amdgcn_global_load_lds(                                                            \
                     (const __attribute__((address_space(1))) void*)((head_piece[i_] ? ph_ : pq_) + goff[i_]),\
                     (__attribute__((address_space(3))) void*)(raw + 256 * i_), 16, 0, 0);                    \
         } else {                                                                                             \
-            const uint8_t* p_ = wbase + (int64_t)(kb) * 68;                                                  \
+            const uint8_t* p_ = scalar_ptr(wbase + (int64_t)(kb) * 68);                                      \
             _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
                 __builtin_amdgcn_global_load_lds(                                                            \
                     (const __attribute__((address_space(1))) void*)(p_ + goff[i_]),                          \
@@ -234,9 +248,10 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     } while (0)
 #define SNGGUF_LOAD_X(kb, stage, I0, I1)                                                                     \
     do {                                                                                                     \
+        const uint8_t* xb_ = scalar_ptr(a.x + (int64_t)(kb) * TK);                                           \
         _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
             __builtin_amdgcn_global_load_lds(                                                                \
-                (const __attribute__((address_space(1))) void*)(xsrc[i_] + (int64_t)(kb) * TK),              \
+                (const __attribute__((address_space(1))) void*)(xb_ + xoff[i_]),                             \
                 (__attribute__((address_space(3))) void*)(xs[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
     } while (0)
 // Scales of the 32 elements this thread decodes out of rw (the pieces of step kbn): Q8_0 the block
