@@ -380,10 +380,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     constexpr bool kQ6 = QT == SNGGUF_TYPE_Q6_K;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    // the wavefront index is the same in all lanes: holding it in a scalar register keeps every address derived
-    // from it (LDS slabs, tile rows) in scalar arithmetic
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
     const int W = GATED ? waves >> 1 : waves;  // wavefronts that share one row group's K
     const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;

@@ -34,10 +34,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
     constexpr int kSlab = 16 * kRowStep;          // LDS bytes per wavefront (4352 or 8704)
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    // the wavefront index is the same in all lanes: holding it in a scalar register keeps every address derived
-    // from it (LDS slabs, tile rows) in scalar arithmetic
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
     const int W = GATED ? waves >> 1 : waves;     // wavefronts that share one row group's K
     const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
@@ -190,10 +187,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    // the wavefront index is the same in all lanes: holding it in a scalar register keeps every address derived
-    // from it (LDS slabs, tile rows) in scalar arithmetic
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
     const int W = GATED ? waves >> 1 : waves;
     const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
