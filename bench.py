@@ -463,6 +463,92 @@ def main() -> None:
         }
         del und, gen, xs, ys, wtmp
 
+    # ---- layer-offload streaming: decoder layers (understanding tower, 7 Q8_0 linears, 205 MB) kept in pinned
+    # host arenas and copied in ahead of their forward on a second stream; the host link bounds this leg ----------
+    if not args.no_extra:
+        from torch import nn
+
+        from sensenova_u1_amd import GGUFLinear, GGUFParameter, gated_mlp
+        from sensenova_u1_amd.layer_offload import ALL_TENSOR_GROUPS, LayerOffloadWrapper
+
+        def qlin(n, k, seed):
+            lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16)
+            lin.weight = GGUFParameter(synthetic.make_packed(Q8_0, n, k, seed=seed, device=dev).cpu(), quant_type=Q8_0)
+            return lin
+
+        class StreamLayer(nn.Module):
+            def __init__(self, s):
+                super().__init__()
+                self.q_proj, self.o_proj = qlin(HIDDEN, HIDDEN, s), qlin(HIDDEN, HIDDEN, s + 1)
+                self.k_proj, self.v_proj = qlin(KV, HIDDEN, s + 2), qlin(KV, HIDDEN, s + 3)
+                self.gate_proj, self.up_proj = qlin(INTER, HIDDEN, s + 4), qlin(INTER, HIDDEN, s + 5)
+                self.down_proj = qlin(HIDDEN, INTER, s + 6)
+
+            def forward(self, h):
+                q = self.q_proj(h)
+                self.k_proj(h)
+                self.v_proj(h)
+                h = h + self.o_proj(q)
+                return h + gated_mlp(h, self.gate_proj, self.up_proj, self.down_proj)
+
+        class StreamModel(nn.Module):
+            def __init__(self, n):
+                super().__init__()
+                self.layers = nn.ModuleList([StreamLayer(8000 + 10 * i) for i in range(n)])
+
+            def forward(self, h):
+                for layer in self.layers:
+                    h = layer(h)
+                return h
+
+        n_sl, passes = 6, 3
+        model = StreamModel(n_sl).eval()
+        layer_bytes = sum(p.numel() for p in model.layers[0].parameters())
+        hs = {m: synthetic.make_activations(m, HIDDEN, seed=13, device=dev) for m in (1, 4096)}
+
+        def timed_passes(fn, h):
+            fn(h)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(passes):
+                fn(h)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / (passes * n_sl) * 1e3
+
+        model.to(dev)
+        stream = {f"M{m}": {"resident_ms_per_layer": round(timed_passes(model, h), 3)} for m, h in hs.items()}
+        model.to("cpu")
+        for prefetch in (0, 2):
+            wrapped = LayerOffloadWrapper(model, "layers", dev, prefetch_count=prefetch)
+            for m, h in hs.items():
+                ms = timed_passes(wrapped, h)
+                stream[f"M{m}"][f"prefetch_{prefetch}"] = {"ms_per_layer": round(ms, 3),
+                                                           "host_link_GBps": round(layer_bytes / ms / 1e6, 2)}
+            if prefetch == 0:
+                store = wrapped.store
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(passes):
+                    for i in range(n_sl):
+                        store.move_to_gpu(i, groups=ALL_TENSOR_GROUPS, non_blocking=True)
+                        store.evict_to_cpu(i)
+                e1.record()
+                torch.cuda.synchronize()
+                copy_ms = e0.elapsed_time(e1) / (passes * n_sl)
+                slots = sum(store.slots_allocated().values())
+            wrapped.teardown()
+        result["offload_stream"] = {
+            "workload": f"{n_sl} decoder layers (7 Q8_0 linears each, {layer_bytes} packed bytes per layer) held in pinned host "
+                        "arenas, one copy per layer into a ring of device slots, forward of the 7 linears per layer at M=1 and "
+                        "M=4096; time per layer over whole passes, wall clock; prefetch_0 copies on the compute stream, "
+                        "prefetch_2 two layers ahead on a second stream",
+            "bytes_per_layer": layer_bytes,
+            "copy_only": {"ms_per_layer": round(copy_ms, 3), "GBps": round(layer_bytes / copy_ms / 1e6, 2), "device_slots": slots},
+            **stream,
+        }
+        del model
+
     # ---- CPU baseline: the oracle's port of GGUFLinear.forward_native on the host cores -----------
     if not args.no_cpu_baseline:
         from oracle import gguf_oracle as go

@@ -2,6 +2,7 @@
 GGUF loader over hand-written HIP kernels (libsngguf.so, C ABI in include/sngguf.h)."""
 from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader, GGUFWriter, NativeGGUFReader
 from .gguf_loader import count_gguf_linear, load_gguf_checkpoint, match_state_dict, set_gguf2meta_model
+from .layer_offload import AsyncPrefetcher, LayerOffloadWrapper, PackedLayerStore
 from .modality import FusedProjections, find_mot_pairs, gated_mlp, grouped_linear
 from .quantized_linear import (
     SUPPORTED_GGUF_QUANT_TYPES,
@@ -15,4 +16,5 @@ __all__ = [
     "load_gguf_checkpoint", "set_gguf2meta_model", "match_state_dict", "count_gguf_linear",
     "GGUFLinear", "GGUFParameter", "SUPPORTED_GGUF_QUANT_TYPES", "dequantize_gguf_tensor",
     "grouped_linear", "find_mot_pairs", "gated_mlp", "FusedProjections", "NativeGGUFReader",
+    "LayerOffloadWrapper", "PackedLayerStore", "AsyncPrefetcher",
 ]
