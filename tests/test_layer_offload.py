@@ -92,7 +92,8 @@ def test_store_packs_each_group_into_one_arena_and_keeps_values_types_and_tags()
     a = layers[0].self_attn.q_proj.weight.data
     b = layers[0].mlp.up_proj.weight.data
     assert a.untyped_storage().data_ptr() == b.untyped_storage().data_ptr()
-    assert a.data_ptr() % 256 == 0 and b.data_ptr() % 256 == 0 and layers[0].norm.bias.data_ptr() % 256 == 0
+    base = a.untyped_storage().data_ptr()   # page-aligned when pinned or on the device
+    assert all((t.data_ptr() - base) % 256 == 0 for t in (a, b, layers[0].norm.bias.data))
     assert a.untyped_storage().data_ptr() != layers[0].self_attn.q_proj_mot_gen.weight.data.untyped_storage().data_ptr()
     assert store.group_nbytes(0, GROUP_UNDERSTANDING) == H * (H // 32 * 34) + I * (H // 32 * 34) + 2 * H * 4
     assert store.group_nbytes(0, GROUP_SHARED) == 12
