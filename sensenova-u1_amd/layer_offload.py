@@ -115,12 +115,18 @@ class PackedLayerStore:
         self._bytes_moved = 0
         self._bytes_moved_by_group = {g: 0 for g in ALL_TENSOR_GROUPS}
         self._copies = 0
+        # A tensor that several layers share cannot follow one layer in and out: it is left unmanaged, which
+        # the wrapper treats like everything outside the layer list (resident on the device).
+        seen: dict[int, int] = {}
+        for layer in layers:
+            for _name, t in itertools.chain(layer.named_parameters(), layer.named_buffers()):
+                seen[id(t)] = seen.get(id(t), 0) + 1
         for layer in layers:
             groups = partition_layer_tensor_names(layer)
             by_group: dict[str, list[tuple[str, torch.Tensor]]] = {}
             for name, t in itertools.chain(layer.named_parameters(), layer.named_buffers()):
-                if id(t) in self._managed:
-                    continue  # shared with an earlier layer: lives in that layer's arena
+                if seen[id(t)] > 1:
+                    continue
                 self._managed.add(id(t))
                 by_group.setdefault(groups.get(name, GROUP_SHARED), []).append((name, t))
             arenas = {g: _Arena(ts, pin_memory) for g, ts in by_group.items()}
@@ -213,7 +219,10 @@ class PackedLayerStore:
         return set(self._managed)
 
     def cleanup(self) -> None:
-        """Evict everything and drop the device ring.  Tensors keep their pinned arena views."""
+        """Evict everything and drop the device ring (after the device has finished with it).  Tensors keep
+        their pinned arena views."""
+        if self.target_device.type == "cuda":
+            torch.cuda.synchronize(self.target_device)
         for idx in range(self.num_layers):
             self.evict_to_cpu(idx)
         for g in self._free:

@@ -140,14 +140,17 @@ def test_store_moves_only_the_requested_groups_and_reuses_slots():
         store.is_on_gpu(3)
 
 
-def test_tensors_shared_between_layers_are_packed_once():
+def test_tensors_shared_between_layers_are_left_to_the_caller():
     a, b = TwoTowerLayer(0), TwoTowerLayer(1)
     b.norm.weight = a.norm.weight
     layers = nn.ModuleList([a, b])
     store = PackedLayerStore(layers, torch.device("cpu"), pin_memory=False)
-    assert len(store.managed_tensor_ids()) == 17
+    ids = store.managed_tensor_ids()
+    assert len(ids) == 16 and id(a.norm.weight) not in ids
+    ptr = a.norm.weight.data_ptr()
     store.move_to_gpu(1, b)
-    assert b.norm.weight is a.norm.weight
+    store.evict_to_cpu(1, b)
+    assert b.norm.weight is a.norm.weight and a.norm.weight.data_ptr() == ptr
 
 
 def test_wrapper_argument_checks():
