@@ -282,6 +282,21 @@ def main() -> None:
         }
         del attn, qkv
 
+    # ---- lm_head at decode: 151936 x 4096 Q8_0 (the vocabulary projection of the think loop), M = 1 ---------------
+    if not args.no_extra:
+        vocab = 151936
+        heads = [synthetic.make_packed(Q8_0, vocab, HIDDEN, seed=9500 + i, device=dev) for i in range(2)]
+        xh = synthetic.make_activations(1, HIDDEN, seed=14, device=dev)
+        logits = torch.empty((1, vocab), dtype=torch.bfloat16, device=dev)
+        n_h = 32
+        _, ev_h = run_region(lambda i: ops.linear_into(xh, heads[i % 2], Q8_0, None, logits, num), n_h, 4)
+        hb = linear_bytes(1, vocab, HIDDEN)
+        result["lm_head"] = {"workload": "Q8_0 lm_head 4096 -> 151936 at M=1, two weight copies alternating",
+                             "bytes_per_launch": hb, "avg_launch_us": round(ev_h / n_h * 1e3, 2),
+                             "value": round(hb / (ev_h / n_h * 1e-3) / 1e9, 1), "unit": "GB/s",
+                             "pct_of_hbm_peak": round(100 * hb / (ev_h / n_h * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        del heads, logits
+
     # ---- M = 4096 generation-tower projections on the MFMA GEMM ----------------------------------
     if not args.no_gemm:
         m = 4096
