@@ -137,12 +137,17 @@ class GGUFLinear(nn.Linear):
       12288 x 4096 matrix and the dense GEMM then runs at 1.5 PFLOP/s.
     * ``"fused"``: the fused dequant-GEMM kernels of the library (``sngguf_linear``), which need
       no transient memory.
+    * ``"resident"``: as ``"two_pass"``, but the bf16 weight is kept (2 * N * K bytes per module) and
+      reused by later calls until the packed bytes move or change: for towers that see thousands of
+      rows many times over (the denoising loop) on a device with memory to spare, it removes the
+      weight pass from every call but the first.  Not meant to be combined with layer offloading.
 
     Other compute dtypes always take dequantize + matmul.
     """
 
     numerics: int = ops.NUM_UPSTREAM_FP16
-    gemm_policy: str = "auto"     # "auto" | "two_pass" | "fused", for inputs beyond the fused GEMV's row limit
+    gemm_policy: str = "auto"     # "auto" | "two_pass" | "fused" | "resident", for inputs beyond the fused GEMV's row limit
+    _dense_cache = None           # (key, bf16 weight) of the "resident" policy
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False,
                  compute_dtype: Optional[torch.dtype] = None, device=None) -> None:
@@ -164,8 +169,8 @@ class GGUFLinear(nn.Linear):
             rows = inputs.numel() // self.in_features if inputs.numel() else 0
             if rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused":
                 return ops.linear(inputs, self.weight, qtype, self.bias, self.numerics)
-            if self.gemm_policy not in ("auto", "two_pass"):
-                raise ValueError(f"GGUFLinear.gemm_policy is {self.gemm_policy!r}; expected 'auto', 'two_pass' or 'fused'")
+            if self.gemm_policy not in ("auto", "two_pass", "resident"):
+                raise ValueError(f"GGUFLinear.gemm_policy is {self.gemm_policy!r}; expected 'auto', 'two_pass', 'fused' or 'resident'")
             out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
             self.two_pass_into(inputs.reshape(-1, self.in_features), out.view(-1, self.out_features))
             return out
@@ -189,11 +194,21 @@ class GGUFLinear(nn.Linear):
         """``out2d[M, N] = x2d[M, K] @ W^T (+ bias)`` for bf16 rows: one dequantize launch to a transient
         bf16 weight, then the dense GEMM writing straight into ``out2d`` (contiguous rows)."""
         # the bf16 the kernel writes is the fp16 chain rounded once more, i.e. `.to(bfloat16)` of the fp16 tensor
-        weight = ops.dequantize(self.weight, self._weight_type(), torch.bfloat16, self.numerics)
+        if self.gemm_policy == "resident":
+            key = (self.weight.data_ptr(), self.weight._version, self._weight_type(), self.numerics)
+            if self._dense_cache is None or self._dense_cache[0] != key:
+                self._dense_cache = (key, ops.dequantize(self.weight, self._weight_type(), torch.bfloat16, self.numerics))
+            weight = self._dense_cache[1]
+        else:
+            weight = ops.dequantize(self.weight, self._weight_type(), torch.bfloat16, self.numerics)
         if self.bias is None:
             torch.matmul(x2d, weight.t(), out=out2d)
         else:
             torch.addmm(self.bias.to(torch.bfloat16), x2d, weight.t(), out=out2d)
+
+    def drop_dense_cache(self) -> None:
+        """Release the bf16 weight the "resident" policy keeps."""
+        self._dense_cache = None
 
     def extra_repr(self) -> str:
         qt = getattr(self.weight, "quant_type", None)

@@ -99,17 +99,40 @@ def test_gemm_policies_agree_with_the_oracle(tmp_path, dev, quant):
             want = go.gguf_linear_forward(x, torch.from_numpy(packed[name + ".weight"]), quant,
                                           mod.bias.cpu() if mod.bias is not None else None)
             outs = {}
-            for policy in ("auto", "two_pass", "fused"):
+            for policy in ("auto", "two_pass", "fused", "resident"):
                 mod.gemm_policy = policy
                 got = mod(x.to(dev).reshape(2, m, -1))
                 assert got.shape == (2, m, mod.out_features) and got.dtype == torch.bfloat16
                 assert go.rel_l2(got.cpu().reshape(2 * m, -1), want) <= TOL, (name, m, policy)
                 outs[policy] = got
-            assert torch.equal(outs["auto"], outs["two_pass"])
+            assert torch.equal(outs["auto"], outs["two_pass"]) and torch.equal(outs["auto"], outs["resident"])
         mod.gemm_policy = "sometimes"
         with pytest.raises(ValueError):
             mod(x.to(dev))
         mod.gemm_policy = "auto"
+
+
+def test_resident_policy_keeps_the_bf16_weight_until_the_packed_bytes_change(tmp_path, dev):
+    print("case module resident policy", flush=True)
+    model, packed = _load(tmp_path, dev, 8)
+    mod = model.get_submodule("layers.0.mlp.down_proj")
+    other = model.get_submodule("layers.1.mlp.down_proj")
+    mod.gemm_policy = "resident"
+    x = synthetic.make_activations(200, mod.in_features, seed=9).to(dev)
+    y0 = mod(x)
+    kept = mod._dense_cache[1]
+    assert kept.dtype == torch.bfloat16 and kept.shape == (mod.out_features, mod.in_features)
+    assert torch.equal(mod(x), y0) and mod._dense_cache[1] is kept          # second call: no new weight pass
+    assert torch.equal(mod(x[:3]), y0[:3])                                  # decode rows do not touch the kept weight
+    old = mod.weight.data
+    mod.weight.data = other.weight.data.clone()                             # the offloader's kind of rebinding
+    other.gemm_policy = "two_pass"
+    assert torch.equal(mod(x), other(x)) and mod._dense_cache[1] is not kept
+    mod.weight.data = old
+    mod.weight.data.copy_(other.weight.data)                                # in-place change at the same address
+    assert torch.equal(mod(x), other(x))
+    mod.drop_dense_cache()
+    assert mod._dense_cache is None
 
 
 @pytest.mark.parametrize("quant", [8, 12, 3])
