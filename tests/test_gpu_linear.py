@@ -312,7 +312,7 @@ def test_grouped_linear_contiguous_split_with_bias(dev, c_oracle):
 
 
 def test_full_size_shapes_row_sample(dev):
-    """BASELINE shapes at full size; a sample of output rows / columns is checked against the
+    """The 8B backbone's projection shapes at full size; a sample of output rows / columns is checked against the
     oracle run on exactly those weight rows (an output element depends on one x row and one
     weight row only)."""
     print("case full size", flush=True)
