@@ -10,6 +10,8 @@ int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
                       hipStream_t stream);
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                 const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
+                      hipStream_t stream);
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
                 const void* residual, void* y,
                 int numerics, hipStream_t stream);
@@ -123,6 +125,24 @@ int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, i
                            const void* residual, void* y, int numerics, void* stream) {
     if (!residual && M > 0 && N > 0) return SNGGUF_E_NULLPTR;
     return linear_impl(x, M, q, qtype, N, K, bias, residual, y, numerics, stream);
+}
+
+int64_t sngguf_linear_workspace_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 && N < kMaxDim && K < kMaxDim ? 2 * N * K : 0; }
+
+int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                     void* workspace, int64_t workspace_bytes, int numerics, void* stream) {
+    const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // The weight pass pays once the matrix work dwarfs it; the dense kernel wants whole K steps, 32-bit activation
+    // offsets and enough 256 x 256 tiles to occupy the chip.  Everything else runs as sngguf_linear does.
+    const bool two_pass = workspace && workspace_bytes >= 2 * N * K && M >= 384 && K % 64 == 0 &&
+                          M * K < ((int64_t)1 << 31) && ((M + 255) / 256) * ((N + 255) / 256) >= 128;
+    if (!two_pass) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
+    const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
+    if (rd != SNGGUF_OK) return rd;
+    return sngguf::launch_gemm_dense(x, M, workspace, N, K, bias, y, s);
 }
 
 int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype, int64_t N, int64_t K,

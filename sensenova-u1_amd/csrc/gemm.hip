@@ -244,6 +244,22 @@ int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, i
     return launch_type(a, qtype, numerics, stream);
 }
 
+// y = x w^T (+ bias) with w already bf16 [N][K]: the tile kernel without its decode stage.
+// Needs K % 64 == 0 and M K < 2^31 (checked by the caller).
+int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
+                      hipStream_t stream) {
+    GemmArgs a{};
+    a.x = static_cast<const bf16_t*>(x);
+    a.y = static_cast<bf16_t*>(y);
+    a.M = M; a.N = N; a.K = K;
+    a.rowmap = nullptr; a.n0_dev = nullptr; a.n0 = M;
+    a.q[0] = a.q[1] = static_cast<const uint8_t*>(w);
+    a.bias[0] = a.bias[1] = static_cast<const bf16_t*>(bias);
+    a.residual = nullptr;
+    a.group_mask = 1;
+    return launch_gemm_tiles(a, 30, SNGGUF_NUM_GGML_FP32, stream);
+}
+
 int64_t grouped_workspace_bytes(int64_t M) { return 16 + 4 * (M > 0 ? M : 0); }
 
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,

@@ -1,4 +1,5 @@
-// Dequant-GEMM, large-tile variant for Q8_0 (K % 64 == 0) and Q4_K: 256 x 256 output tile per
+// Dequant-GEMM, large-tile variant for Q8_0 (K % 64 == 0) and Q4_K - and, as the second pass of the
+// workspace route, for weights already decoded to bf16: 256 x 256 output tile per
 // workgroup, K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32,
 // 128 accumulator registers each, two wavefronts per SIMD - and two LDS stages.
 //
@@ -45,6 +46,7 @@ constexpr int TK = 64;       // K step
 constexpr int kTileBytes = 256 * 64 * 2;          // one operand tile in LDS (rows of 128 bytes, swizzled)
 constexpr int kRawDwords = 64 * 12;               // raw slab of one wavefront: 64 rows x 3 pieces of 16 bytes
 constexpr int kLdsBytes = 4 * kTileBytes + 8 * kRawDwords * 4;  // two stages of both tiles + raw slabs
+constexpr int kTypeBF16 = 30;                     // ggml's id for plain bf16 rows: weights that need no decode
 
 // Q4_K: (D, DM) = (d * sc, dmin * mn) of sub-block j from the super-block head, as the bit pattern
 // the decode uses: NUM 1 the fp16 product copied into both halves of a dword, NUM 0 the fp32 product.
@@ -100,6 +102,7 @@ __device__ __forceinline__ const uint8_t* scalar_ptr(const void* p) {
 template <int QT, int NUM>
 __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     constexpr bool kQ4K = QT == SNGGUF_TYPE_Q4_K;
+    constexpr bool kDense = QT == kTypeBF16;  // weights already bf16 [N][K]: both operand tiles are plain copies
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     const uint8_t* __restrict__ q = a.q[g];
     const bf16_t* __restrict__ bias = a.bias[g];
     const int64_t nb0 = tn * TN;
-    const int64_t row_bytes = kQ4K ? (a.K >> 8) * 144 : (a.K >> 5) * 34;
+    const int64_t row_bytes = kDense ? 2 * a.K : kQ4K ? (a.K >> 8) * 144 : (a.K >> 5) * 34;
     const int ksteps = (int)(a.K / TK);
 
     // ---- LDS: two stages of (activation tile, weight tile) + one raw-weight slab per wavefront ------------
@@ -177,6 +180,16 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         xoff[i] = (uint32_t)(2 * (gr * a.K + 8 * ((tid & 7) ^ ((tid >> 4) & 7))));
     }
     const int xrow0 = 8 * wave;  // first tile row this wavefront fills with instruction 0 (+ 64 i)
+    // dense weights: the weight tile is filled the same way, from rows nb0 .. nb0 + 255 of q
+    uint32_t woff[4] = {0, 0, 0, 0};
+    if constexpr (kDense) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int64_t n = (tid >> 3) + 64 * i;                 // row of the tile
+            if (nb0 + n >= a.N) n = a.N - 1 - nb0;           // rows past the end re-read the last row
+            woff[i] = (uint32_t)(2 * (n * a.K + 8 * ((tid & 7) ^ ((tid >> 4) & 7))));
+        }
+    }
     // weights: wavefront w decodes elements 32 `wblk` .. + 31 (wblk = w / 4) of the K step for rows
     // 64 (w % 4) .. + 63, one row per lane.  The bytes it needs are fetched as three pieces per row,
     // consecutive lanes walking along a row (3 lanes per row), into the wavefront's raw slab and
@@ -253,6 +266,14 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
             __builtin_amdgcn_global_load_lds(                                                                \
                 (const __attribute__((address_space(1))) void*)(xb_ + xoff[i_]),                             \
                 (__attribute__((address_space(3))) void*)(xs[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
+    } while (0)
+#define SNGGUF_LOAD_WD(kb, stage, I0, I1)                                                                    \
+    do {                                                                                                     \
+        const uint8_t* wb_ = scalar_ptr(wbase + (int64_t)(kb) * (2 * TK));                                   \
+        _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
+            __builtin_amdgcn_global_load_lds(                                                                \
+                (const __attribute__((address_space(1))) void*)(wb_ + woff[i_]),                             \
+                (__attribute__((address_space(3))) void*)(ws[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
     } while (0)
 // Scales of the 32 elements this thread decodes out of rw (the pieces of step kbn): Q8_0 the block
 // scale copied into both halves of sc_a (first block of a pair: low half of dword 0, second: high
@@ -333,6 +354,76 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         __syncthreads();                                                                                     \
     } while (0)
 
+// Dense weights (plain bf16 rows): the same tile loop without the decode stage.  The workgroup's one barrier per
+// step sits in front of the LAST 16-wide slice: by then every wavefront holds the fragments of that slice in
+// registers, so stage CUR is free, and the copies into the other stage - requested a whole step earlier, behind
+// the previous barrier - have had a step's worth of matrix work to arrive.  The copies of step kb + 2 go into stage
+// CUR behind the barrier, half of them at once, half in the first slice of the next step.
+#define SNGGUF_INTERLEAVE_DENSE()                                            \
+    do {                                                                     \
+        _Pragma("unroll") for (int m_ = 0; m_ < 8; m_++) {                   \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               \
+            if (m_ < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   \
+        }                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                   \
+    } while (0)
+#define SNGGUF_K_STEP_DENSE(kb, CUR, NEXT, FETCH)                                                            \
+    do {                                                                                                     \
+        const bf16_t* a_base_ = ws[CUR] + wn * 128 * 64;                                                     \
+        const bf16_t* b_base_ = xs[CUR] + wm * 64 * 64;                                                      \
+        bf16x8_t af_[2][4], bf_[2][2];                                                                       \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                        \
+            af_[0][i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[0]);                 \
+        _Pragma("unroll") for (int j = 0; j < 2; j++)                                                        \
+            bf_[0][j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[0]);                 \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
+            if (ks < 3) {                                                                                    \
+                _Pragma("unroll") for (int i = 0; i < 4; i++)                                                \
+                    af_[(ks + 1) & 1][i] =                                                                   \
+                        *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[(ks + 1) & 3]);      \
+                _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
+                    bf_[(ks + 1) & 1][j] =                                                                   \
+                        *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[(ks + 1) & 3]);      \
+            }                                                                                                \
+            if (ks == 0 && (NEXT)) {                                                                         \
+                SNGGUF_LOAD_WD((kb) + 1, (CUR) ^ 1, 2, 4);                                                   \
+                SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 2, 4);                                                    \
+            }                                                                                                \
+            if (ks == 3) {                                                                                   \
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                  \
+                __syncthreads();                                                                             \
+                if (FETCH) {                                                                                 \
+                    SNGGUF_LOAD_WD((kb) + 2, CUR, 0, 2);                                                     \
+                    SNGGUF_LOAD_X((kb) + 2, CUR, 0, 2);                                                      \
+                }                                                                                            \
+            }                                                                                                \
+            _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
+                _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[ks & 1][i], bf_[ks & 1][j],      \
+                                                                        acc[i][j], 0, 0, 0);                 \
+            SNGGUF_INTERLEAVE_DENSE();                                                                       \
+        }                                                                                                    \
+    } while (0)
+
+    if constexpr (kDense) {
+        SNGGUF_LOAD_X(0, 0, 0, 4);
+        SNGGUF_LOAD_WD(0, 0, 0, 4);
+        if (ksteps > 1) {
+            SNGGUF_LOAD_X(1, 1, 0, 2);
+            SNGGUF_LOAD_WD(1, 1, 0, 2);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        int kd = 0;
+        for (; kd + 3 < ksteps; kd += 2) {
+            SNGGUF_K_STEP_DENSE(kd, 0, true, true);
+            SNGGUF_K_STEP_DENSE(kd + 1, 1, true, true);
+        }
+        for (; kd < ksteps; kd += 2) {
+            SNGGUF_K_STEP_DENSE(kd, 0, kd + 1 < ksteps, kd + 2 < ksteps);
+            if (kd + 1 < ksteps) SNGGUF_K_STEP_DENSE(kd + 1, 1, kd + 2 < ksteps, kd + 3 < ksteps);
+        }
+    } else {
     // ---- prologue: stage 0 holds K step 0, the raw slab step 1 ------------------------------------------------
     SNGGUF_LOAD_X(0, 0, 0, 4);
     SNGGUF_FETCH_W(0, 0, 3);
@@ -365,7 +456,11 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
             SNGGUF_K_STEP(kb + 1, 1, next, fetch);
         }
     }
+    }  // quantized weights
 #undef SNGGUF_K_STEP
+#undef SNGGUF_K_STEP_DENSE
+#undef SNGGUF_INTERLEAVE_DENSE
+#undef SNGGUF_LOAD_WD
 #undef SNGGUF_INTERLEAVE
 #undef SNGGUF_DECODE_W
 #undef SNGGUF_SCALES_W
@@ -472,13 +567,15 @@ int launch_tiles(const GemmArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-// Q8_0 with K % 64 == 0 (rows are then 4-byte aligned) or Q4_K; both row groups of that type.
+// Q8_0 with K % 64 == 0 (rows are then 4-byte aligned), Q4_K, or type 30 = weights that are already bf16 rows
+// (K % 64 == 0; the numerics mode plays no role); both row groups of that type.
 int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
 #define SNGGUF_CASE(QT, NUM) if (qtype == QT && numerics == NUM) return launch_tiles<QT, NUM>(a, stream)
     SNGGUF_CASE(SNGGUF_TYPE_Q8_0, SNGGUF_NUM_GGML_FP32);
     SNGGUF_CASE(SNGGUF_TYPE_Q8_0, SNGGUF_NUM_UPSTREAM_FP16);
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_GGML_FP32);
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_UPSTREAM_FP16);
+    if (qtype == kTypeBF16) return launch_tiles<kTypeBF16, SNGGUF_NUM_GGML_FP32>(a, stream);
 #undef SNGGUF_CASE
     return SNGGUF_E_BADTYPE;
 }

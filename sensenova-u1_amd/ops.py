@@ -32,7 +32,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
-    "sngguf_linear", "sngguf_linear_residual", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -70,6 +70,10 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear.restype = ci
     lib.sngguf_linear_residual.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, ci, vp]
     lib.sngguf_linear_residual.restype = ci
+    lib.sngguf_linear_workspace_bytes.argtypes = [i64, i64]
+    lib.sngguf_linear_workspace_bytes.restype = i64
+    lib.sngguf_linear_ws.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, i64, ci, vp]
+    lib.sngguf_linear_ws.restype = ci
     lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu.restype = ci
     lib.sngguf_grouped_workspace_bytes.argtypes = [i64]
@@ -169,6 +173,24 @@ def linear_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: 
         rc = load_library().sngguf_linear(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
                                           _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_linear")
+
+
+def linear_workspace_bytes(n: int, k: int) -> int:
+    """Bytes of workspace with which ``linear_ws_into`` can take the weight-pass route (2 * n * k)."""
+    return int(load_library().sngguf_linear_workspace_bytes(n, k))
+
+
+def linear_ws_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],
+                   y2d: torch.Tensor, workspace: Optional[torch.Tensor], numerics: int) -> None:
+    """As ``linear_into``; with a device ``workspace`` of at least ``linear_workspace_bytes(N, K)`` bytes large
+    problems run as one weight pass into the workspace (bf16) and the library's dense tile GEMM."""
+    dev = x2d.device
+    n, k = y2d.shape[1], x2d.shape[1]
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_linear_ws(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
+                                             _ptr(y2d), _ptr(workspace), ws_bytes, numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_linear_ws")
 
 
 def linear_residual_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],

@@ -65,6 +65,10 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_linear_residual(p, 1, p, 8, 4, 64, None, None, p, 1, None) == E_NULL   # residual is required
     assert lib.sngguf_linear_residual(p, 1, p, 8, 4, 64, None, odd, p, 1, None) == E_ALIGN
     assert lib.sngguf_linear_residual(p, 0, p, 8, 4, 64, None, None, p, 1, None) == 0
+    assert lib.sngguf_linear_workspace_bytes(12288, 4096) == 2 * 12288 * 4096 and lib.sngguf_linear_workspace_bytes(0, 5) == 0
+    assert lib.sngguf_linear_ws(p, 1, p, 8, 4, 48, None, p, None, 0, 1, None) == E_SHAPE      # same checks as sngguf_linear
+    assert lib.sngguf_linear_ws(p, 1, p, 8, 4, 64, None, p, odd, 64, 1, None) == E_ALIGN       # workspace alignment
+    assert lib.sngguf_linear_ws(p, 0, p, 8, 4, 64, None, p, None, 0, 1, None) == 0
     assert lib.sngguf_gate_up_silu(p, 17, p, p, 8, 4, 64, p, 1, None) == E_SHAPE  # decode only
     assert lib.sngguf_linear(p, 1, p, 2, 4, 48, None, p, 1, None) == E_SHAPE    # Q4_0: K % 32
     assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL

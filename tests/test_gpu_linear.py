@@ -193,6 +193,39 @@ def test_gemm_q8_0_large_tile_kernel(dev, c_oracle, numerics):
     _check(got[rows], sub)
 
 
+@pytest.mark.parametrize("qt", TYPES)
+def test_linear_with_workspace(dev, qt):
+    """sngguf_linear_ws: with a large enough workspace big problems go through the weight pass + the dense tile
+    kernel (every type; ragged M / N, bias, one K step and many, odd and even step counts, blocked and plain tile
+    order); with no or too small a workspace, or a problem below the thresholds, it is sngguf_linear."""
+    print(f"case linear_ws qt={qt}", flush=True)
+    bs = go.GGML_QUANT_SIZES[qt][0]
+    for numerics, (m, n, k) in [(1, (3072, 2816, 256)), (0, (3000, 2904, 768)), (1, (2048, 4096, 512)), (1, (8300, 1030, 256))]:
+        packed = synthetic.make_packed(qt, n, k, seed=m + n + k + qt)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16)
+        want = go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics)
+        xd, pd, bd = x.to(dev), packed.to(dev), bias.to(dev)
+        ws = torch.full((ops.linear_workspace_bytes(n, k) // 2,), float("nan"), dtype=torch.bfloat16, device=dev)
+        y = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        ops.linear_ws_into(xd, pd, qt, bd, y, ws, numerics)
+        _check(y.cpu(), want)
+        # the workspace now holds the decoded weight: bit-identical to the standalone dequantize
+        assert torch.equal(ws.view(n, k), ops.dequantize(pd, qt, torch.bfloat16, numerics))
+        fused = ops.linear(xd, pd, qt, bd, numerics)
+        for small in (None, ws[:n * k - 8]):
+            y2 = torch.empty_like(y)
+            ops.linear_ws_into(xd, pd, qt, bd, y2, small, numerics)
+            assert torch.equal(y2, fused)
+    # below the thresholds (few rows): the fused path although a workspace is there
+    x = synthetic.make_activations(40, k, seed=4).to(dev)
+    y3 = torch.empty((40, n), dtype=torch.bfloat16, device=dev)
+    ws.fill_(float("nan"))
+    ops.linear_ws_into(x, pd, qt, None, y3, ws, 1)
+    assert torch.equal(y3, ops.linear(x, pd, qt, None, 1)) and bool(torch.isnan(ws.float()).all())
+    assert bs in (32, 256)
+
+
 @pytest.mark.parametrize("numerics", [0, 1])
 def test_gemm_q4_k_large_tile_kernel(dev, c_oracle, numerics):
     """Q4_K through the 256 x 256 tile kernel (M >= 384, at least 128 tiles): every chunk position of
