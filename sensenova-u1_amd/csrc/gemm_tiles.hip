@@ -358,7 +358,9 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 // step sits in front of the LAST 16-wide slice: by then every wavefront holds the fragments of that slice in
 // registers, so stage CUR is free, and the copies into the other stage - requested a whole step earlier, behind
 // the previous barrier - have had a step's worth of matrix work to arrive.  The copies of step kb + 2 go into stage
-// CUR behind the barrier, half of them at once, half in the first slice of the next step.
+// CUR behind the barrier, half of them at once, half in the first slice of the next step; the fragments of the next
+// step's first slice are read there too (its stage has just been declared complete), so a step starts with its
+// operands in registers.
 #define SNGGUF_INTERLEAVE_DENSE()                                            \
     do {                                                                     \
         _Pragma("unroll") for (int m_ = 0; m_ < 8; m_++) {                   \
@@ -367,24 +369,19 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         }                                                                    \
         __builtin_amdgcn_sched_barrier(0);                                   \
     } while (0)
+#define SNGGUF_FRAGS_DENSE(stage, ks_, buf)                                                                  \
+    do {                                                                                                     \
+        const bf16_t* a_base_ = ws[stage] + wn * 128 * 64;                                                   \
+        const bf16_t* b_base_ = xs[stage] + wm * 64 * 64;                                                    \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                        \
+            daf_[buf][i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[ks_]);            \
+        _Pragma("unroll") for (int j = 0; j < 2; j++)                                                        \
+            dbf_[buf][j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[ks_]);            \
+    } while (0)
 #define SNGGUF_K_STEP_DENSE(kb, CUR, NEXT, FETCH)                                                            \
     do {                                                                                                     \
-        const bf16_t* a_base_ = ws[CUR] + wn * 128 * 64;                                                     \
-        const bf16_t* b_base_ = xs[CUR] + wm * 64 * 64;                                                      \
-        bf16x8_t af_[2][4], bf_[2][2];                                                                       \
-        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                        \
-            af_[0][i] = *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[0]);                 \
-        _Pragma("unroll") for (int j = 0; j < 2; j++)                                                        \
-            bf_[0][j] = *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[0]);                 \
         _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
-            if (ks < 3) {                                                                                    \
-                _Pragma("unroll") for (int i = 0; i < 4; i++)                                                \
-                    af_[(ks + 1) & 1][i] =                                                                   \
-                        *reinterpret_cast<const bf16x8_t*>(a_base_ + i * 32 * 64 + foff[(ks + 1) & 3]);      \
-                _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
-                    bf_[(ks + 1) & 1][j] =                                                                   \
-                        *reinterpret_cast<const bf16x8_t*>(b_base_ + j * 32 * 64 + foff[(ks + 1) & 3]);      \
-            }                                                                                                \
+            if (ks < 3) SNGGUF_FRAGS_DENSE(CUR, ks + 1, (ks + 1) & 1);                                       \
             if (ks == 0 && (NEXT)) {                                                                         \
                 SNGGUF_LOAD_WD((kb) + 1, (CUR) ^ 1, 2, 4);                                                   \
                 SNGGUF_LOAD_X((kb) + 1, (CUR) ^ 1, 2, 4);                                                    \
@@ -392,6 +389,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
             if (ks == 3) {                                                                                   \
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                  \
                 __syncthreads();                                                                             \
+                if (NEXT) SNGGUF_FRAGS_DENSE((CUR) ^ 1, 0, 0);                                               \
                 if (FETCH) {                                                                                 \
                     SNGGUF_LOAD_WD((kb) + 2, CUR, 0, 2);                                                     \
                     SNGGUF_LOAD_X((kb) + 2, CUR, 0, 2);                                                      \
@@ -399,13 +397,14 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
             }                                                                                                \
             _Pragma("unroll") for (int i = 0; i < 4; i++)                                                    \
                 _Pragma("unroll") for (int j = 0; j < 2; j++)                                                \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[ks & 1][i], bf_[ks & 1][j],      \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(daf_[ks & 1][i], dbf_[ks & 1][j],    \
                                                                         acc[i][j], 0, 0, 0);                 \
             SNGGUF_INTERLEAVE_DENSE();                                                                       \
         }                                                                                                    \
     } while (0)
 
     if constexpr (kDense) {
+        bf16x8_t daf_[2][4], dbf_[2][2];
         SNGGUF_LOAD_X(0, 0, 0, 4);
         SNGGUF_LOAD_WD(0, 0, 0, 4);
         if (ksteps > 1) {
@@ -414,6 +413,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        SNGGUF_FRAGS_DENSE(0, 0, 0);
         int kd = 0;
         for (; kd + 3 < ksteps; kd += 2) {
             SNGGUF_K_STEP_DENSE(kd, 0, true, true);
@@ -459,6 +459,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     }  // quantized weights
 #undef SNGGUF_K_STEP
 #undef SNGGUF_K_STEP_DENSE
+#undef SNGGUF_FRAGS_DENSE
 #undef SNGGUF_INTERLEAVE_DENSE
 #undef SNGGUF_LOAD_WD
 #undef SNGGUF_INTERLEAVE
