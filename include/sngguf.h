@@ -173,6 +173,20 @@ int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, in
                           void* y, void* workspace, int numerics, void* stream);
 
 /*
+ * sngguf_grouped_linear with the weight-pass route of sngguf_linear_ws (no counterpart in the reference either):
+ * with dense_workspace (device memory, 16-byte aligned) of at least 2 * sngguf_linear_workspace_bytes(N, K) =
+ * 4 N K bytes and a problem that fits that route (same conditions as sngguf_linear_ws) both weight sets are
+ * decoded into it once as bf16 and ONE dense tile-GEMM launch serves both row groups - whatever the two quant
+ * types are.  Otherwise it is sngguf_grouped_linear.  workspace is the row-map scratch of
+ * sngguf_grouped_linear (needed with an indicator).  Never allocates.
+ */
+int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text,
+                             const void* q_und, int qtype_und, const void* q_gen, int qtype_gen,
+                             int64_t N, int64_t K, const void* bias_und, const void* bias_gen, void* y,
+                             void* workspace, void* dense_workspace, int64_t dense_workspace_bytes,
+                             int numerics, void* stream);
+
+/*
  * ---- GGUF container reader (host only, no GPU call) -----------------------------------
  * What the reference gets from gguf.GGUFReader at
  * src/sensenova_u1/utils/gguf_loader.py:29-44: open the file, walk `reader.tensors`, read each

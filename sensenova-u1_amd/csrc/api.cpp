@@ -127,6 +127,14 @@ int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, i
     return linear_impl(x, M, q, qtype, N, K, bias, residual, y, numerics, stream);
 }
 
+namespace {
+// The weight pass pays once the matrix work dwarfs it; the dense kernel wants whole K steps, 32-bit activation
+// offsets and enough 256 x 256 tiles to occupy the chip.
+bool dense_route_fits(int64_t M, int64_t N, int64_t K) {
+    return M >= 384 && K % 64 == 0 && M * K < ((int64_t)1 << 31) && ((M + 255) / 256) * ((N + 255) / 256) >= 128;
+}
+}  // namespace
+
 int64_t sngguf_linear_workspace_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 && N < kMaxDim && K < kMaxDim ? 2 * N * K : 0; }
 
 int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
@@ -135,10 +143,8 @@ int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // The weight pass pays once the matrix work dwarfs it; the dense kernel wants whole K steps, 32-bit activation
-    // offsets and enough 256 x 256 tiles to occupy the chip.  Everything else runs as sngguf_linear does.
-    const bool two_pass = workspace && workspace_bytes >= 2 * N * K && M >= 384 && K % 64 == 0 &&
-                          M * K < ((int64_t)1 << 31) && ((M + 255) / 256) * ((N + 255) / 256) >= 128;
+    // everything that does not fit the dense route runs as sngguf_linear does
+    const bool two_pass = workspace && workspace_bytes >= 2 * N * K && dense_route_fits(M, N, K);
     if (!two_pass) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
     if (rd != SNGGUF_OK) return rd;
@@ -172,6 +178,36 @@ int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, in
     }
     return sngguf::launch_grouped_gemm(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und,
                                        bias_gen, y, workspace, numerics, static_cast<hipStream_t>(stream));
+}
+
+int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
+                             int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
+                             const void* bias_gen, void* y, void* workspace, void* dense_workspace,
+                             int64_t dense_workspace_bytes, int numerics, void* stream) {
+    const bool two_pass = dense_workspace && dense_workspace_bytes >= 4 * N * K && K > 0 && N > 0 && dense_route_fits(M, N, K);
+    if (!two_pass)
+        return sngguf_grouped_linear(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und, bias_gen, y,
+                                     workspace, numerics, stream);
+    int rc = check_matmul(x, M, q_und, qtype_und, N, K, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    rc = check_matmul(x, M, q_gen, qtype_gen, N, K, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    if (!aligned(dense_workspace, 16)) return SNGGUF_E_ALIGN;
+    if (indicator) {
+        if (!workspace) return SNGGUF_E_NULLPTR;
+        if (!aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+    } else if (n_text < 0 || n_text > M) {
+        return SNGGUF_E_BADSHAPE;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint8_t* w_und = static_cast<uint8_t*>(dense_workspace);
+    uint8_t* w_gen = w_und + 2 * N * K;
+    rc = sngguf::launch_dequantize(q_und, qtype_und, N, K, w_und, SNGGUF_OUT_BF16, numerics, s);
+    if (rc != SNGGUF_OK) return rc;
+    rc = sngguf::launch_dequantize(q_gen, qtype_gen, N, K, w_gen, SNGGUF_OUT_BF16, numerics, s);
+    if (rc != SNGGUF_OK) return rc;
+    return sngguf::launch_grouped_gemm(x, M, indicator, n_text, w_und, 30, w_gen, 30, N, K, bias_und, bias_gen, y, workspace,
+                                       numerics, s);
 }
 
 }  // extern "C"

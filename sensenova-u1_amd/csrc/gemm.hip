@@ -219,6 +219,7 @@ int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t st
 static int launch_type(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
     // Q8_0 / Q4_K problems with enough 256 x 256 tiles to occupy the chip: the large-tile kernel;
     // everything else: the 128 x 128 kernel below
+    if (qtype == 30) return launch_gemm_tiles(a, 30, numerics, stream);  // weights already bf16 (workspace routes)
     const int64_t big_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
     const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 && a.K % 64 == 0) || qtype == SNGGUF_TYPE_Q4_K;
     // (the large-tile kernel addresses activations with 32-bit byte offsets)

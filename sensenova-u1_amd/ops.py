@@ -33,6 +33,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
     "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_grouped_linear_ws",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -80,6 +81,8 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_grouped_workspace_bytes.restype = i64
     lib.sngguf_grouped_linear.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, ci, vp]
     lib.sngguf_grouped_linear.restype = ci
+    lib.sngguf_grouped_linear_ws.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, vp, i64, ci, vp]
+    lib.sngguf_grouped_linear_ws.restype = ci
     # host-only GGUF container reader
     cp = ctypes.c_char_p
     lib.sngguf_file_open.argtypes = [cp, ctypes.POINTER(vp), cp, i64]
@@ -175,6 +178,11 @@ def linear_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: 
     _check(rc, "sngguf_linear")
 
 
+def grouped_workspace_bytes(m: int) -> int:
+    """Bytes of row-map scratch the grouped launcher needs for ``m`` rows when it is given an indicator."""
+    return int(load_library().sngguf_grouped_workspace_bytes(m))
+
+
 def linear_workspace_bytes(n: int, k: int) -> int:
     """Bytes of workspace with which ``linear_ws_into`` can take the weight-pass route (2 * n * k)."""
     return int(load_library().sngguf_linear_workspace_bytes(n, k))
@@ -223,6 +231,20 @@ def grouped_linear_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, 
             y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), numerics,
             ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_grouped_linear")
+
+
+def grouped_linear_ws_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, y2d,
+                           workspace, dense_workspace, numerics) -> None:
+    """As ``grouped_linear_into``; with a device ``dense_workspace`` of at least ``2 * linear_workspace_bytes(N, K)``
+    bytes large problems decode both weight sets once and run one dense tile-GEMM launch over both row groups."""
+    dev = x2d.device
+    dw_bytes = dense_workspace.numel() * dense_workspace.element_size() if dense_workspace is not None else 0
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_grouped_linear_ws(
+            _ptr(x2d), x2d.shape[0], _ptr(indicator), n_text, _ptr(packed_und), qt_und, _ptr(packed_gen), qt_gen,
+            y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), _ptr(dense_workspace),
+            dw_bytes, numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_grouped_linear_ws")
 
 
 def _as_bf16_rows(x: torch.Tensor, k: int, what: str) -> torch.Tensor:
@@ -319,7 +341,7 @@ def _grouped_linear_hip(x, indicator, n_text, packed_und, qt_und, packed_gen, qt
             raise SnGgufError(f"grouped_linear: indicator has {indicator.numel()} entries for {m} rows")
         ind = indicator.detach().reshape(-1)
         ind = (ind != 0).to(torch.uint8) if ind.dtype != torch.uint8 else ind.contiguous()
-        ws = torch.empty(load_library().sngguf_grouped_workspace_bytes(m), dtype=torch.uint8, device=x.device)
+        ws = torch.empty(grouped_workspace_bytes(m), dtype=torch.uint8, device=x.device)
     grouped_linear_into(x2d, ind, n_text, pu, qt_und, pg, qt_gen, _bias_bf16(bias_und, n, "grouped_linear"),
                         _bias_bf16(bias_gen, n, "grouped_linear"), y.view(-1, n), ws, numerics)
     return y

@@ -74,3 +74,7 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL
     assert lib.sngguf_grouped_linear(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_NULL  # no workspace
     assert lib.sngguf_grouped_linear(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_SHAPE  # n_text > M
+    # without a dense workspace the _ws form is the plain one, with the same checks
+    assert lib.sngguf_grouped_linear_ws(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_SHAPE
+    assert lib.sngguf_grouped_linear_ws(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_NULL
+    assert lib.sngguf_grouped_linear_ws(p, 0, None, 0, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == 0

@@ -268,6 +268,48 @@ def _grouped_large_tiles(dev, m, n, k):
     assert torch.equal(got[~split], yu[~split]) and torch.equal(got[split], yg[split])
 
 
+@pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q6_K), (go.Q5_0, go.Q3_K)])
+def test_grouped_linear_with_dense_workspace(dev, qt_pair):
+    """sngguf_grouped_linear_ws: both weight sets decoded once into the workspace, one dense launch over both row
+    groups - equal quant types or not, with an indicator (row map) and with the contiguous split, biases; and the
+    plain grouped launcher when the workspace is missing or too small."""
+    qu, qg = qt_pair
+    print(f"case grouped_ws {qu} {qg}", flush=True)
+    m, n, k = 3100, 2904, 512
+    und = synthetic.make_packed(qu, n, k, seed=51)
+    gen = synthetic.make_packed(qg, n, k, seed=52)
+    x = synthetic.make_activations(m, k, seed=53)
+    g = torch.Generator().manual_seed(54)
+    ind = torch.rand(m, generator=g) < 0.6
+    bu = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16)
+    bg = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16)
+    want = torch.empty((m, n), dtype=torch.bfloat16)
+    want[~ind] = go.gguf_linear_forward(x[~ind], und, qu, bu)
+    want[ind] = go.gguf_linear_forward(x[ind], gen, qg, bg)
+    xd, ud, gd, bud, bgd = x.to(dev), und.to(dev), gen.to(dev), bu.to(dev), bg.to(dev)
+    indd = ind.to(torch.uint8).to(dev)
+    ws = torch.empty(ops.grouped_workspace_bytes(m), dtype=torch.uint8, device=dev)
+    dw = torch.empty(2 * ops.linear_workspace_bytes(n, k) // 2, dtype=torch.bfloat16, device=dev)
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.grouped_linear_ws_into(xd, indd, 0, ud, qu, gd, qg, bud, bgd, y, ws, dw, 1)
+    _check(y.cpu(), want)
+    assert torch.equal(dw[:n * k].view(n, k), ops.dequantize(ud, qu, torch.bfloat16, 1))
+    assert torch.equal(dw[n * k:].view(n, k), ops.dequantize(gd, qg, torch.bfloat16, 1))
+    # contiguous [text | image] layout, no row map
+    n_text = 1300
+    want2 = torch.cat([go.gguf_linear_forward(x[:n_text], und, qu, bu), go.gguf_linear_forward(x[n_text:], gen, qg, bg)])
+    y2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.grouped_linear_ws_into(xd, None, n_text, ud, qu, gd, qg, bud, bgd, y2, None, dw, 1)
+    _check(y2.cpu(), want2)
+    # no / short dense workspace: the plain grouped launcher
+    plain = torch.empty_like(y)
+    ops.grouped_linear_into(xd, indd, 0, ud, qu, gd, qg, bud, bgd, plain, ws, 1)
+    for short in (None, dw[:2 * n * k - 8]):
+        y3 = torch.empty_like(y)
+        ops.grouped_linear_ws_into(xd, indd, 0, ud, qu, gd, qg, bud, bgd, y3, ws, short, 1)
+        assert torch.equal(y3, plain)
+
+
 def test_gemm_q8_0_odd_block_count(dev):
     print("case gemm odd blocks", flush=True)
     packed = synthetic.make_packed(go.Q8_0, 70, 96, seed=1)
