@@ -177,21 +177,29 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
 // step, line 16 for the last step - always has the lines a step needs in the ring and only
 // overwrites lines whose blocks are done.  A block that runs over the end of the ring is read
 // with wrapped addresses.
+// Rows from which the gated pair runs in the paired mode of the span kernel: measured 12288 x 4096 gate/up,
+// unpaired / paired us: M=2 26.8 / 30.7, M=4 27.4 / 30.8, M=8 28.2 / 29.7, M=16 34.5 / 30.2.
+constexpr int kPairedMinM = 12;
 constexpr int kRing = 512;        // ring bytes per row
 constexpr int kRingRow = 528;     // LDS bytes per row: 132 dwords, rows fall on distinct banks
 constexpr int kSpanBytes = 2176;  // 64 blocks = 17 lines
 
-template <int NUM, bool GATED, int WMAX, bool XLDS>
+// PAIRED (gated only): one wavefront works on the gate AND the up matrix of its K range, so that each activation
+// fragment is fetched once for both - with several activation rows those fetches, not the weights, fill the
+// vector memory path (16 rows x 64 bytes per matrix instruction against 544 bytes of weights).
+template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
+    constexpr int NQ = PAIRED ? 2 : 1;   // matrices per wavefront
     const int waves = blockDim.x >> 6;
-    const int W = GATED ? waves >> 1 : waves;
-    const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
-    const uint8_t* __restrict__ q = (GATED && wave >= W) ? qb : qa;
+    const int W = (GATED && !PAIRED) ? waves >> 1 : waves;
+    const int kw = (GATED && !PAIRED) ? (wave >= W ? wave - W : wave) : wave;
+    const uint8_t* __restrict__ q = (GATED && !PAIRED && wave >= W) ? qb : qa;
     const int r = lane & 15, g = lane >> 4;
     const int64_t row_bytes = (K >> 5) * 34;
     const int64_t n0 = (int64_t)blockIdx.x * 16;
@@ -214,7 +222,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         goff1[i] = (uint32_t)((n - n0) * row_bytes + 2048 + 16 * (lane & 7));
     }
     const uint8_t* __restrict__ base = q + n0 * row_bytes;
-    uint8_t* slab = lds + wave * (16 * kRingRow);
+    const uint8_t* __restrict__ base2 = qb + n0 * row_bytes;           // PAIRED: the second matrix
+    constexpr int kSlab = 16 * kRingRow;
+    uint8_t* slab = lds + wave * (NQ * kSlab);                         // PAIRED: two rings per wavefront
     uint8_t* lw2 = slab + (lane >> 4) * kRingRow + 16 * (lane & 15);  // + 4 i rows, + 256 for odd groups
     uint8_t* lw1 = slab + (lane >> 3) * kRingRow + 16 * (lane & 7);   // + 8 i rows (line 16 -> ring slot 0)
     const uint8_t* lr = slab + r * kRingRow;                           // this lane's weight row
@@ -227,22 +237,29 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     // workgroup and the B fragments come from there; otherwise they are fetched from global
     // memory one step ahead.
     const int64_t xs_stride = 2 * K + 64;   // bytes per activation row in LDS (+64: rows on different banks)
-    uint8_t* xs = lds + waves * (16 * kRingRow);
+    uint8_t* xs = lds + waves * (NQ * kSlab);
     const uint8_t* xsrow = xs + (has_x ? r : M - 1) * xs_stride + 16 * g;
 
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    u32x4_t pa[4], pb[4];     // fetched lines on their way to the ring
-    u32x4_t xa[8], xb[8];     // activation fragments of the current / next step (global path)
+    f32x4_t acc[NQ];
+#pragma unroll
+    for (int h = 0; h < NQ; h++) acc[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    u32x4_t pa[NQ][4], pb[NQ][4];   // fetched lines on their way to the ring(s)
+    u32x4_t xa[8], xb[8];           // activation fragments of the current / next step (global path)
 
-    auto fetch2 = [&](int t, int grp, u32x4_t (&dst)[4]) {
-        const uint8_t* p = base + (int64_t)t * kSpanBytes + 256 * grp;
+    auto fetch2 = [&](int t, int grp, u32x4_t (&dst)[NQ][4]) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = *reinterpret_cast<const u32x4_t*>(p + goff2[i]);
+        for (int h = 0; h < NQ; h++) {
+            const uint8_t* p = (h ? base2 : base) + (int64_t)t * kSpanBytes + 256 * grp;
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[h][i] = *reinterpret_cast<const u32x4_t*>(p + goff2[i]);
+        }
     };
-    auto store2 = [&](int grp, const u32x4_t (&src)[4]) {
+    auto store2 = [&](int grp, const u32x4_t (&src)[NQ][4]) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            *reinterpret_cast<u32x4_t*>(lw2 + 4 * i * kRingRow + ((grp & 1) << 8)) = src[i];
+        for (int h = 0; h < NQ; h++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                *reinterpret_cast<u32x4_t*>(lw2 + h * kSlab + 4 * i * kRingRow + ((grp & 1) << 8)) = src[h][i];
     };
     auto fetch_x = [&](int t, int s, u32x4_t (&dst)[8]) {
         if constexpr (!XLDS) {
@@ -282,7 +299,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                 store2(s + 1, pa);
             } else {
 #pragma unroll
-                for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4_t*>(lw1 + 8 * i * kRingRow) = pa[i];
+                for (int h = 0; h < NQ; h++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4_t*>(lw1 + h * kSlab + 8 * i * kRingRow) = pa[h][i];
             }
             // -- requests for the next step: activations first, so that waiting for them does not
             //    also wait for the weight lines
@@ -292,8 +311,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                     fetch2(t, s + 2, pa);
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
-                        pa[i] = *reinterpret_cast<const u32x4_t*>(base + (int64_t)t * kSpanBytes + goff1[i]);
+                    for (int h = 0; h < NQ; h++)
+#pragma unroll
+                        for (int i = 0; i < 2; i++)
+                            pa[h][i] = *reinterpret_cast<const u32x4_t*>((h ? base2 : base) + (int64_t)t * kSpanBytes + goff1[i]);
                 }
             } else if (t + 1 < t1) {
                 fetch_x(t + 1, 0, xn);
@@ -307,43 +328,48 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                 const int ro = (34 * b) & (kRing - 1);    // ring offset of the block (compile-time)
                 const int qo = (b & 1) ? ro + 2 : ro;     // first 4-byte aligned dword this lane reads, before + 8 g
                 const int nd = (b & 1) ? 2 : 3;           // dwords read
-                const uint16_t d = *reinterpret_cast<const uint16_t*>(lr + ro);
-                uint32_t w[3];
-                if (qo + 24 + 4 * nd <= kRing) {
-                    const uint32_t* src = reinterpret_cast<const uint32_t*>(lr + qo + 8 * g);
-#pragma unroll
-                    for (int k = 0; k < 3; k++)
-                        if (k < nd) w[k] = src[k];
-                } else {  // the block runs over the end of the ring
-#pragma unroll
-                    for (int k = 0; k < 3; k++)
-                        if (k < nd) w[k] = *reinterpret_cast<const uint32_t*>(lr + ((qo + 8 * g + 4 * k) & (kRing - 1)));
-                }
-                uint32_t q0, q1;
-                if (b & 1) {
-                    q0 = w[0];
-                    q1 = w[1];
-                } else {  // quants start 2 bytes into the first dword
-                    q0 = __builtin_amdgcn_alignbit(w[1], w[0], 16);
-                    q1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
-                }
-                uint32_t a0, a1, a2, a3;
-                q8_dword_bf16<NUM>(d, q0, a0, a1);
-                q8_dword_bf16<NUM>(d, q1, a2, a3);
-                const u32x4_t a = {a0, a1, a2, a3};
                 u32x4_t xfrag;
                 if constexpr (XLDS) xfrag = *reinterpret_cast<const u32x4_t*>(xsrow + ((int64_t)t * 64 + b) * 64);
                 else xfrag = xc[bb];
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                              __builtin_bit_cast(bf16x8_t, xfrag), acc, 0, 0, 0);
+#pragma unroll
+                for (int h = 0; h < NQ; h++) {
+                    const uint8_t* lrh = lr + h * kSlab;
+                    const uint16_t d = *reinterpret_cast<const uint16_t*>(lrh + ro);
+                    uint32_t w[3];
+                    if (qo + 24 + 4 * nd <= kRing) {
+                        const uint32_t* src = reinterpret_cast<const uint32_t*>(lrh + qo + 8 * g);
+#pragma unroll
+                        for (int k = 0; k < 3; k++)
+                            if (k < nd) w[k] = src[k];
+                    } else {  // the block runs over the end of the ring
+#pragma unroll
+                        for (int k = 0; k < 3; k++)
+                            if (k < nd) w[k] = *reinterpret_cast<const uint32_t*>(lrh + ((qo + 8 * g + 4 * k) & (kRing - 1)));
+                    }
+                    uint32_t q0, q1;
+                    if (b & 1) {
+                        q0 = w[0];
+                        q1 = w[1];
+                    } else {  // quants start 2 bytes into the first dword
+                        q0 = __builtin_amdgcn_alignbit(w[1], w[0], 16);
+                        q1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
+                    }
+                    uint32_t a0, a1, a2, a3;
+                    q8_dword_bf16<NUM>(d, q0, a0, a1);
+                    q8_dword_bf16<NUM>(d, q1, a2, a3);
+                    const u32x4_t a = {a0, a1, a2, a3};
+                    acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                                     __builtin_bit_cast(bf16x8_t, xfrag), acc[h], 0, 0, 0);
+                }
             }
         }
     }
 
     // ---- add the wavefronts' partial sums (the rings are dead: reuse them) ---------------------------
     __syncthreads();
-    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][64]
-    red[wave * 64 + lane] = acc;
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [gate partial sums of the W K ranges | up partial sums][64]
+    red[wave * 64 + lane] = acc[0];
+    if constexpr (PAIRED) red[(W + wave) * 64 + lane] = acc[NQ - 1];
     __syncthreads();
     if (wave != 0 || !has_x) return;
     f32x4_t sum = red[lane];
@@ -389,13 +415,15 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
     if (gated && w > 4) w = 4;
     while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 16) w--;   // plenty of row groups: fewer, longer wavefronts
-    const int waves = gated ? 2 * w : w;
-    const size_t ring_bytes = (size_t)waves * 16 * kRingRow;
     // stage the activations in LDS when they are small enough to leave room for three workgroups
     // per compute unit (or, for few row groups, one)
     const size_t x_bytes = (size_t)M * (2 * K + 64);
     const size_t x_budget = groups >= 512 ? 16 * 1024 : 96 * 1024;
     const bool xlds = x_bytes <= x_budget;
+    // activations fetched from global memory for a gated pair: one wavefront takes both matrices of its K range
+    const bool paired = gated && !xlds && M >= kPairedMinM;
+    const int waves = (gated && !paired) ? 2 * w : w;
+    const size_t ring_bytes = (size_t)(gated ? 2 * w : w) * 16 * kRingRow;
     const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0);
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     // the rings of 8 wavefronts plus staged activations can exceed the default dynamic-LDS limit:
@@ -413,7 +441,13 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
         if (xlds) SNGGUF_LAUNCH_ONE(G, WM, true); \
         else SNGGUF_LAUNCH_ONE(G, WM, false); \
     } while (0)
-    if (gated) {
+    if (paired) {
+        static const hipError_t attr = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, true, 4, false, true>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
+        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y);
+    } else if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
     } else {

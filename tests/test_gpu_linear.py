@@ -346,6 +346,22 @@ def test_gate_up_silu(dev, c_oracle, qt, m):
     _check(got, c_oracle.silu_mul(g, u))
 
 
+@pytest.mark.parametrize("m", [1, 2, 11, 12, 13, 16])
+def test_gate_up_silu_line_aligned_kernel(dev, m):
+    """Q8_0 gate/up with K a multiple of 2048 and enough row groups takes the line-aligned kernel: activations staged
+    in LDS (m = 1), fetched per wavefront (m < 12), and from 12 rows on one wavefront working on both matrices of
+    its K range; ragged N."""
+    print(f"case gate_up span m={m}", flush=True)
+    n, k = 8200, 4096
+    gate = synthetic.make_packed(go.Q8_0, n, k, seed=61)
+    up = synthetic.make_packed(go.Q8_0, n, k, seed=62)
+    x = synthetic.make_activations(m, k, seed=63 + m)
+    g = go.gguf_linear_forward(x, gate, go.Q8_0)
+    u = go.gguf_linear_forward(x, up, go.Q8_0)
+    got = ops.gate_up_silu(x.to(dev), gate.to(dev), up.to(dev), go.Q8_0).cpu()
+    _check(got, torch.nn.functional.silu(g) * u)
+
+
 @pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q4_K), (go.Q6_K, go.Q6_K), (go.Q4_K, go.Q6_K), (go.Q5_K, go.Q8_0),
                                      (go.Q4_0, go.Q3_K), (go.Q5_1, go.Q2_K)])
 def test_grouped_linear_indicator(dev, qt_pair):
