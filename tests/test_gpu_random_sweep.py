@@ -1,0 +1,116 @@
+"""GPU: seeded random sweep over the dispatch boundaries of the linear entry points (row counts around 16 / 64 /
+384, ragged N, K down to one block, the line-aligned and the large-tile shapes, every type, both numerics modes,
+bias, residual, gated pair, workspace route) and of the grouped launcher (indicator / contiguous split / one empty
+group, equal and different types, with and without the dense workspace), each case against the oracle."""
+import random
+
+import pytest
+import torch
+
+from oracle import gguf_oracle as go
+from sensenova_u1_amd import ops, synthetic
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q8_0, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K]
+ROWS = [1, 2, 3, 5, 8, 11, 12, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 129, 383, 384, 385, 512, 700]
+
+
+def _ok(got, want, tag):
+    assert bool(torch.isfinite(got.float()).all()), tag
+    assert go.rel_l2(got, want) <= TOL, tag
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_linear_cases(dev, seed):
+    rnd = random.Random(seed)
+    for it in range(70):
+        qt = rnd.choice(TYPES)
+        bs = go.GGML_QUANT_SIZES[qt][0]
+        m = rnd.choice(ROWS)
+        mode = rnd.random()
+        if mode < 0.15:      # Q8_0 rows that are whole 2048-element spans, many row groups
+            qt, k, n = go.Q8_0, rnd.choice([2048, 4096, 6144]), rnd.choice([8192, 8200, 9000, 16400])
+        elif mode < 0.3:     # enough 256 x 256 tiles for the large-tile kernels
+            m = rnd.choice([384, 500, 1000, 2100])
+            n = rnd.choice([5632, 4100, 8200, 33000 if m < 600 else 3000])
+            k = bs * rnd.randint(1, max(1, 1024 // bs))
+        else:
+            n, k = rnd.randint(1, 2500), bs * rnd.randint(1, max(1, 3072 // bs))
+        if m * n > 6_000_000:
+            n = max(1, 6_000_000 // m)
+        numerics = rnd.choice([0, 1])
+        kind = rnd.choice(["linear", "linear", "residual", "gate_up", "ws"])
+        if kind == "gate_up" and m > 16:
+            kind = "linear"
+        use_bias = kind != "gate_up" and rnd.random() < 0.4
+        tag = f"seed={seed} it={it} kind={kind} qt={qt} m={m} n={n} k={k} numerics={numerics} bias={use_bias}"
+        print("case", tag, flush=True)
+        packed = synthetic.make_packed(qt, n, k, seed=it)
+        x = synthetic.make_activations(m, k, seed=1000 + it)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(it)) * 0.5).to(torch.bfloat16) if use_bias else None
+        xd, pd = x.to(dev), packed.to(dev)
+        bd = bias.to(dev) if bias is not None else None
+        want = go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics)
+        if kind == "linear":
+            got = ops.linear(xd, pd, qt, bd, numerics)
+        elif kind == "ws":
+            got = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            ws = torch.empty(n * k + 8, dtype=torch.bfloat16, device=dev)
+            ops.linear_ws_into(xd, pd, qt, bd, got, ws, numerics)
+        elif kind == "residual":
+            res = synthetic.make_activations(m, n, seed=5000 + it)
+            got = ops.linear_residual(xd, pd, qt, res.to(dev), bd, numerics)
+            want = (res.float() + want.float()).to(torch.bfloat16)
+        else:
+            up = synthetic.make_packed(qt, n, k, seed=9000 + it)
+            want = torch.nn.functional.silu(want) * go.gguf_linear_forward(x, up, qt, None, numerics=numerics)
+            got = ops.gate_up_silu(xd, pd, up.to(dev), qt, numerics)
+        _ok(got.cpu(), want, tag)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_grouped_cases(dev, seed):
+    rnd = random.Random(seed)
+    for it in range(50):
+        qu, qg = rnd.choice(TYPES), rnd.choice(TYPES)
+        if rnd.random() < 0.4:
+            qg = qu
+        step = max(go.GGML_QUANT_SIZES[qu][0], go.GGML_QUANT_SIZES[qg][0])
+        m = rnd.choice([1, 7, 17, 64, 65, 200, 383, 384, 600, 1500, 3000])
+        big = rnd.random() < 0.3
+        n = rnd.choice([2816, 4100, 8200]) if big else rnd.randint(1, 1500)
+        k = step * rnd.randint(1, max(1, (512 if big else 2048) // step))
+        if m * n > 6_000_000:
+            n = 6_000_000 // m
+        numerics = rnd.choice([0, 1])
+        form = rnd.choice(["indicator", "split", "all_text", "all_image"])
+        dense = rnd.random() < 0.5
+        tag = f"seed={seed} it={it} qu={qu} qg={qg} m={m} n={n} k={k} numerics={numerics} form={form} dense_ws={dense}"
+        print("case", tag, flush=True)
+        und, gen = synthetic.make_packed(qu, n, k, seed=it), synthetic.make_packed(qg, n, k, seed=7000 + it)
+        x = synthetic.make_activations(m, k, seed=100 + it)
+        g = torch.Generator().manual_seed(it)
+        n_text = rnd.randint(0, m)
+        ind = {"indicator": torch.rand(m, generator=g) < rnd.random(), "split": torch.arange(m) >= n_text,
+               "all_text": torch.zeros(m, dtype=torch.bool), "all_image": torch.ones(m, dtype=torch.bool)}[form]
+        bu = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if rnd.random() < 0.5 else None
+        bg = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if rnd.random() < 0.5 else None
+        want = torch.empty((m, n), dtype=torch.bfloat16)
+        if bool((~ind).any()):
+            want[~ind] = go.gguf_linear_forward(x[~ind], und, qu, bu, numerics=numerics)
+        if bool(ind.any()):
+            want[ind] = go.gguf_linear_forward(x[ind], gen, qg, bg, numerics=numerics)
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        row_ws = torch.empty(ops.grouped_workspace_bytes(m), dtype=torch.uint8, device=dev)
+        dense_ws = torch.empty(2 * n * k, dtype=torch.bfloat16, device=dev) if dense else None
+
+        def put(t):
+            return t.to(dev) if t is not None else None
+
+        if form == "split":
+            ops.grouped_linear_ws_into(put(x), None, n_text, put(und), qu, put(gen), qg, put(bu), put(bg), y, None, dense_ws, numerics)
+        else:
+            ops.grouped_linear_ws_into(put(x), put(ind.to(torch.uint8)), 0, put(und), qu, put(gen), qg, put(bu), put(bg), y,
+                                       row_ws, dense_ws, numerics)
+        _ok(y.cpu(), want, tag)
