@@ -465,6 +465,19 @@ def main() -> None:
             tflops = flops / (wall / gs * 1e-3) / 1e12
             kq["tower_M4096"] = {"value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(wall / gs, 4),
                                  "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2)}
+            kws = torch.empty(INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
+
+            def ktower_ws(i):
+                wsets = ktower[i % 2]
+                for j, (_, n, k, qt) in enumerate(kshapes):
+                    ops.linear_ws_into(xs[k], wsets[j], qt, None, ys[n], kws, num)
+
+            wall_kws, _ = run_region(ktower_ws, gs, max(2, args.gemm_warmup // 2))
+            tf_kws = flops / (wall_kws / gs * 1e-3) / 1e12
+            kq["tower_M4096_workspace"] = {"what": "the same tower through sngguf_linear_ws (weight pass + dense tile kernel)",
+                                           "value": round(tf_kws, 2), "unit": "TFLOP/s", "ms_per_step": round(wall_kws / gs, 4),
+                                           "pct_of_bf16_mfma_peak": round(100 * tf_kws / MFMA_BF16_PEAK_TFLOPS, 2)}
+            del kws
             del ktower, xs, ys
         kq["workload"] = ("configs[3]: Q4_K for q/k/v/o/gate/up, Q6_K for down; decode MLP at M=1,16 "
                           "(GB/s over packed weights + activations) and the 7 tower projections at M=4096")
