@@ -219,6 +219,35 @@ def main() -> None:
                            "down_us": round(dn * 1e3, 3)}
     result["decode_other_M"] = decode
 
+    # ---- the same MLP on the opt-in operand-order ("tiled") copy of the weights (made once at load time) ------------
+    if not args.no_extra:
+        tiled = [tuple(ops.q8_0_tile(t) for t in layer) for layer in layers]
+        torch.cuda.synchronize()
+        tl = {}
+        for m in (1, 4, 16):
+            xt = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
+            ht = torch.empty((m, INTER), dtype=torch.bfloat16, device=dev)
+            yt = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
+
+            def tstep(i):
+                tg, tu, td = tiled[i % L]
+                ops.gate_up_silu_tiled_into(xt, tg, tu, ht, num)
+                ops.linear_tiled_into(ht, td, None, None, yt, num)
+
+            kt = K if m == 1 else max(64, K // 4)
+            wall_t, _ = run_region(tstep, kt, min(W, 16))
+            _, ev_tg = run_region(lambda i: ops.gate_up_silu_tiled_into(xt, tiled[i % L][0], tiled[i % L][1], ht, num), kt, min(W, 16))
+            _, ev_td = run_region(lambda i: ops.linear_tiled_into(ht, tiled[i % L][2], None, None, yt, num), kt, min(W, 16))
+            gb = mlp_bytes(m) / (wall_t / kt * 1e-3) / 1e9
+            tl[f"M{m}"] = {"value": round(gb, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gb / HBM_PEAK_GBPS, 2),
+                           "ms_per_step": round(wall_t / kt, 6), "gate_up_us": round(ev_tg / kt * 1e3, 3),
+                           "down_us": round(ev_td / kt * 1e3, 3)}
+        tl["workload"] = ("the Q8_0 decode MLP of the headline leg with the weights in the opt-in operand-order copy "
+                          "(sngguf_q8_0_tile, same 34 bytes per block; GGUFLinear.decode_layout = 'tiled'): "
+                          "sngguf_gate_up_silu_tiled + sngguf_linear_tiled")
+        result["mlp_tiled_layout"] = tl
+        del tiled
+
     # ---- all seven linears of one decoder layer at M = 1: separate q / k / v launches against one launch over the
     # row-wise stacked q|k|v weight (modality.FusedProjections); gate/up fused with SiLU in both ---------------------
     if not args.no_extra:

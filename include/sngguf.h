@@ -153,6 +153,29 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
                         int64_t N, int64_t K, void* h, int numerics, void* stream);
 
 /*
+ * Operand-order ("tiled") copy of a Q8_0 matrix for the decode path.  No counterpart in the reference, which keeps
+ * the GGUF rows as they are in the file (src/sensenova_u1/utils/gguf_loader.py:42) - and so do all entry points
+ * above.  For a model that stays resident on the device a second arrangement of the same blocks, made once at
+ * load time, lets the decode GEMV load the weights in the order its matrix instruction consumes them (no staging,
+ * no realignment of 34-byte blocks): measured 8 - 10 % faster on the M = 1 MLP step.
+ *
+ *   sngguf_q8_0_tiled_bytes(N, K)   size of the copy (N rows padded to a multiple of 16; 34 bytes per block as before);
+ *                                   0 unless K % 256 == 0
+ *   sngguf_q8_0_tile                GGUF Q8_0 rows [N][K / 32 * 34] -> tiled (device to device, on `stream`)
+ *   sngguf_linear_tiled             y[M][N] = x[M][K] . W^T (+ bias) (+ residual, as sngguf_linear_residual), 1 <= M <= 16
+ *   sngguf_gate_up_silu_tiled       as sngguf_gate_up_silu on two tiled matrices
+ * Results are those of sngguf_linear / sngguf_gate_up_silu on the GGUF rows (same decode and rounding chain; the
+ * summation order over K differs, as it does between the other kernels).  M > 16 returns SNGGUF_E_BADSHAPE: larger
+ * inputs go through the GGUF-native entry points.
+ */
+int64_t sngguf_q8_0_tiled_bytes(int64_t N, int64_t K);
+int sngguf_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, void* stream);
+int sngguf_linear_tiled(const void* x, int64_t M, const void* tiled, int64_t N, int64_t K, const void* bias,
+                        const void* residual, void* y, int numerics, void* stream);
+int sngguf_gate_up_silu_tiled(const void* x, int64_t M, const void* tiled_gate, const void* tiled_up,
+                              int64_t N, int64_t K, void* h, int numerics, void* stream);
+
+/*
  * Modality-grouped linear: rows of x whose indicator is 0 use the understanding weights
  * q_und, rows whose indicator is non-zero use the generation weights q_gen, in one pass:
  *     y[~ind] = x[~ind] . W_und^T ;  y[ind] = x[ind] . W_gen^T

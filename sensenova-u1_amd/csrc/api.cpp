@@ -10,6 +10,10 @@ int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
                       hipStream_t stream);
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                 const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
+int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
+int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
+                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
 int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
                       hipStream_t stream);
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
@@ -159,6 +163,49 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
     if (M > 16) return SNGGUF_E_BADSHAPE;
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+}
+
+int64_t sngguf_q8_0_tiled_bytes(int64_t N, int64_t K) {
+    if (N <= 0 || K <= 0 || N >= kMaxDim || K >= kMaxDim || K % 256 != 0) return 0;
+    return sngguf::q8_0_tiled_bytes(N, K);
+}
+
+int sngguf_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, void* stream) {
+    if (N < 0 || K <= 0 || N >= kMaxDim || K >= kMaxDim || K % 256 != 0) return SNGGUF_E_BADSHAPE;
+    if (N == 0) return SNGGUF_OK;
+    if (!q || !tiled) return SNGGUF_E_NULLPTR;
+    if (!aligned(q, 16) || !aligned(tiled, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_q8_0_tile(q, N, K, tiled, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+int check_tiled(const void* x, int64_t M, const void* t, int64_t N, int64_t K, const void* y, int numerics) {
+    if (!known_numerics(numerics)) return SNGGUF_E_BADTYPE;
+    if (M < 0 || M > 16 || N < 0 || K <= 0 || N >= kMaxDim || K >= kMaxDim || K % 256 != 0) return SNGGUF_E_BADSHAPE;
+    if (M == 0 || N == 0) return SNGGUF_OK;
+    if (!x || !t || !y) return SNGGUF_E_NULLPTR;
+    if (!aligned(x, 16) || !aligned(y, 16) || !aligned(t, 16)) return SNGGUF_E_ALIGN;
+    return SNGGUF_OK;
+}
+}  // namespace
+
+int sngguf_linear_tiled(const void* x, int64_t M, const void* tiled, int64_t N, int64_t K, const void* bias,
+                        const void* residual, void* y, int numerics, void* stream) {
+    const int rc = check_tiled(x, M, tiled, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (residual && !aligned(residual, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_gemv_q8_tiled(x, M, tiled, nullptr, N, K, bias, residual, y, numerics, false,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int sngguf_gate_up_silu_tiled(const void* x, int64_t M, const void* tiled_gate, const void* tiled_up, int64_t N, int64_t K,
+                              void* h, int numerics, void* stream) {
+    const int rc = check_tiled(x, M, tiled_gate, N, K, h, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (!tiled_up) return SNGGUF_E_NULLPTR;
+    if (!aligned(tiled_up, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_gemv_q8_tiled(x, M, tiled_gate, tiled_up, N, K, nullptr, nullptr, h, numerics, true,
+                                        static_cast<hipStream_t>(stream));
 }
 
 int64_t sngguf_grouped_workspace_bytes(int64_t M) { return sngguf::grouped_workspace_bytes(M); }

@@ -128,8 +128,16 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     projections and the SiLU product run as one fused GEMV launch."""
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     same = int(gate_proj.weight.quant_type) == int(up_proj.weight.quant_type)
-    if 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16 \
-            and gate_proj.in_features % 64 == 0:
+    decode = 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16
+    # the tiled gated kernel has no paired mode: beyond 8 rows the GGUF-native pair kernel is the faster one
+    tg = gate_proj.tiled_weight() if decode and rows <= 8 else None
+    tu = up_proj.tiled_weight() if decode and tg is not None else None
+    if tu is not None:
+        x2d = x.reshape(-1, gate_proj.in_features)
+        h = torch.empty((*x.shape[:-1], gate_proj.out_features), dtype=torch.bfloat16, device=x.device)
+        ops.gate_up_silu_tiled_into(x2d if x2d.is_contiguous() else x2d.contiguous(), tg, tu,
+                                    h.view(-1, gate_proj.out_features), gate_proj.numerics)
+    elif decode and gate_proj.in_features % 64 == 0:
         h = ops.gate_up_silu(x, gate_proj.weight, up_proj.weight, int(gate_proj.weight.quant_type), gate_proj.numerics)
     else:
         h = torch.nn.functional.silu(gate_proj(x)) * up_proj(x)

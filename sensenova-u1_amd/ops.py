@@ -33,7 +33,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
     "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
-    "sngguf_grouped_linear_ws",
+    "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -83,6 +83,14 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_grouped_linear.restype = ci
     lib.sngguf_grouped_linear_ws.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, vp, i64, ci, vp]
     lib.sngguf_grouped_linear_ws.restype = ci
+    lib.sngguf_q8_0_tiled_bytes.argtypes = [i64, i64]
+    lib.sngguf_q8_0_tiled_bytes.restype = i64
+    lib.sngguf_q8_0_tile.argtypes = [vp, i64, i64, vp, vp]
+    lib.sngguf_q8_0_tile.restype = ci
+    lib.sngguf_linear_tiled.argtypes = [vp, i64, vp, i64, i64, vp, vp, vp, ci, vp]
+    lib.sngguf_linear_tiled.restype = ci
+    lib.sngguf_gate_up_silu_tiled.argtypes = [vp, i64, vp, vp, i64, i64, vp, ci, vp]
+    lib.sngguf_gate_up_silu_tiled.restype = ci
     # host-only GGUF container reader
     cp = ctypes.c_char_p
     lib.sngguf_file_open.argtypes = [cp, ctypes.POINTER(vp), cp, i64]
@@ -245,6 +253,39 @@ def grouped_linear_ws_into(x2d, indicator, n_text, packed_und, qt_und, packed_ge
             y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), _ptr(dense_workspace),
             dw_bytes, numerics, ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_grouped_linear_ws")
+
+
+def q8_0_tile(packed: torch.Tensor) -> torch.Tensor:
+    """Operand-order copy of a Q8_0 weight ``[N, K / 32 * 34]`` (device tensor, K a multiple of 256) for the tiled decode
+    entry points; a flat uint8 tensor of ``sngguf_q8_0_tiled_bytes(N, K)`` bytes."""
+    n, k = packed.shape[0], packed.shape[1] // 34 * 32
+    nbytes = int(load_library().sngguf_q8_0_tiled_bytes(n, k))
+    if nbytes == 0 and n > 0:
+        raise SnGgufError(f"q8_0_tile: in_features = {k} is not a multiple of 256")
+    out = torch.empty(nbytes, dtype=torch.uint8, device=packed.device)
+    with torch.cuda.device(packed.device):
+        rc = load_library().sngguf_q8_0_tile(_ptr(packed), n, k, _ptr(out), ctypes.c_void_p(_stream(packed.device)))
+    _check(rc, "sngguf_q8_0_tile")
+    return out
+
+
+def linear_tiled_into(x2d: torch.Tensor, tiled: torch.Tensor, bias: Optional[torch.Tensor], residual: Optional[torch.Tensor],
+                      y2d: torch.Tensor, numerics: int) -> None:
+    """y2d[M, N] = x2d[M, K] @ W^T (+ bias) (+ residual) with W given as its tiled copy; M <= 16."""
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_linear_tiled(_ptr(x2d), x2d.shape[0], _ptr(tiled), y2d.shape[1], x2d.shape[1], _ptr(bias),
+                                                _ptr(residual), _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_linear_tiled")
+
+
+def gate_up_silu_tiled_into(x2d: torch.Tensor, tiled_gate: torch.Tensor, tiled_up: torch.Tensor, h2d: torch.Tensor,
+                            numerics: int) -> None:
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_gate_up_silu_tiled(_ptr(x2d), x2d.shape[0], _ptr(tiled_gate), _ptr(tiled_up), h2d.shape[1],
+                                                      x2d.shape[1], _ptr(h2d), numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_gate_up_silu_tiled")
 
 
 def _as_bf16_rows(x: torch.Tensor, k: int, what: str) -> torch.Tensor:

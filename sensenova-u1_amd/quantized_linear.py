@@ -142,12 +142,19 @@ class GGUFLinear(nn.Linear):
       rows many times over (the denoising loop) on a device with memory to spare, it removes the
       weight pass from every call but the first.  Not meant to be combined with layer offloading.
 
+    ``decode_layout = "tiled"`` (Q8_0 with ``in_features`` a multiple of 256 only; default ``"native"``) makes the
+    decode calls (at most 16 rows) read an operand-order copy of the weight that is built on first use and kept
+    beside the GGUF bytes (the same 34 bytes per block again): 8 - 10 % faster on the M = 1 MLP step, for models
+    that stay resident on the device.  The copy follows the packed bytes: it is rebuilt when they move or change.
+
     Other compute dtypes always take dequantize + matmul.
     """
 
     numerics: int = ops.NUM_UPSTREAM_FP16
     gemm_policy: str = "auto"     # "auto" | "two_pass" | "fused" | "resident", for inputs beyond the fused GEMV's row limit
     _dense_cache = None           # (key, bf16 weight) of the "resident" policy
+    decode_layout: str = "native"  # "native" | "tiled": weight layout the decode kernels read
+    _tiled_cache = None           # (key, operand-order copy) of the "tiled" decode layout
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False,
                  compute_dtype: Optional[torch.dtype] = None, device=None) -> None:
@@ -160,6 +167,35 @@ class GGUFLinear(nn.Linear):
             raise RuntimeError("GGUFLinear.weight is not a GGUFParameter (no quant_type); was the checkpoint loaded?")
         return int(w.quant_type)
 
+    def tiled_weight(self) -> Optional[torch.Tensor]:
+        """The operand-order copy of the weight when ``decode_layout == "tiled"`` applies to this module (Q8_0,
+        ``in_features`` a multiple of 256, weight on the device), built on first use; else ``None``."""
+        if self.decode_layout != "tiled":
+            if self.decode_layout != "native":
+                raise ValueError(f"GGUFLinear.decode_layout is {self.decode_layout!r}; expected 'native' or 'tiled'")
+            return None
+        if self._weight_type() != ops.Q8_0 or self.in_features % 256 != 0 or self.weight.device.type != "cuda":
+            return None
+        key = (self.weight.data_ptr(), self.weight._version)
+        if self._tiled_cache is None or self._tiled_cache[0] != key:
+            self._tiled_cache = (key, ops.q8_0_tile(self.weight.data))
+        return self._tiled_cache[1]
+
+    def _decode_tiled(self, inputs: torch.Tensor, residual: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        rows = inputs.numel() // self.in_features if inputs.numel() else 0
+        if not 0 < rows <= 16:
+            return None
+        tiled = self.tiled_weight()
+        if tiled is None:
+            return None
+        x2d = inputs.reshape(-1, self.in_features)
+        x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
+        out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
+        bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
+        res2d = residual.reshape(-1, self.out_features).contiguous() if residual is not None else None
+        ops.linear_tiled_into(x2d, tiled, bias, res2d, out.view(-1, self.out_features), self.numerics)
+        return out
+
     def forward(self, inputs: torch.Tensor) -> torch.Tensor:
         qtype = self._weight_type()
         compute_dtype = self.compute_dtype or inputs.dtype
@@ -167,6 +203,10 @@ class GGUFLinear(nn.Linear):
             raise RuntimeError(f"GGUFLinear: input dtype {inputs.dtype} does not match compute dtype {compute_dtype}")
         if compute_dtype == torch.bfloat16:
             rows = inputs.numel() // self.in_features if inputs.numel() else 0
+            if self.decode_layout != "native":
+                out = self._decode_tiled(inputs, None)
+                if out is not None:
+                    return out
             if rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused":
                 return ops.linear(inputs, self.weight, qtype, self.bias, self.numerics)
             if self.gemm_policy not in ("auto", "two_pass", "resident"):
@@ -187,6 +227,10 @@ class GGUFLinear(nn.Linear):
         fused_rows = rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused"
         if inputs.dtype == torch.bfloat16 and (self.compute_dtype or inputs.dtype) == torch.bfloat16 and fused_rows \
                 and residual.dtype == torch.bfloat16:
+            if self.decode_layout != "native":
+                out = self._decode_tiled(inputs, residual)
+                if out is not None:
+                    return out
             return ops.linear_residual(inputs, self.weight, self._weight_type(), residual, self.bias, self.numerics)
         return residual + self(inputs)
 
@@ -209,6 +253,10 @@ class GGUFLinear(nn.Linear):
     def drop_dense_cache(self) -> None:
         """Release the bf16 weight the "resident" policy keeps."""
         self._dense_cache = None
+
+    def drop_tiled_cache(self) -> None:
+        """Release the operand-order copy the "tiled" decode layout keeps."""
+        self._tiled_cache = None
 
     def extra_repr(self) -> str:
         qt = getattr(self.weight, "quant_type", None)

@@ -74,6 +74,15 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_gate_up_silu(p, 1, p, None, 8, 4, 64, p, 1, None) == E_NULL
     assert lib.sngguf_grouped_linear(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_NULL  # no workspace
     assert lib.sngguf_grouped_linear(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, 1, None) == E_SHAPE  # n_text > M
+    assert lib.sngguf_q8_0_tiled_bytes(4096, 4096) == 4096 * 4096 // 32 * 34 and lib.sngguf_q8_0_tiled_bytes(17, 256) == 32 * 8 * 34
+    assert lib.sngguf_q8_0_tiled_bytes(16, 288) == 0                                          # K % 256
+    assert lib.sngguf_q8_0_tile(p, 16, 288, p, None) == E_SHAPE
+    assert lib.sngguf_q8_0_tile(None, 16, 256, p, None) == E_NULL
+    assert lib.sngguf_linear_tiled(p, 17, p, 16, 256, None, None, p, 1, None) == E_SHAPE      # decode rows only
+    assert lib.sngguf_linear_tiled(p, 1, p, 16, 256, None, None, odd, 1, None) == E_ALIGN
+    assert lib.sngguf_linear_tiled(p, 1, p, 16, 256, None, None, p, 5, None) == E_TYPE
+    assert lib.sngguf_gate_up_silu_tiled(p, 1, p, None, 16, 256, p, 1, None) == E_NULL
+    assert lib.sngguf_linear_tiled(p, 0, p, 16, 256, None, None, p, 1, None) == 0
     # without a dense workspace the _ws form is the plain one, with the same checks
     assert lib.sngguf_grouped_linear_ws(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_SHAPE
     assert lib.sngguf_grouped_linear_ws(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_NULL

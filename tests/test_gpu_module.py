@@ -135,6 +135,51 @@ def test_resident_policy_keeps_the_bf16_weight_until_the_packed_bytes_change(tmp
     assert mod._dense_cache is None
 
 
+def test_tiled_decode_layout(tmp_path, dev):
+    """decode_layout = "tiled": decode calls read the operand-order copy (built once, rebuilt when the packed bytes move),
+    larger inputs and other formats take the usual routes; results agree with the oracle and, closely, with the native layout."""
+    print("case module tiled decode layout", flush=True)
+    model, packed = _load(tmp_path, dev, 8)
+    mlp = model.layers[0].mlp
+    w = {n: torch.from_numpy(packed[f"layers.0.mlp.{n}.weight"]) for n in ("gate_proj", "up_proj", "down_proj")}
+    for m in (1, 5, 16):
+        x = synthetic.make_activations(m, H, seed=30 + m)
+        want, _ = go.mlp_forward(x, w["gate_proj"], w["up_proj"], w["down_proj"], (8, 8, 8))
+        native = gated_mlp(x.to(dev), mlp.gate_proj, mlp.up_proj, mlp.down_proj)
+        for mod in (mlp.gate_proj, mlp.up_proj, mlp.down_proj):
+            mod.decode_layout = "tiled"
+        got = gated_mlp(x.to(dev), mlp.gate_proj, mlp.up_proj, mlp.down_proj)
+        assert go.rel_l2(got.cpu(), want) <= 2 * TOL and go.rel_l2(got.cpu(), native.cpu()) <= 1e-3
+        kept = mlp.down_proj._tiled_cache[1]
+        h = synthetic.make_activations(m, I, seed=40 + m).to(dev)
+        res = synthetic.make_activations(m, H, seed=41 + m).to(dev)
+        y = mlp.down_proj(h.reshape(1, m, I))
+        assert y.shape == (1, m, H) and mlp.down_proj._tiled_cache[1] is kept
+        wantd = go.gguf_linear_forward(h.cpu(), w["down_proj"], 8)
+        assert go.rel_l2(y.cpu().reshape(m, H), wantd) <= TOL
+        yr = mlp.down_proj.forward_residual(h, res)
+        assert go.rel_l2(yr.cpu(), (res.cpu().float() + wantd.float()).to(torch.bfloat16)) <= TOL
+        for mod in (mlp.gate_proj, mlp.up_proj, mlp.down_proj):
+            mod.decode_layout = "native"
+    mod = mlp.down_proj
+    mod.decode_layout = "tiled"
+    big = synthetic.make_activations(40, I, seed=9).to(dev)
+    assert go.rel_l2(mod(big).cpu(), go.gguf_linear_forward(big.cpu(), w["down_proj"], 8)) <= TOL   # beyond 16 rows: native routes
+    other = model.layers[1].mlp.down_proj
+    mod.weight.data = other.weight.data.clone()                                     # packed bytes move: the copy follows
+    x1 = synthetic.make_activations(1, I, seed=3).to(dev)
+    assert go.rel_l2(mod(x1).cpu(), other(x1).cpu()) <= 1e-3
+    mod.drop_tiled_cache()
+    assert mod._tiled_cache is None
+    mod.decode_layout = "sideways"
+    with pytest.raises(ValueError):
+        mod(x1)
+    mod.decode_layout = "native"
+    q4 = _load(tmp_path, dev, 12)[0].layers[0].mlp.down_proj
+    q4.decode_layout = "tiled"                                                       # not Q8_0: stays on the native path
+    assert q4.tiled_weight() is None and q4(x1).shape == (1, H)
+
+
 @pytest.mark.parametrize("quant", [8, 12, 3])
 def test_fused_qkv_projections(tmp_path, dev, quant):
     """Projections that read the same hidden states (q / k / v in the model; here the four H-input projections the
