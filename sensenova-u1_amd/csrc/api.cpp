@@ -181,7 +181,7 @@ int sngguf_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, void* str
 namespace {
 int check_tiled(const void* x, int64_t M, const void* t, int64_t N, int64_t K, const void* y, int numerics) {
     if (!known_numerics(numerics)) return SNGGUF_E_BADTYPE;
-    if (M < 0 || M > 16 || N < 0 || K <= 0 || N >= kMaxDim || K >= kMaxDim || K % 256 != 0) return SNGGUF_E_BADSHAPE;
+    if (M < 0 || M > 16 || N < 0 || K <= 0 || N >= kMaxDim || K >= ((int64_t)1 << 27) || K % 256 != 0) return SNGGUF_E_BADSHAPE;  // 32-bit offsets inside a row group
     if (M == 0 || N == 0) return SNGGUF_OK;
     if (!x || !t || !y) return SNGGUF_E_NULLPTR;
     if (!aligned(x, 16) || !aligned(y, 16) || !aligned(t, 16)) return SNGGUF_E_ALIGN;

@@ -62,33 +62,34 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     const int r = lane & 15, g = lane >> 4;
     const int64_t rg = blockIdx.x, G = (N + 15) >> 4;
     const int runs = (int)(K >> 8);                       // runs of eight blocks
-    const int r0 = (int)((int64_t)kw * runs / W), r1 = (int)((int64_t)(kw + 1) * runs / W);
+    const int r0 = kw * runs / W, r1 = (kw + 1) * runs / W;
+    // Bases in 64 bits once, everything inside the loop as 32-bit offsets (a group's quants are 16 K bytes, K < 2^27 is
+    // checked by the launcher): with 64-bit index arithmetic per request the kernel measured 14.6 instead of 12.6 us.
     const uint8_t* __restrict__ qp = t + rg * (K >> 5) * 512 + 16 * lane;                  // + run * 4096 + pair * 1024
     const uint8_t* __restrict__ sp = t + 16 * G * K + rg * runs * 256 + 16 * r;            // + run * 256
 
     const bool has_x = r < M;
     const int xr = has_x ? r : M - 1;   // columns >= M are never stored: those lanes re-read the last activation row
     const bf16_t* xrow = x + (int64_t)xr * K + 8 * g;
-    const int64_t xs_stride = 2 * K + 64;                 // bytes per activation row in LDS (+64: rows on different banks)
+    const int xs_stride = 2 * (int)K + 64;                // bytes per activation row in LDS (+64: rows on different banks)
     const uint8_t* xsrow = lds + xr * xs_stride + 16 * g;
 
     u32x4_t wq[2][4], ws[2], xf[2][8];
     auto fetch = [&](int run, int buf) {
 #pragma unroll
-        for (int p = 0; p < 4; p++) wq[buf][p] = *reinterpret_cast<const u32x4_t*>(qp + (int64_t)run * 4096 + p * 1024);
-        ws[buf] = *reinterpret_cast<const u32x4_t*>(sp + (int64_t)run * 256);
+        for (int p = 0; p < 4; p++) wq[buf][p] = *reinterpret_cast<const u32x4_t*>(qp + (uint32_t)(run * 4096 + p * 1024));
+        ws[buf] = *reinterpret_cast<const u32x4_t*>(sp + (uint32_t)(run * 256));
         if constexpr (!XLDS) {
 #pragma unroll
-            for (int b = 0; b < 8; b++) xf[buf][b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)run * 8 + b) * 32);
+            for (int b = 0; b < 8; b++) xf[buf][b] = *reinterpret_cast<const u32x4_t*>(xrow + (uint32_t)((run * 8 + b) * 32));
         }
     };
     if (r0 < r1) fetch(r0, 0);   // the weights are requested before the activations are staged
     if constexpr (XLDS) {
         const int pieces_per_row = (int)(K >> 3);
-        for (int f = tid; f < M * pieces_per_row; f += blockDim.x) {
-            const int m = f / pieces_per_row, c = f - m * pieces_per_row;
-            *reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + 8 * c);
-        }
+        for (int m = 0; m < M; m++)
+            for (int c = tid; c < pieces_per_row; c += (int)blockDim.x)
+                *reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (uint32_t)(m * (int)K + 8 * c));
         __syncthreads();
     }
 
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
                 q8_dword_bf16<NUM>(d, wq[buf][p][2 * h + 1], a2, a3);
                 const u32x4_t a = {a0, a1, a2, a3};
                 u32x4_t xb;
-                if constexpr (XLDS) xb = *reinterpret_cast<const u32x4_t*>(xsrow + ((int64_t)run * 8 + b) * 64);
+                if constexpr (XLDS) xb = *reinterpret_cast<const u32x4_t*>(xsrow + (run * 8 + b) * 64);
                 else xb = xf[buf][b];
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                               __builtin_bit_cast(bf16x8_t, xb), acc, 0, 0, 0);
