@@ -40,9 +40,12 @@ def test_random_linear_cases(dev, seed):
         if m * n > 6_000_000:
             n = max(1, 6_000_000 // m)
         numerics = rnd.choice([0, 1])
-        kind = rnd.choice(["linear", "linear", "residual", "gate_up", "ws"])
+        kind = rnd.choice(["linear", "linear", "residual", "gate_up", "ws", "tiled"])
         if kind == "gate_up" and m > 16:
             kind = "linear"
+        if kind == "tiled":   # the operand-order copy: Q8_0, decode rows, whole 256-element runs
+            qt, bs, m = go.Q8_0, 32, rnd.choice([r for r in ROWS if r <= 16])
+            k = 256 * max(1, k // 256)
         use_bias = kind != "gate_up" and rnd.random() < 0.4
         tag = f"seed={seed} it={it} kind={kind} qt={qt} m={m} n={n} k={k} numerics={numerics} bias={use_bias}"
         print("case", tag, flush=True)
@@ -58,6 +61,12 @@ def test_random_linear_cases(dev, seed):
             got = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
             ws = torch.empty(n * k + 8, dtype=torch.bfloat16, device=dev)
             ops.linear_ws_into(xd, pd, qt, bd, got, ws, numerics)
+        elif kind == "tiled":
+            res = synthetic.make_activations(m, n, seed=5000 + it) if rnd.random() < 0.5 else None
+            got = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            ops.linear_tiled_into(xd, ops.q8_0_tile(pd), bd, res.to(dev) if res is not None else None, got, numerics)
+            if res is not None:
+                want = (res.float() + want.float()).to(torch.bfloat16)
         elif kind == "residual":
             res = synthetic.make_activations(m, n, seed=5000 + it)
             got = ops.linear_residual(xd, pd, qt, res.to(dev), bd, numerics)
