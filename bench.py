@@ -296,17 +296,40 @@ def main() -> None:
             ops.linear_into(x1, qkv[i % nl], Q8_0, None, yqkv, num)
             layer_rest(i, True)
 
+        # the same layer with its two RMSNorms (input_layernorm in front of q|k|v, post_attention_layernorm in front of
+        # the MLP): as one library norm launch each, and folded into the q|k|v and gate/up launches
+        gammas = [(torch.rand(HIDDEN, generator=torch.Generator().manual_seed(70 + i)) + 0.5).to(torch.bfloat16).to(dev) for i in range(2)]
+        eps = 1e-6
+
+        def layer_norms_separate(i):
+            n1 = torch.nn.functional.rms_norm(x1, (HIDDEN,), gammas[0], eps)
+            ops.linear_into(n1, qkv[i % nl], Q8_0, None, yqkv, num)
+            gate, up, down = layers[i % len(layers)]
+            ops.linear_residual_into(yq, attn[i % nl][3], Q8_0, None, res, hid, num)
+            n2 = torch.nn.functional.rms_norm(hid, (HIDDEN,), gammas[1], eps)
+            ops.gate_up_silu_into(n2, gate, up, Q8_0, h1, num)
+            ops.linear_residual_into(h1, down, Q8_0, None, hid, yo, num)
+
+        def layer_norms_fused(i):
+            ops.rmsnorm_linear_into(x1, gammas[0], eps, qkv[i % nl], Q8_0, None, yqkv, num)
+            gate, up, down = layers[i % len(layers)]
+            ops.linear_residual_into(yq, attn[i % nl][3], Q8_0, None, res, hid, num)
+            ops.rmsnorm_gate_up_silu_into(hid, gammas[1], eps, gate, up, Q8_0, h1, num)
+            ops.linear_residual_into(h1, down, Q8_0, None, hid, yo, num)
+
         k3 = max(64, K // 4)
         lbytes = (2 * linear_bytes(1, HIDDEN, HIDDEN) + 2 * linear_bytes(1, KV, HIDDEN) + mlp_bytes(1))
         legs = {}
         for name, fn, launches in (("separate", layer_separate, "6 linears + 2 adds"), ("stacked_qkv", layer_stacked, "4 linears + 2 adds"),
-                                   ("stacked_qkv_fused_residual", layer_stacked_residual, "4 linears")):
+                                   ("stacked_qkv_fused_residual", layer_stacked_residual, "4 linears"),
+                                   ("with_norms_separate", layer_norms_separate, "4 linears + 2 torch rms_norm"),
+                                   ("with_norms_fused", layer_norms_fused, "4 linears, both RMSNorms inside the q|k|v and gate/up launches")):
             wall_l, _ = run_region(fn, k3, min(W, 16))
             legs[name] = {"launches": launches, "us_per_layer": round(wall_l / k3 * 1e3, 2),
                           "value": round(lbytes / (wall_l / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"}
         result["decode_layer"] = {
             "workload": "the 7 Q8_0 linears of one decoder layer at M=1 (q,o 4096^2; k,v 4096->1024; gate/up fused with SiLU; "
-                        "down) and its two residual adds; no attention, no norms",
+                        "down) and its two residual adds; no attention; the with_norms legs add the layer's two RMSNorms",
             "bytes_per_layer": lbytes, **legs,
         }
         del attn, qkv
@@ -388,6 +411,25 @@ def main() -> None:
 
         wall3, _ = run_region(tower_resident, gs, args.gemm_warmup)
         del dense
+        # q | k | v as one [6144, 4096] matrix (rows of the three packed weights one after another, what
+        # FusedProjections builds at load): 384 large tiles in one launch instead of 256 + 64 + 64
+        qkv = [torch.cat([tower[r][0], tower[r][1], tower[r][2]], dim=0).contiguous() for r in range(2)]
+        y_qkv = torch.empty((m, HIDDEN + 2 * KV), dtype=torch.bfloat16, device=dev)
+        rest = [(j, n, k) for j, (nm, n, k) in enumerate(shapes) if nm not in ("q", "k", "v")]
+
+        def tower_stacked(i):
+            ops.linear_into(xs[HIDDEN], qkv[i % 2], Q8_0, None, y_qkv, num)
+            for j, n, k in rest:
+                ops.linear_into(xs[k], tower[i % 2][j], Q8_0, None, ys[n], num)
+
+        def tower_stacked_ws(i):
+            ops.linear_ws_into(xs[HIDDEN], qkv[i % 2], Q8_0, None, y_qkv, wtmp, num)
+            for j, n, k in rest:
+                ops.linear_ws_into(xs[k], tower[i % 2][j], Q8_0, None, ys[n], wtmp, num)
+
+        wall_st, _ = run_region(tower_stacked, gs, args.gemm_warmup)
+        wall_st_ws, _ = run_region(tower_stacked_ws, gs, args.gemm_warmup)
+        del qkv, y_qkv
         gate_tflops = 2.0 * m * INTER * HIDDEN / (gate_ms * 1e-3) / 1e12
         result["gemm"] = {
             "workload": "configs[2]: Q8_0 generation-tower projections over M=4096 image tokens "
@@ -426,6 +468,16 @@ def main() -> None:
                 "pct_of_bf16_mfma_peak": round(100 * flops / (wall_ws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
                 "gate_us": round(ev_gate_ws / (gs * 2) * 1e3, 2),
                 "gate_tflops": round(2.0 * m * INTER * HIDDEN / (ev_gate_ws / (gs * 2) * 1e-3) / 1e12, 2),
+            },
+            "stacked_qkv": {
+                "what": "the same tower with q, k and v as one stacked [6144, 4096] weight (one launch of 384 large tiles "
+                        "instead of 256 + 64 + 64; k / v alone have too few tiles for the large-tile kernel), fused route "
+                        "and workspace route",
+                "value": round(flops / (wall_st / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(wall_st / gs, 4),
+                "pct_of_bf16_mfma_peak": round(100 * flops / (wall_st / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+                "workspace_value": round(flops / (wall_st_ws / gs * 1e-3) / 1e12, 2),
+                "workspace_ms_per_step": round(wall_st_ws / gs, 4),
+                "workspace_pct_of_bf16_mfma_peak": round(100 * flops / (wall_st_ws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
             },
             "resident": {
                 "what": "gemm_policy 'resident': the bf16 weights written once by sngguf dequantize and kept "

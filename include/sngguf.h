@@ -153,6 +153,27 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
                         int64_t N, int64_t K, void* h, int numerics, void* stream);
 
 /*
+ * RMSNorm fused in front of a decode projection.  In the decoder layer the q / k / v projections read
+ * input_layernorm(hidden) and gate / up read post_attention_layernorm(hidden)
+ * (src/sensenova_u1/models/neo_unify/modeling_qwen3.py:919, :938; Qwen3RMSNorm.forward at :192-197):
+ *     v = bf16( x * rsqrt(mean(x^2) + eps) )      fp32 arithmetic, one rounding
+ *     n = bf16( gamma * v )                       gamma: the norm's weight, K bf16 values, 16-byte aligned
+ * and these two entry points contract n instead of x, applying the norm to the activations a workgroup has
+ * staged in LDS - no launch and no buffer for the normalized rows.  Offered where that staging exists
+ * (sngguf_rmsnorm_fits: Q8_0, K % 256 == 0, M (2 K + 64) <= 16384, i.e. one row at K = 4096, three at 2048);
+ * other types or sizes return SNGGUF_E_BADTYPE / SNGGUF_E_BADSHAPE and the caller runs the norm on its own.
+ * The sum of squares is added up in a different order than torch's mean, so a normalized value can differ
+ * from the reference's by one bf16 unit where the rounding is a near tie; everything after is the same chain
+ * as sngguf_linear / sngguf_gate_up_silu.
+ */
+int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K);
+int sngguf_rmsnorm_linear(const void* x, int64_t M, const void* gamma, float eps, const void* q, int qtype,
+                          int64_t N, int64_t K, const void* bias, void* y, int numerics, void* stream);
+int sngguf_rmsnorm_gate_up_silu(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate,
+                                const void* q_up, int qtype, int64_t N, int64_t K, void* h, int numerics,
+                                void* stream);
+
+/*
  * Operand-order ("tiled") copy of a Q8_0 matrix for the decode path.  No counterpart in the reference, which keeps
  * the GGUF rows as they are in the file (src/sensenova_u1/utils/gguf_loader.py:42) - and so do all entry points
  * above.  For a model that stays resident on the device a second arrangement of the same blocks, made once at

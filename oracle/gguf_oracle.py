@@ -234,6 +234,18 @@ def gguf_linear_forward(x: torch.Tensor, packed: torch.Tensor, quant_type: int, 
     return torch.nn.functional.linear(x.detach().cpu().to(compute_dtype), w, b)
 
 
+def qwen3_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Qwen3RMSNorm.forward, op by op (src/sensenova_u1/models/neo_unify/modeling_qwen3.py:192-197): upcast to
+    fp32, variance = mean of squares over the last dim, x * rsqrt(variance + eps), cast back to the input dtype,
+    then the product with the weight in the input dtype.  Pinned in tests/test_oracle_rmsnorm.py against closed
+    forms (constant rows, one-hot rows, scale invariance) and torch.nn.functional.rms_norm."""
+    input_dtype = x.dtype
+    h = x.to(torch.float32)
+    variance = h.pow(2).mean(-1, keepdim=True)
+    h = h * torch.rsqrt(variance + eps)
+    return weight * h.to(input_dtype)
+
+
 def mlp_forward(x, gate, up, down, quant_types, numerics=NUM_UPSTREAM_FP16):
     """Qwen3MLP.forward (modeling_qwen3.py:214-216): down(silu(gate(x)) * up(x)), each a GGUFLinear."""
     g = gguf_linear_forward(x, gate, quant_types[0], numerics=numerics)

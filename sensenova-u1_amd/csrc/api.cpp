@@ -10,6 +10,9 @@ int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
                       hipStream_t stream);
 int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                 const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
+                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
+                        float eps);
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
 int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
@@ -163,6 +166,44 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
     if (M > 16) return SNGGUF_E_BADSHAPE;
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+}
+
+int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K) {
+    // the fused norm works on activations staged in LDS: Q8_0 rows of whole 256-element runs, M (2 K + 64) <= 16 KB
+    return qtype == SNGGUF_TYPE_Q8_0 && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
+}
+
+namespace {
+int check_rmsnorm(const void* x, int64_t M, const void* gamma, float eps, const void* q, int qtype, int64_t N, int64_t K,
+                  const void* y, int numerics) {
+    const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    if (qtype != SNGGUF_TYPE_Q8_0) return SNGGUF_E_BADTYPE;
+    if (!(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
+    if (M == 0 || N == 0) return SNGGUF_OK;
+    if (!sngguf_rmsnorm_fits(qtype, M, K)) return SNGGUF_E_BADSHAPE;
+    if (!gamma) return SNGGUF_E_NULLPTR;
+    if (!aligned(gamma, 16)) return SNGGUF_E_ALIGN;
+    return SNGGUF_OK;
+}
+}  // namespace
+
+int sngguf_rmsnorm_linear(const void* x, int64_t M, const void* gamma, float eps, const void* q, int qtype, int64_t N,
+                          int64_t K, const void* bias, void* y, int numerics, void* stream) {
+    const int rc = check_rmsnorm(x, M, gamma, eps, q, qtype, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    return sngguf::launch_gemv_q8_mfma(x, M, q, nullptr, N, K, bias, nullptr, y, numerics, false,
+                                       static_cast<hipStream_t>(stream), gamma, eps);
+}
+
+int sngguf_rmsnorm_gate_up_silu(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate,
+                                const void* q_up, int qtype, int64_t N, int64_t K, void* h, int numerics, void* stream) {
+    const int rc = check_rmsnorm(x, M, gamma, eps, q_gate, qtype, N, K, h, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (!q_up) return SNGGUF_E_NULLPTR;
+    if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_gemv_q8_mfma(x, M, q_gate, q_up, N, K, nullptr, nullptr, h, numerics, true,
+                                       static_cast<hipStream_t>(stream), gamma, eps);
 }
 
 int64_t sngguf_q8_0_tiled_bytes(int64_t N, int64_t K) {

@@ -246,7 +246,8 @@ static int launch_num(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* 
 }
 
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
-                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
+                        const void* gamma = nullptr, float eps = 0.f);
 
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);

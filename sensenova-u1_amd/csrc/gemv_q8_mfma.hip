@@ -21,12 +21,46 @@
 
 namespace sngguf {
 
+// ---- RMSNorm in front of the contraction -------------------------------------------------------------
+// The decoder layers feed q / k / v and gate / up with RMSNorm(hidden) (modeling_qwen3.py:183-197, :919, :938):
+//   v = bf16(x * rsqrt(mean(x^2) + eps))   (fp32 arithmetic, one rounding)      out = bf16(gamma * v)
+// With `gamma` given, a kernel below applies it to the activations it has staged in LDS, so the norm needs no
+// launch and no buffer of its own.  Only offered where the activations are staged once per workgroup (or once
+// per wavefront share) - a few rows; applied per fragment it would cost as much vector work as the weight decode.
+__device__ __forceinline__ float sumsq_piece(u32x4_t xv) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t d = xv[i];
+        const float a = __builtin_bit_cast(float, d << 16), b = __builtin_bit_cast(float, d & 0xFFFF0000u);
+        ss += a * a;
+        ss += b * b;
+    }
+    return ss;
+}
+__device__ __forceinline__ u32x4_t rmsnorm_piece(u32x4_t xv, u32x4_t gv, float rstd) {
+    u32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t xd = xv[i], gd = gv[i];
+        const float x0 = __builtin_bit_cast(float, xd << 16), x1 = __builtin_bit_cast(float, xd & 0xFFFF0000u);
+        const float g0 = __builtin_bit_cast(float, gd << 16), g1 = __builtin_bit_cast(float, gd & 0xFFFF0000u);
+        const float v0 = bf16_to_f32(f32_to_bf16(x0 * rstd)), v1 = bf16_to_f32(f32_to_bf16(x1 * rstd));
+        o[i] = pack_bf16(g0 * v0, g1 * v1);
+    }
+    return o;
+}
+
 // CB: blocks per step.  GATED: wavefronts [0, W) work on qa (gate), [W, 2W) on qb (up).
-template <int NUM, int CB, bool GATED, int WMAX>
+// XN: RMSNorm(x) with weight `gamma` is what gets contracted.  Each wavefront stages the K range it works on
+// (all M rows) in LDS behind the slabs, the workgroup adds up the sums of squares, and every wavefront then
+// normalizes its own share in place; the B fragments come from there.
+template <int NUM, int CB, bool GATED, int WMAX, bool XN = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                             const uint8_t* __restrict__ qa,
                                                             const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                            const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
+                                                            const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
+                                                            const bf16_t* __restrict__ gamma, float eps) {
     constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
     constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
     constexpr int kPieces = 16 * kRowPieces;      // per slab
@@ -75,6 +109,11 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
     const bool has_x = r < M;
     const bf16_t* xrow = x + (int64_t)(has_x ? r : M - 1) * K + 8 * g;
     const uint8_t* lrow = slab + r * kRowStep + 8 * g;
+    // XN: this wavefront's normalized activations, [M][xrow_b bytes]; fragment (step s, block b) of row m at
+    // byte ((s - s0) CB + b) * 64 + 16 g of row m
+    const int xrow_b = XN ? ((steps + W - 1) / W) * CB * 64 + 16 : 0;
+    uint8_t* xw = lds + waves * kSlab + wave * (M * xrow_b);
+    const uint8_t* xwrow = xw + (has_x ? r : M - 1) * xrow_b + 16 * g;
 
     // One step: slab of step s is in `pre`, its activations in `xc`.  The next step's activations
     // (into `xn`) and slab (into `pre`) are requested before this step's MFMAs, so a full step of
@@ -84,8 +123,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
         for (int i = 0; i < kLoads - 1; i++) *reinterpret_cast<u32x4_t*>(slab + 16 * (lane + 64 * i)) = pre[i];
         if (tail_lane) *reinterpret_cast<u32x4_t*>(slab + 16 * (lane + 64 * (kLoads - 1))) = pre[kLoads - 1];
         if (s + 1 < s1) {
+            if constexpr (!XN) {
 #pragma unroll
-            for (int b = 0; b < CB; b++) xn[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)(s + 1) * CB + b) * 32);
+                for (int b = 0; b < CB; b++) xn[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)(s + 1) * CB + b) * 32);
+            }
             fetch(s + 1);
         }
 #pragma unroll
@@ -108,15 +149,47 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
             q8_dword_bf16<NUM>(d, q0, a0, a1);
             q8_dword_bf16<NUM>(d, q1, a2, a3);
             const u32x4_t a = {a0, a1, a2, a3};
+            u32x4_t xfrag;
+            if constexpr (XN) xfrag = *reinterpret_cast<const u32x4_t*>(xwrow + ((s - s0) * CB + b) * 64);
+            else xfrag = xc[b];
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                          __builtin_bit_cast(bf16x8_t, xc[b]), acc, 0, 0, 0);
+                                                          __builtin_bit_cast(bf16x8_t, xfrag), acc, 0, 0, 0);
         }
     };
     u32x4_t xa[CB], xb[CB];
     if (s0 < s1) {
+        if constexpr (!XN) {
 #pragma unroll
-        for (int b = 0; b < CB; b++) xa[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)s0 * CB + b) * 32);
+            for (int b = 0; b < CB; b++) xa[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)s0 * CB + b) * 32);
+        }
         fetch(s0);
+    }
+    if constexpr (XN) {
+        // the first slab is on its way; stage and normalize this wavefront's activations underneath
+        float* ssum = reinterpret_cast<float*>(lds + waves * kSlab + waves * (M * xrow_b));  // [M][waves]
+        const int pieces = (s1 - s0) * CB * 4;             // 16-byte pieces per row in this wavefront's K range
+        const int64_t k0 = (int64_t)s0 * CB * 32;
+        for (int m = 0; m < M; m++) {
+            float ss = 0.f;
+            for (int c = lane; c < pieces; c += 64) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + k0 + 8 * c);
+                *reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * c) = v;
+                ss += sumsq_piece(v);
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) ssum[m * waves + wave] = ss;
+        }
+        __syncthreads();
+        for (int m = 0; m < M; m++) {
+            float tot = 0.f;
+            for (int w = 0; w < W; w++) tot += ssum[m * waves + w];   // wavefronts [0, W) cover K once
+            const float rstd = rsqrtf(tot / (float)K + eps);
+            for (int c = lane; c < pieces; c += 64) {
+                u32x4_t* cell = reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * c);
+                const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + k0 + 8 * c);
+                *cell = rmsnorm_piece(*cell, gv, rstd);
+            }
+        }
     }
     for (int s = s0; s < s1; s += 2) {
         step(s, xa, xb);
@@ -191,7 +264,8 @@ template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
+                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
+                                                                 const bf16_t* __restrict__ gamma, float eps) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
@@ -276,9 +350,36 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
             fetch2(t0, 1, pb);
         }
         const int pieces_per_row = (int)(K >> 3);  // 16-byte pieces
-        for (int f = tid; f < M * pieces_per_row; f += blockDim.x) {
-            const int m = f / pieces_per_row, c = f - m * pieces_per_row;
-            *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + 8 * c);
+        if (gamma == nullptr) {
+            for (int f = tid; f < M * pieces_per_row; f += blockDim.x) {
+                const int m = f / pieces_per_row, c = f - m * pieces_per_row;
+                *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + 8 * c);
+            }
+        } else {
+            // RMSNorm(x) is what gets contracted: stage the rows, add up their squares over the workgroup, then
+            // every thread normalizes the pieces it staged
+            float* ssum = reinterpret_cast<float*>(xs + M * xs_stride);   // [M][waves]
+            for (int m = 0; m < M; m++) {
+                float ss = 0.f;
+                for (int c = tid; c < pieces_per_row; c += blockDim.x) {
+                    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + 8 * c);
+                    *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = v;
+                    ss += sumsq_piece(v);
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) ssum[m * waves + wave] = ss;
+            }
+            __syncthreads();
+            for (int m = 0; m < M; m++) {
+                float tot = 0.f;
+                for (int w = 0; w < waves; w++) tot += ssum[m * waves + w];
+                const float rstd = rsqrtf(tot / (float)K + eps);
+                for (int c = tid; c < pieces_per_row; c += blockDim.x) {
+                    u32x4_t* cell = reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c);
+                    const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + 8 * c);
+                    *cell = rmsnorm_piece(*cell, gv, rstd);
+                }
+            }
         }
         __syncthreads();
     } else if (t0 < t1) {
@@ -409,7 +510,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 
 template <int NUM>
 static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                       const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+                       const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
+                       hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int spans = (int)(K >> 11);
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
@@ -424,7 +526,8 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     const bool paired = gated && !xlds && M >= kPairedMinM;
     const int waves = (gated && !paired) ? 2 * w : w;
     const size_t ring_bytes = (size_t)(gated ? 2 * w : w) * 16 * kRingRow;
-    const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0);
+    if (gamma && !xlds) return SNGGUF_E_BADSHAPE;   // the norm is applied to activations staged in LDS
+    const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0) + (gamma ? (((size_t)4 * M * waves + 15) & ~(size_t)15) : 0);
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     // the rings of 8 wavefronts plus staged activations can exceed the default dynamic-LDS limit:
     // raise it once per kernel instance
@@ -434,7 +537,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL>), \
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
-        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y); \
+        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps); \
     } while (0)
 #define SNGGUF_LAUNCH(G, WM) \
     do { \
@@ -446,7 +549,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, true, 4, false, true>),
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
-        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y);
+        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f);
     } else if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
@@ -473,15 +576,33 @@ static int pick_k_split(int64_t groups, int steps, bool gated) {
 
 template <int NUM, int CB>
 static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
+                     hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int steps = (int)(K / (32 * CB));
     const int w = pick_k_split(groups, steps, gated);
     const int waves = gated ? 2 * w : w;
-    const size_t lds_bytes = (size_t)waves * 16 * CB * 34;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
+    if (gamma) {
+        // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares;
+        // the caller keeps M (2 K + 64) within 16 KB, so this stays below the default dynamic-LDS limit
+        const size_t xrow_b = (size_t)((steps + w - 1) / w) * CB * 64 + 16;
+        const size_t lds_norm = (size_t)waves * 16 * CB * 34 + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
+        if (lds_norm > 64 * 1024) return SNGGUF_E_BADSHAPE;
+#define SNGGUF_LAUNCH_XN(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps)
+        if (gated) {
+            if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
+            else SNGGUF_LAUNCH_XN(true, 8);
+        } else {
+            if (waves <= 4) SNGGUF_LAUNCH_XN(false, 4);
+            else SNGGUF_LAUNCH_XN(false, 8);
+        }
+#undef SNGGUF_LAUNCH_XN
+        return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+    }
+    const size_t lds_bytes = (size_t)waves * 16 * CB * 34;
     // WMAX only sets the register budget the compiler may assume for the workgroup size
-#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y)
+#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f)
     if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
@@ -495,27 +616,31 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 
 template <int NUM>
 static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
-                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+                     const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
+                     hipStream_t stream) {
     // The line-aligned variant needs whole 2048-element spans per wavefront; with few row groups
     // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
     // every 256 elements) is the better fit.
     const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
     if (K % 2048 == 0 && span_waves >= 2048)
-        return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
-    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
+        return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
+    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
 }
 
-// Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).
+// Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).  `gamma` (K bf16, 16-byte
+// aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
-                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
+                        const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
+                        float eps) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
     const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
+    const bf16_t* gp = static_cast<const bf16_t*>(gamma);
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
     return SNGGUF_E_BADTYPE;
 }
 

@@ -19,7 +19,7 @@ import torch
 from torch import nn
 
 from . import ops
-from .quantized_linear import GGUFLinear
+from .quantized_linear import GGUFLinear, rms_norm
 
 MOT_GEN_SUFFIX = "_mot_gen"
 
@@ -117,18 +117,34 @@ class FusedProjections(nn.Module):
             for mod in projections:
                 mod.weight.data = torch.empty((0, mod.weight.shape[-1]), dtype=torch.uint8, device=mod.weight.device)
 
-    def forward(self, x: torch.Tensor):
-        return torch.split(self.fused(x), self.splits, dim=-1)
+    def forward(self, x: torch.Tensor, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6):
+        """With ``norm_weight`` the projections read ``RMSNorm(x)`` (``GGUFLinear.forward_normed``): for the q / k / v
+        stack that is ``input_layernorm`` (``modeling_qwen3.py:919``), folded into the same launch at decode."""
+        y = self.fused(x) if norm_weight is None else self.fused.forward_normed(x, norm_weight, eps)
+        return torch.split(y, self.splits, dim=-1)
 
 
-def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_proj: GGUFLinear) -> torch.Tensor:
+def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_proj: GGUFLinear,
+              norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:
     """``down_proj(silu(gate_proj(x)) * up_proj(x))`` (``Qwen3MLP.forward``, modeling_qwen3.py:214-216).
 
     For decode (at most 16 rows, same quant type on gate and up, no bias) the gate and up
-    projections and the SiLU product run as one fused GEMV launch."""
+    projections and the SiLU product run as one fused GEMV launch.  With ``norm_weight`` the MLP reads
+    ``RMSNorm(x)`` (``post_attention_layernorm``, modeling_qwen3.py:938); where ``ops.rmsnorm_fits`` allows, the norm
+    is part of that same launch."""
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     same = int(gate_proj.weight.quant_type) == int(up_proj.weight.quant_type)
     decode = 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16
+    if norm_weight is not None:
+        if (decode and x.is_cuda and norm_weight.dtype == torch.bfloat16 and gate_proj.decode_layout == "native"
+                and ops.rmsnorm_fits(int(gate_proj.weight.quant_type), rows, gate_proj.in_features)):
+            x2d = x.reshape(-1, gate_proj.in_features)
+            h = torch.empty((*x.shape[:-1], gate_proj.out_features), dtype=torch.bfloat16, device=x.device)
+            ops.rmsnorm_gate_up_silu_into(x2d if x2d.is_contiguous() else x2d.contiguous(), norm_weight, eps,
+                                          gate_proj.weight, up_proj.weight, int(gate_proj.weight.quant_type),
+                                          h.view(-1, gate_proj.out_features), gate_proj.numerics)
+            return down_proj(h)
+        x = rms_norm(x, norm_weight, eps)
     # the tiled gated kernel has no paired mode: beyond 8 rows the GGUF-native pair kernel is the faster one
     tg = gate_proj.tiled_weight() if decode and rows <= 8 else None
     tu = up_proj.tiled_weight() if decode and tg is not None else None

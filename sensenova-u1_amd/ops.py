@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
     "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
+    "sngguf_rmsnorm_fits", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -91,6 +92,13 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_tiled.restype = ci
     lib.sngguf_gate_up_silu_tiled.argtypes = [vp, i64, vp, vp, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu_tiled.restype = ci
+    cf = ctypes.c_float
+    lib.sngguf_rmsnorm_fits.argtypes = [ci, i64, i64]
+    lib.sngguf_rmsnorm_fits.restype = ci
+    lib.sngguf_rmsnorm_linear.argtypes = [vp, i64, vp, cf, vp, ci, i64, i64, vp, vp, ci, vp]
+    lib.sngguf_rmsnorm_linear.restype = ci
+    lib.sngguf_rmsnorm_gate_up_silu.argtypes = [vp, i64, vp, cf, vp, vp, ci, i64, i64, vp, ci, vp]
+    lib.sngguf_rmsnorm_gate_up_silu.restype = ci
     # host-only GGUF container reader
     cp = ctypes.c_char_p
     lib.sngguf_file_open.argtypes = [cp, ctypes.POINTER(vp), cp, i64]
@@ -228,6 +236,34 @@ def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, q
                                                 h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
                                                 ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_gate_up_silu")
+
+
+def rmsnorm_fits(quant_type: int, m: int, k: int) -> bool:
+    """Whether the fused-norm entry points take ``m`` rows of width ``k`` for this weight type."""
+    return bool(load_library().sngguf_rmsnorm_fits(quant_type, m, k))
+
+
+def rmsnorm_linear_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, packed: torch.Tensor, quant_type: int,
+                        bias: Optional[torch.Tensor], y2d: torch.Tensor, numerics: int) -> None:
+    """y2d[M, N] = RMSNorm(x2d; gamma, eps) @ W^T (+ bias), the norm of Qwen3RMSNorm
+    (modeling_qwen3.py:192-197) applied inside the projection kernel; shapes as ``rmsnorm_fits`` allows."""
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_rmsnorm_linear(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(packed), quant_type,
+                                                  y2d.shape[1], x2d.shape[1], _ptr(bias), _ptr(y2d), numerics,
+                                                  ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_rmsnorm_linear")
+
+
+def rmsnorm_gate_up_silu_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, gate: torch.Tensor, up: torch.Tensor,
+                              quant_type: int, h2d: torch.Tensor, numerics: int) -> None:
+    """h2d = silu(n @ Wg^T) * (n @ Wu^T) with n = RMSNorm(x2d; gamma, eps), in one launch."""
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_rmsnorm_gate_up_silu(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(gate), _ptr(up),
+                                                        quant_type, h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
+                                                        ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_rmsnorm_gate_up_silu")
 
 
 def grouped_linear_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, y2d,

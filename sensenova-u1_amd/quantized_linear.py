@@ -123,6 +123,14 @@ def dequantize_gguf_tensor(tensor: torch.Tensor, dtype: Optional[torch.dtype] = 
     return ops.dequantize(tensor, int(tensor.quant_type), dtype, numerics)
 
 
+def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMSNorm as the decoder layers compute it (``Qwen3RMSNorm.forward``, ``modeling_qwen3.py:192-197``): statistic
+    and scaling in fp32, one rounding to the input dtype, then the product with the weight in that dtype."""
+    h = hidden_states.float()
+    h = h * torch.rsqrt(h.square().mean(dim=-1, keepdim=True) + eps)
+    return weight * h.to(hidden_states.dtype)
+
+
 class GGUFLinear(nn.Linear):
     """``nn.Linear`` whose weight is a :class:`GGUFParameter`.
 
@@ -218,6 +226,24 @@ class GGUFLinear(nn.Linear):
                                 else torch.float32, self.numerics).to(compute_dtype)
         bias = self.bias.to(compute_dtype) if self.bias is not None else None
         return torch.nn.functional.linear(inputs, weight, bias)
+
+    def forward_normed(self, inputs: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> torch.Tensor:
+        """``self(RMSNorm(inputs))`` with the norm of the decoder layers (``Qwen3RMSNorm``,
+        ``modeling_qwen3.py:192-197``; it feeds q / k / v at ``:919`` and the MLP at ``:938``).  Where the library
+        offers it (Q8_0, a decode-sized input: ``ops.rmsnorm_fits``) the norm runs inside the projection kernel on
+        the activations staged in LDS; otherwise as torch operations in front of ``forward``."""
+        rows = inputs.numel() // self.in_features if inputs.numel() else 0
+        fused = (inputs.is_cuda and rows > 0 and inputs.dtype == torch.bfloat16 and norm_weight.dtype == torch.bfloat16
+                 and (self.compute_dtype or inputs.dtype) == torch.bfloat16 and self.decode_layout == "native"
+                 and ops.rmsnorm_fits(int(self.weight.quant_type), rows, self.in_features))
+        if not fused:
+            return self.forward(rms_norm(inputs, norm_weight, eps))
+        x2d = inputs.reshape(-1, self.in_features)
+        out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
+        bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
+        ops.rmsnorm_linear_into(x2d if x2d.is_contiguous() else x2d.contiguous(), norm_weight.contiguous(), eps, self.weight,
+                                self._weight_type(), bias, out.view(-1, self.out_features), self.numerics)
+        return out
 
     def forward_residual(self, inputs: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
         """``residual + self(inputs)`` (the decoder layer's ``hidden_states = residual + o_proj(...)`` /

@@ -271,3 +271,38 @@ def test_mlp_forward_under_hip_graph(tmp_path, dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_y, want)
+
+
+def test_fused_rmsnorm_through_the_module_helpers(dev):
+    """FusedProjections / gated_mlp with a norm weight: one decode row takes the fused-norm kernels, more rows (or a
+    K-quant) the torch norm in front of the projection; both agree with the oracle's norm + projection."""
+    from sensenova_u1_amd import FusedProjections, gated_mlp
+    from sensenova_u1_amd.quantized_linear import rms_norm
+    k, eps = 2048, 1e-6
+    gamma = (torch.rand(k, generator=torch.Generator().manual_seed(3)) + 0.5).to(torch.bfloat16)
+
+    def lin(n, kk, qt, seed):
+        mod = GGUFLinear(kk, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+        mod.weight = GGUFParameter(synthetic.make_packed(qt, n, kk, seed=seed).to(dev), quant_type=qt)
+        return mod
+
+    for qt in (go.Q8_0, go.Q4_K):
+        q, kp, v = lin(512, k, qt, 1), lin(128, k, qt, 2), lin(128, k, qt, 3)
+        stack = FusedProjections([q, kp, v])
+        gate, up, down = lin(1024, k, qt, 4), lin(1024, k, qt, 5), lin(k, 1024, qt, 6)
+        for rows in (1, 5):
+            print(f"case module_rmsnorm qt={qt} rows={rows}", flush=True)
+            x = (synthetic.make_activations(rows, k, seed=10 + rows).float() * 2.0).to(torch.bfloat16)
+            normed = go.qwen3_rms_norm(x, gamma, eps)
+            # the package's own torch norm (the unfused route) against the oracle's: the reduction order on the device can
+            # move a near-tie by one bf16 step
+            dn = (rms_norm(x.to(dev), gamma.to(dev), eps).cpu().float() - normed.float()).abs()
+            assert float((dn > 0).float().mean()) < 0.01 and bool((dn <= normed.float().abs() * 2 ** -6).all())
+            outs = stack(x.to(dev), gamma.to(dev), eps)
+            for mod, got in zip((q, kp, v), outs):
+                want = go.gguf_linear_forward(normed, mod.weight.as_tensor().cpu(), qt)
+                assert go.rel_l2(got.cpu(), want) <= 1e-3
+            got = gated_mlp(x.to(dev), gate, up, down, gamma.to(dev), eps)
+            want, _ = go.mlp_forward(normed, gate.weight.as_tensor().cpu(), up.weight.as_tensor().cpu(),
+                                     down.weight.as_tensor().cpu(), (qt, qt, qt))
+            assert go.rel_l2(got.cpu(), want) <= 2e-3     # two chained projections

@@ -1,0 +1,101 @@
+"""GPU: RMSNorm fused in front of the decode projections (sngguf_rmsnorm_linear, sngguf_rmsnorm_gate_up_silu)
+against the oracle's norm followed by the oracle's projection, and against the library's own unfused entry points
+fed with the oracle's normalized rows."""
+import pytest
+import torch
+
+from oracle import gguf_oracle as go
+from sensenova_u1_amd import ops, synthetic
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3   # rel-L2 of the bf16 outputs
+EPS = 1e-6   # rms_norm_eps of the 8B configuration
+
+
+def _gamma(k, seed):
+    return (torch.rand(k, generator=torch.Generator().manual_seed(seed)) * 1.5 + 0.25).to(torch.bfloat16)
+
+
+# (m, n, k): the stacked q|k|v and single projections (block-aligned kernel), the lm_head-like wide matrix
+# (line-aligned kernel), small K with several rows, N not a multiple of 16
+LINEAR_SHAPES = [(1, 6144, 4096), (1, 4096, 4096), (1, 1024, 4096), (1, 40000, 4096), (3, 2048, 2048), (2, 1000, 2048),
+                 (7, 530, 512), (16, 64, 256), (1, 37, 256), (1, 4096, 6144)]
+
+
+@pytest.mark.parametrize("numerics", [0, 1])
+@pytest.mark.parametrize("shape", LINEAR_SHAPES)
+def test_rmsnorm_linear_parity(dev, numerics, shape):
+    m, n, k = shape
+    print(f"case rmsnorm_linear m={m} n={n} k={k} numerics={numerics}", flush=True)
+    assert ops.rmsnorm_fits(go.Q8_0, m, k)
+    packed = synthetic.make_packed(go.Q8_0, n, k, seed=n + k)
+    x = (synthetic.make_activations(m, k, seed=m + k).float() * 3.0).to(torch.bfloat16)   # rows off unit RMS
+    gamma = _gamma(k, k)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16) if n % 2 else None
+    normed = go.qwen3_rms_norm(x, gamma, EPS)
+    want = go.gguf_linear_forward(normed, packed, go.Q8_0, bias, numerics=numerics)
+    pd = packed.to(dev)
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.rmsnorm_linear_into(x.to(dev), gamma.to(dev), EPS, pd, go.Q8_0, bias.to(dev) if bias is not None else None, y, numerics)
+    assert bool(torch.isfinite(y.float()).all())
+    assert go.rel_l2(y.cpu(), want) <= TOL
+    # against the unfused kernel on the oracle's normalized rows: the same weights and rounding chain; what differs is
+    # the summation order and, rarely, one bf16 step in a normalized value
+    unfused = ops.linear(normed.to(dev), pd, go.Q8_0, bias.to(dev) if bias is not None else None, numerics)
+    assert go.rel_l2(y.cpu(), unfused.cpu()) <= 5e-4
+
+
+@pytest.mark.parametrize("shape", [(1, 12288, 4096), (1, 1000, 4096), (3, 4096, 2048), (2, 48, 256), (1, 12288, 6144)])
+def test_rmsnorm_gate_up_silu_parity(dev, c_oracle, shape):
+    m, n, k = shape
+    print(f"case rmsnorm_gate_up m={m} n={n} k={k}", flush=True)
+    gate = synthetic.make_packed(go.Q8_0, n, k, seed=81)
+    up = synthetic.make_packed(go.Q8_0, n, k, seed=82)
+    x = (synthetic.make_activations(m, k, seed=83 + m).float() * 0.3).to(torch.bfloat16)
+    gamma = _gamma(k, 84)
+    normed = go.qwen3_rms_norm(x, gamma, EPS)
+    g = go.gguf_linear_forward(normed, gate, go.Q8_0)
+    u = go.gguf_linear_forward(normed, up, go.Q8_0)
+    h = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.rmsnorm_gate_up_silu_into(x.to(dev), gamma.to(dev), EPS, gate.to(dev), up.to(dev), go.Q8_0, h, 1)
+    assert bool(torch.isfinite(h.float()).all())
+    assert go.rel_l2(h.cpu(), torch.nn.functional.silu(g) * u) <= TOL
+    assert go.rel_l2(h.cpu(), c_oracle.silu_mul(g, u)) <= TOL
+
+
+def test_normalized_rows_match_the_oracle_elementwise(dev):
+    """An identity-like weight (scale 1.0, one quant of 1 per row) makes the projection return the normalized row itself:
+    every element must equal the oracle's, up to one bf16 step in the rare near-tie of the first rounding."""
+    for m, k in [(1, 4096), (3, 2048), (1, 256)]:
+        print(f"case rmsnorm_identity m={m} k={k}", flush=True)
+        blocks = torch.zeros((k, k // 32, 34), dtype=torch.uint8)
+        blocks[:, :, 0:2] = torch.tensor([0x00, 0x3C], dtype=torch.uint8)     # fp16 1.0, little-endian
+        idx = torch.arange(k)
+        blocks[idx, idx // 32, 2 + idx % 32] = 1
+        packed = blocks.view(k, -1).contiguous()
+        x = (synthetic.make_activations(m, k, seed=91 + k).float() * 5.0).to(torch.bfloat16)
+        gamma = _gamma(k, 92)
+        want = go.qwen3_rms_norm(x, gamma, EPS)
+        y = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+        ops.rmsnorm_linear_into(x.to(dev), gamma.to(dev), EPS, packed.to(dev), go.Q8_0, None, y, 1)
+        diff = (y.cpu().float() - want.float()).abs()
+        assert float((diff > 0).float().mean()) < 0.01
+        assert bool((diff <= want.float().abs() * 2 ** -6 + 1e-30).all())
+
+
+def test_rmsnorm_argument_errors(dev):
+    packed = synthetic.make_packed(go.Q8_0, 64, 4096, seed=1).to(dev)
+    gamma = _gamma(4096, 2).to(dev)
+    x = synthetic.make_activations(2, 4096, seed=3).to(dev)
+    y = torch.empty((2, 64), dtype=torch.bfloat16, device=dev)
+    assert not ops.rmsnorm_fits(go.Q8_0, 2, 4096)           # two rows of 4096 do not fit the staging area
+    assert not ops.rmsnorm_fits(go.Q4_K, 1, 4096)
+    with pytest.raises(ops.SnGgufError):
+        ops.rmsnorm_linear_into(x, gamma, EPS, packed, go.Q8_0, None, y, 1)
+    with pytest.raises(ops.SnGgufError):
+        ops.rmsnorm_linear_into(x[:1], None, EPS, packed, go.Q8_0, None, y[:1], 1)          # gamma required
+    k4 = synthetic.make_packed(go.Q4_K, 64, 4096, seed=4).to(dev)
+    with pytest.raises(ops.SnGgufError):
+        ops.rmsnorm_linear_into(x[:1], gamma, EPS, k4, go.Q4_K, None, y[:1], 1)             # Q8_0 only
+    with pytest.raises(ops.SnGgufError):
+        ops.rmsnorm_linear_into(x[:1], gamma, -1.0, packed, go.Q8_0, None, y[:1], 1)        # eps < 0
