@@ -317,13 +317,28 @@ def main() -> None:
             ops.rmsnorm_gate_up_silu_into(hid, gammas[1], eps, gate, up, Q8_0, h1, num)
             ops.linear_residual_into(h1, down, Q8_0, None, hid, yo, num)
 
+        # ... and on the tiled copies of all seven weights
+        t_mlp = [tuple(ops.q8_0_tile(t) for t in layer) for layer in layers]
+        t_qkv = [ops.q8_0_tile(w) for w in qkv]
+        t_o = [ops.q8_0_tile(a[3]) for a in attn]
+        torch.cuda.synchronize()
+
+        def layer_tiled_norms_fused(i):
+            ops.rmsnorm_linear_tiled_into(x1, gammas[0], eps, t_qkv[i % nl], None, yqkv, num)
+            tg, tu, td = t_mlp[i % len(layers)]
+            ops.linear_tiled_into(yq, t_o[i % nl], None, res, hid, num)
+            ops.rmsnorm_gate_up_silu_tiled_into(hid, gammas[1], eps, tg, tu, h1, num)
+            ops.linear_tiled_into(h1, td, None, hid, yo, num)
+
         k3 = max(64, K // 4)
         lbytes = (2 * linear_bytes(1, HIDDEN, HIDDEN) + 2 * linear_bytes(1, KV, HIDDEN) + mlp_bytes(1))
         legs = {}
         for name, fn, launches in (("separate", layer_separate, "6 linears + 2 adds"), ("stacked_qkv", layer_stacked, "4 linears + 2 adds"),
                                    ("stacked_qkv_fused_residual", layer_stacked_residual, "4 linears"),
                                    ("with_norms_separate", layer_norms_separate, "4 linears + 2 torch rms_norm"),
-                                   ("with_norms_fused", layer_norms_fused, "4 linears, both RMSNorms inside the q|k|v and gate/up launches")):
+                                   ("with_norms_fused", layer_norms_fused, "4 linears, both RMSNorms inside the q|k|v and gate/up launches"),
+                                   ("tiled_with_norms_fused", layer_tiled_norms_fused,
+                                    "as with_norms_fused on the operand-order (tiled) copies of the seven weights")):
             wall_l, _ = run_region(fn, k3, min(W, 16))
             legs[name] = {"launches": launches, "us_per_layer": round(wall_l / k3 * 1e3, 2),
                           "value": round(lbytes / (wall_l / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"}
@@ -332,7 +347,7 @@ def main() -> None:
                         "down) and its two residual adds; no attention; the with_norms legs add the layer's two RMSNorms",
             "bytes_per_layer": lbytes, **legs,
         }
-        del attn, qkv
+        del attn, qkv, t_mlp, t_qkv, t_o
 
     # ---- lm_head at decode: 151936 x 4096 Q8_0 (the vocabulary projection of the think loop), M = 1 ---------------
     if not args.no_extra:

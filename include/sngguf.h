@@ -172,6 +172,13 @@ int sngguf_rmsnorm_linear(const void* x, int64_t M, const void* gamma, float eps
 int sngguf_rmsnorm_gate_up_silu(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate,
                                 const void* q_up, int qtype, int64_t N, int64_t K, void* h, int numerics,
                                 void* stream);
+/* The same two on the operand-order ("tiled") copy of Q8_0 weights described below (sngguf_q8_0_tile); the size
+ * rule is sngguf_rmsnorm_fits(SNGGUF_TYPE_Q8_0, M, K). */
+int sngguf_rmsnorm_linear_tiled(const void* x, int64_t M, const void* gamma, float eps, const void* tiled,
+                                int64_t N, int64_t K, const void* bias, void* y, int numerics, void* stream);
+int sngguf_rmsnorm_gate_up_silu_tiled(const void* x, int64_t M, const void* gamma, float eps,
+                                      const void* tiled_gate, const void* tiled_up, int64_t N, int64_t K, void* h,
+                                      int numerics, void* stream);
 
 /*
  * Operand-order ("tiled") copy of a Q8_0 matrix for the decode path.  No counterpart in the reference, which keeps

@@ -16,7 +16,8 @@ int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
 int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
-                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
+                         const void* gamma = nullptr, float eps = 0.f);
 int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
                       hipStream_t stream);
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
@@ -247,6 +248,38 @@ int sngguf_gate_up_silu_tiled(const void* x, int64_t M, const void* tiled_gate, 
     if (!aligned(tiled_up, 16)) return SNGGUF_E_ALIGN;
     return sngguf::launch_gemv_q8_tiled(x, M, tiled_gate, tiled_up, N, K, nullptr, nullptr, h, numerics, true,
                                         static_cast<hipStream_t>(stream));
+}
+
+namespace {
+int check_rmsnorm_tiled(const void* x, int64_t M, const void* gamma, float eps, const void* t, int64_t N, int64_t K,
+                        const void* y, int numerics) {
+    const int rc = check_tiled(x, M, t, N, K, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    if (!(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
+    if (M == 0 || N == 0) return SNGGUF_OK;
+    if (!sngguf_rmsnorm_fits(SNGGUF_TYPE_Q8_0, M, K)) return SNGGUF_E_BADSHAPE;
+    if (!gamma) return SNGGUF_E_NULLPTR;
+    if (!aligned(gamma, 16)) return SNGGUF_E_ALIGN;
+    return SNGGUF_OK;
+}
+}  // namespace
+
+int sngguf_rmsnorm_linear_tiled(const void* x, int64_t M, const void* gamma, float eps, const void* tiled, int64_t N,
+                                int64_t K, const void* bias, void* y, int numerics, void* stream) {
+    const int rc = check_rmsnorm_tiled(x, M, gamma, eps, tiled, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    return sngguf::launch_gemv_q8_tiled(x, M, tiled, nullptr, N, K, bias, nullptr, y, numerics, false,
+                                        static_cast<hipStream_t>(stream), gamma, eps);
+}
+
+int sngguf_rmsnorm_gate_up_silu_tiled(const void* x, int64_t M, const void* gamma, float eps, const void* tiled_gate,
+                                      const void* tiled_up, int64_t N, int64_t K, void* h, int numerics, void* stream) {
+    const int rc = check_rmsnorm_tiled(x, M, gamma, eps, tiled_gate, N, K, h, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (!tiled_up) return SNGGUF_E_NULLPTR;
+    if (!aligned(tiled_up, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_gemv_q8_tiled(x, M, tiled_gate, tiled_up, N, K, nullptr, nullptr, h, numerics, true,
+                                        static_cast<hipStream_t>(stream), gamma, eps);
 }
 
 int64_t sngguf_grouped_workspace_bytes(int64_t M) { return sngguf::grouped_workspace_bytes(M); }

@@ -21,36 +21,6 @@
 
 namespace sngguf {
 
-// ---- RMSNorm in front of the contraction -------------------------------------------------------------
-// The decoder layers feed q / k / v and gate / up with RMSNorm(hidden) (modeling_qwen3.py:183-197, :919, :938):
-//   v = bf16(x * rsqrt(mean(x^2) + eps))   (fp32 arithmetic, one rounding)      out = bf16(gamma * v)
-// With `gamma` given, a kernel below applies it to the activations it has staged in LDS, so the norm needs no
-// launch and no buffer of its own.  Only offered where the activations are staged once per workgroup (or once
-// per wavefront share) - a few rows; applied per fragment it would cost as much vector work as the weight decode.
-__device__ __forceinline__ float sumsq_piece(u32x4_t xv) {
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t d = xv[i];
-        const float a = __builtin_bit_cast(float, d << 16), b = __builtin_bit_cast(float, d & 0xFFFF0000u);
-        ss += a * a;
-        ss += b * b;
-    }
-    return ss;
-}
-__device__ __forceinline__ u32x4_t rmsnorm_piece(u32x4_t xv, u32x4_t gv, float rstd) {
-    u32x4_t o;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t xd = xv[i], gd = gv[i];
-        const float x0 = __builtin_bit_cast(float, xd << 16), x1 = __builtin_bit_cast(float, xd & 0xFFFF0000u);
-        const float g0 = __builtin_bit_cast(float, gd << 16), g1 = __builtin_bit_cast(float, gd & 0xFFFF0000u);
-        const float v0 = bf16_to_f32(f32_to_bf16(x0 * rstd)), v1 = bf16_to_f32(f32_to_bf16(x1 * rstd));
-        o[i] = pack_bf16(g0 * v0, g1 * v1);
-    }
-    return o;
-}
-
 // CB: blocks per step.  GATED: wavefronts [0, W) work on qa (gate), [W, 2W) on qb (up).
 // XN: RMSNorm(x) with weight `gamma` is what gets contracted.  Each wavefront stages the K range it works on
 // (all M rows) in LDS behind the slabs, the workgroup adds up the sums of squares, and every wavefront then

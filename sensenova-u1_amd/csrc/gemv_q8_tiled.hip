@@ -52,7 +52,8 @@ template <int NUM, bool GATED, int WMAX, bool XLDS>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* __restrict__ x, int M,
                                                                   const uint8_t* __restrict__ ta, const uint8_t* __restrict__ tb,
                                                                   int64_t N, int64_t K, const bf16_t* __restrict__ bias,
-                                                                  const bf16_t* residual, bf16_t* __restrict__ y) {
+                                                                  const bf16_t* residual, bf16_t* __restrict__ y,
+                                                                  const bf16_t* __restrict__ gamma, float eps) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
@@ -87,9 +88,36 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     if (r0 < r1) fetch(r0, 0);   // the weights are requested before the activations are staged
     if constexpr (XLDS) {
         const int pieces_per_row = (int)(K >> 3);
-        for (int m = 0; m < M; m++)
-            for (int c = tid; c < pieces_per_row; c += (int)blockDim.x)
-                *reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (uint32_t)(m * (int)K + 8 * c));
+        if (gamma == nullptr) {
+            for (int m = 0; m < M; m++)
+                for (int c = tid; c < pieces_per_row; c += (int)blockDim.x)
+                    *reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (uint32_t)(m * (int)K + 8 * c));
+        } else {
+            // RMSNorm(x) with weight gamma is what gets contracted (see rmsnorm_piece): stage the rows, add up their
+            // squares over the workgroup, then every thread normalizes the pieces it staged
+            float* ssum = reinterpret_cast<float*>(lds + M * xs_stride);   // [M][waves]
+            for (int m = 0; m < M; m++) {
+                float ss = 0.f;
+                for (int c = tid; c < pieces_per_row; c += (int)blockDim.x) {
+                    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (uint32_t)(m * (int)K + 8 * c));
+                    *reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c) = v;
+                    ss += sumsq_piece(v);
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) ssum[m * waves + wave] = ss;
+            }
+            __syncthreads();
+            for (int m = 0; m < M; m++) {
+                float tot = 0.f;
+                for (int w = 0; w < waves; w++) tot += ssum[m * waves + w];
+                const float rstd = rsqrtf(tot / (float)K + eps);
+                for (int c = tid; c < pieces_per_row; c += (int)blockDim.x) {
+                    u32x4_t* cell = reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c);
+                    const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + 8 * c);
+                    *cell = rmsnorm_piece(*cell, gv, rstd);
+                }
+            }
+        }
         __syncthreads();
     }
 
@@ -167,7 +195,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
 
 template <int NUM>
 int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, int64_t N, int64_t K, const bf16_t* bias,
-                 const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+                 const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int runs = (int)(K >> 8);
     // wavefronts per matrix and row group: measured best at 8 (4 for the gated pair, which doubles them); fewer when
@@ -179,9 +207,11 @@ int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, i
     const size_t x_bytes = (size_t)M * (2 * K + 64);
     const bool xlds = x_bytes <= 16 * 1024;
     const size_t red_bytes = (size_t)waves * 1024;
-    const size_t lds_bytes = xlds && x_bytes > red_bytes ? x_bytes : red_bytes;
+    if (gamma && !xlds) return SNGGUF_E_BADSHAPE;   // the norm is applied to activations staged in LDS
+    const size_t stage_bytes = x_bytes + (gamma ? (((size_t)4 * M * waves + 15) & ~(size_t)15) : 0);
+    const size_t lds_bytes = xlds && stage_bytes > red_bytes ? stage_bytes : red_bytes;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
-#define SNGGUF_LAUNCH(G, XL) gemv_q8_tiled_kernel<NUM, G, 8, XL><<<grid, block, lds_bytes, stream>>>(x, M, ta, tb, N, K, bias, residual, y)
+#define SNGGUF_LAUNCH(G, XL) gemv_q8_tiled_kernel<NUM, G, 8, XL><<<grid, block, lds_bytes, stream>>>(x, M, ta, tb, N, K, bias, residual, y, gamma, eps)
     if (gated) {
         if (xlds) SNGGUF_LAUNCH(true, true);
         else SNGGUF_LAUNCH(true, false);
@@ -211,16 +241,19 @@ int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream
 }
 
 // 1 <= M <= 16, K % 256 == 0, 16-byte aligned pointers (checked by the caller).
+// `gamma` (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
-                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
+                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
+                         float eps) {
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(ta);
     const uint8_t* b = static_cast<const uint8_t*>(tb);
     const bf16_t* bp = static_cast<const bf16_t*>(bias);
     const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_tiled<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_tiled<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);
+    const bf16_t* gp = static_cast<const bf16_t*>(gamma);
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_tiled<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_tiled<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
     return SNGGUF_E_BADTYPE;
 }
 

@@ -136,13 +136,19 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     same = int(gate_proj.weight.quant_type) == int(up_proj.weight.quant_type)
     decode = 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16
     if norm_weight is not None:
-        if (decode and x.is_cuda and norm_weight.dtype == torch.bfloat16 and gate_proj.decode_layout == "native"
+        if (decode and x.is_cuda and norm_weight.dtype == torch.bfloat16
                 and ops.rmsnorm_fits(int(gate_proj.weight.quant_type), rows, gate_proj.in_features)):
             x2d = x.reshape(-1, gate_proj.in_features)
+            x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
             h = torch.empty((*x.shape[:-1], gate_proj.out_features), dtype=torch.bfloat16, device=x.device)
-            ops.rmsnorm_gate_up_silu_into(x2d if x2d.is_contiguous() else x2d.contiguous(), norm_weight, eps,
-                                          gate_proj.weight, up_proj.weight, int(gate_proj.weight.quant_type),
-                                          h.view(-1, gate_proj.out_features), gate_proj.numerics)
+            tg, tu = gate_proj.tiled_weight(), up_proj.tiled_weight()
+            if tg is not None and tu is not None:
+                ops.rmsnorm_gate_up_silu_tiled_into(x2d, norm_weight.contiguous(), eps, tg, tu,
+                                                    h.view(-1, gate_proj.out_features), gate_proj.numerics)
+            else:
+                ops.rmsnorm_gate_up_silu_into(x2d, norm_weight.contiguous(), eps, gate_proj.weight, up_proj.weight,
+                                              int(gate_proj.weight.quant_type), h.view(-1, gate_proj.out_features),
+                                              gate_proj.numerics)
             return down_proj(h)
         x = rms_norm(x, norm_weight, eps)
     # the tiled gated kernel has no paired mode: beyond 8 rows the GGUF-native pair kernel is the faster one

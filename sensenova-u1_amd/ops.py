@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_rmsnorm_fits", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
+    "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -99,6 +100,10 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_rmsnorm_linear.restype = ci
     lib.sngguf_rmsnorm_gate_up_silu.argtypes = [vp, i64, vp, cf, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_rmsnorm_gate_up_silu.restype = ci
+    lib.sngguf_rmsnorm_linear_tiled.argtypes = [vp, i64, vp, cf, vp, i64, i64, vp, vp, ci, vp]
+    lib.sngguf_rmsnorm_linear_tiled.restype = ci
+    lib.sngguf_rmsnorm_gate_up_silu_tiled.argtypes = [vp, i64, vp, cf, vp, vp, i64, i64, vp, ci, vp]
+    lib.sngguf_rmsnorm_gate_up_silu_tiled.restype = ci
     # host-only GGUF container reader
     cp = ctypes.c_char_p
     lib.sngguf_file_open.argtypes = [cp, ctypes.POINTER(vp), cp, i64]
@@ -264,6 +269,28 @@ def rmsnorm_gate_up_silu_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float
                                                         quant_type, h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
                                                         ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_rmsnorm_gate_up_silu")
+
+
+def rmsnorm_linear_tiled_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, tiled: torch.Tensor,
+                              bias: Optional[torch.Tensor], y2d: torch.Tensor, numerics: int) -> None:
+    """``rmsnorm_linear_into`` with W given as its tiled copy."""
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_rmsnorm_linear_tiled(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(tiled),
+                                                        y2d.shape[1], x2d.shape[1], _ptr(bias), _ptr(y2d), numerics,
+                                                        ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_rmsnorm_linear_tiled")
+
+
+def rmsnorm_gate_up_silu_tiled_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, tiled_gate: torch.Tensor,
+                                    tiled_up: torch.Tensor, h2d: torch.Tensor, numerics: int) -> None:
+    """``rmsnorm_gate_up_silu_into`` on two tiled matrices."""
+    dev = x2d.device
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_rmsnorm_gate_up_silu_tiled(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(tiled_gate),
+                                                              _ptr(tiled_up), h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
+                                                              ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_rmsnorm_gate_up_silu_tiled")
 
 
 def grouped_linear_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, y2d,

@@ -234,15 +234,21 @@ class GGUFLinear(nn.Linear):
         the activations staged in LDS; otherwise as torch operations in front of ``forward``."""
         rows = inputs.numel() // self.in_features if inputs.numel() else 0
         fused = (inputs.is_cuda and rows > 0 and inputs.dtype == torch.bfloat16 and norm_weight.dtype == torch.bfloat16
-                 and (self.compute_dtype or inputs.dtype) == torch.bfloat16 and self.decode_layout == "native"
+                 and (self.compute_dtype or inputs.dtype) == torch.bfloat16
                  and ops.rmsnorm_fits(int(self.weight.quant_type), rows, self.in_features))
         if not fused:
             return self.forward(rms_norm(inputs, norm_weight, eps))
         x2d = inputs.reshape(-1, self.in_features)
+        x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
         out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
         bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
-        ops.rmsnorm_linear_into(x2d if x2d.is_contiguous() else x2d.contiguous(), norm_weight.contiguous(), eps, self.weight,
-                                self._weight_type(), bias, out.view(-1, self.out_features), self.numerics)
+        tiled = self.tiled_weight() if self.decode_layout != "native" else None
+        if tiled is not None:
+            ops.rmsnorm_linear_tiled_into(x2d, norm_weight.contiguous(), eps, tiled, bias, out.view(-1, self.out_features),
+                                          self.numerics)
+        else:
+            ops.rmsnorm_linear_into(x2d, norm_weight.contiguous(), eps, self.weight, self._weight_type(), bias,
+                                    out.view(-1, self.out_features), self.numerics)
         return out
 
     def forward_residual(self, inputs: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:

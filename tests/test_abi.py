@@ -101,3 +101,8 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_rmsnorm_linear(p, 0, p, eps, p, 8, 16, 256, None, p, 1, None) == 0
     assert lib.sngguf_rmsnorm_gate_up_silu(p, 1, p, eps, p, None, 8, 16, 256, p, 1, None) == E_NULL
     assert lib.sngguf_rmsnorm_gate_up_silu(p, 1, p, eps, p, p, 8, 16, 256, p, 7, None) == E_TYPE
+    assert lib.sngguf_rmsnorm_linear_tiled(p, 2, p, eps, p, 16, 4096, None, p, 1, None) == E_SHAPE
+    assert lib.sngguf_rmsnorm_linear_tiled(p, 1, None, eps, p, 16, 256, None, p, 1, None) == E_NULL
+    assert lib.sngguf_rmsnorm_linear_tiled(p, 0, p, eps, p, 16, 256, None, p, 1, None) == 0
+    assert lib.sngguf_rmsnorm_gate_up_silu_tiled(p, 1, p, eps, p, None, 16, 256, p, 1, None) == E_NULL
+    assert lib.sngguf_rmsnorm_gate_up_silu_tiled(p, 1, odd, eps, p, p, 16, 256, p, 1, None) == E_ALIGN

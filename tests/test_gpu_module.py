@@ -286,12 +286,14 @@ def test_fused_rmsnorm_through_the_module_helpers(dev):
         mod.weight = GGUFParameter(synthetic.make_packed(qt, n, kk, seed=seed).to(dev), quant_type=qt)
         return mod
 
-    for qt in (go.Q8_0, go.Q4_K):
+    for qt, layout in ((go.Q8_0, "native"), (go.Q4_K, "native"), (go.Q8_0, "tiled")):
         q, kp, v = lin(512, k, qt, 1), lin(128, k, qt, 2), lin(128, k, qt, 3)
         stack = FusedProjections([q, kp, v])
         gate, up, down = lin(1024, k, qt, 4), lin(1024, k, qt, 5), lin(k, 1024, qt, 6)
+        for mod in (stack.fused, gate, up, down):
+            mod.decode_layout = layout
         for rows in (1, 5):
-            print(f"case module_rmsnorm qt={qt} rows={rows}", flush=True)
+            print(f"case module_rmsnorm qt={qt} layout={layout} rows={rows}", flush=True)
             x = (synthetic.make_activations(rows, k, seed=10 + rows).float() * 2.0).to(torch.bfloat16)
             normed = go.qwen3_rms_norm(x, gamma, eps)
             # the package's own torch norm (the unfused route) against the oracle's: the reduction order on the device can

@@ -99,3 +99,35 @@ def test_rmsnorm_argument_errors(dev):
         ops.rmsnorm_linear_into(x[:1], gamma, EPS, k4, go.Q4_K, None, y[:1], 1)             # Q8_0 only
     with pytest.raises(ops.SnGgufError):
         ops.rmsnorm_linear_into(x[:1], gamma, -1.0, packed, go.Q8_0, None, y[:1], 1)        # eps < 0
+
+
+@pytest.mark.parametrize("shape", [(1, 6144, 4096), (1, 1030, 4096), (3, 2048, 2048), (5, 37, 256)])
+def test_rmsnorm_tiled_parity(dev, c_oracle, shape):
+    """The same fusion on the operand-order copy of the weights: linear (with bias) and the gated pair."""
+    m, n, k = shape
+    print(f"case rmsnorm_tiled m={m} n={n} k={k}", flush=True)
+    gate = synthetic.make_packed(go.Q8_0, n, k, seed=101)
+    up = synthetic.make_packed(go.Q8_0, n, k, seed=102)
+    x = (synthetic.make_activations(m, k, seed=103 + m).float() * 1.7).to(torch.bfloat16)
+    gamma = _gamma(k, 104)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16)
+    normed = go.qwen3_rms_norm(x, gamma, EPS)
+    tg, tu = ops.q8_0_tile(gate.to(dev)), ops.q8_0_tile(up.to(dev))
+    for numerics in (0, 1):
+        want = go.gguf_linear_forward(normed, gate, go.Q8_0, bias, numerics=numerics)
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.rmsnorm_linear_tiled_into(x.to(dev), gamma.to(dev), EPS, tg, bias.to(dev), y, numerics)
+        assert go.rel_l2(y.cpu(), want) <= TOL
+    g = go.gguf_linear_forward(normed, gate, go.Q8_0)
+    u = go.gguf_linear_forward(normed, up, go.Q8_0)
+    h = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.rmsnorm_gate_up_silu_tiled_into(x.to(dev), gamma.to(dev), EPS, tg, tu, h, 1)
+    assert go.rel_l2(h.cpu(), c_oracle.silu_mul(g, u)) <= TOL
+    # the fused norm of the two layouts works on the same staged rows: same normalized values, another summation order
+    h_native = torch.empty_like(h)
+    ops.rmsnorm_gate_up_silu_into(x.to(dev), gamma.to(dev), EPS, gate.to(dev), up.to(dev), go.Q8_0, h_native, 1)
+    assert go.rel_l2(h.cpu(), h_native.cpu()) <= 5e-4
+    if 16 * (2 * k + 64) > 16384:      # sixteen rows of this width do not fit the staging area
+        big = synthetic.make_activations(16, k, seed=1).to(dev)
+        with pytest.raises(ops.SnGgufError):
+            ops.rmsnorm_linear_tiled_into(big, gamma.to(dev), EPS, tg, None, torch.empty((16, n), dtype=torch.bfloat16, device=dev), 1)
