@@ -129,8 +129,7 @@ int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, i
  * materialises the dequantized weight on every call (diffusers GGUFLinear.forward_native, reached from
  * src/sensenova_u1/utils/gguf_loader.py:64-81): this is that route for callers of the bare ABI.  With
  * workspace (device memory, 16-byte aligned) of at least sngguf_linear_workspace_bytes(N, K) = 2 N K bytes
- * and a problem large enough for it (M >= 384, K % 64 == 0, M K < 2^31, at least 128 tiles of 256 x 256
- * outputs) the weights are decoded once into the workspace as bf16 - the same values, same rounding chain,
+ * and a problem it fits (M >= 65, K % 64 == 0, M K < 2^31) the weights are decoded once into the workspace as bf16 - the same values, same rounding chain,
  * as the fused kernels decode on the fly - and a dense bf16 tile GEMM consumes them; any of the ten types then
  * runs at the rate of that GEMM.  Otherwise (workspace NULL or too small included) it behaves exactly as
  * sngguf_linear.  The workspace holds nothing the caller needs afterwards; calls sharing one workspace must

@@ -136,9 +136,14 @@ int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, i
 }
 
 namespace {
-// The weight pass pays once the matrix work dwarfs it; the dense kernel wants whole K steps, 32-bit activation
-// offsets and enough 256 x 256 tiles to occupy the chip.
+// The dense kernel wants whole K steps and 32-bit activation offsets.  One weight pass + the dense kernel beat the
+// fused kernels from 65 rows on (measured on the four projection shapes of the 8B model, 65 ... 4096 rows); the
+// grouped form decodes two weight sets, which pays from a few hundred rows and enough tiles to occupy the chip.
 bool dense_route_fits(int64_t M, int64_t N, int64_t K) {
+    (void)N;
+    return M >= 65 && K % 64 == 0 && M * K < ((int64_t)1 << 31);
+}
+bool grouped_dense_route_fits(int64_t M, int64_t N, int64_t K) {
     return M >= 384 && K % 64 == 0 && M * K < ((int64_t)1 << 31) && ((M + 255) / 256) * ((N + 255) / 256) >= 128;
 }
 }  // namespace
@@ -305,7 +310,7 @@ int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator,
                              int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
                              const void* bias_gen, void* y, void* workspace, void* dense_workspace,
                              int64_t dense_workspace_bytes, int numerics, void* stream) {
-    const bool two_pass = dense_workspace && dense_workspace_bytes >= 4 * N * K && K > 0 && N > 0 && dense_route_fits(M, N, K);
+    const bool two_pass = dense_workspace && dense_workspace_bytes >= 4 * N * K && K > 0 && N > 0 && grouped_dense_route_fits(M, N, K);
     if (!two_pass)
         return sngguf_grouped_linear(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und, bias_gen, y,
                                      workspace, numerics, stream);
