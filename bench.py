@@ -540,6 +540,23 @@ def main() -> None:
             kq[f"mlp_M{m}"] = {"value": round(gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
                                "bytes_per_step": nbytes, "ms_per_step": round(wall / k2, 6),
                                "gate_up_us": round(gu * 1e3, 3), "down_us": round(dn * 1e3, 3)}
+        # post_attention_layernorm in front of the Q4_K gate/up pair at M = 1: one torch rms_norm launch + the pair,
+        # against the norm folded into the pair's launch
+        xk = synthetic.make_activations(1, HIDDEN, seed=21, device=dev)
+        hk = torch.empty((1, INTER), dtype=torch.bfloat16, device=dev)
+        gk = (torch.rand(HIDDEN, generator=torch.Generator().manual_seed(22)) + 0.5).to(torch.bfloat16).to(dev)
+
+        def kq_norm_separate(i):
+            nk = torch.nn.functional.rms_norm(xk, (HIDDEN,), gk, 1e-6)
+            ops.gate_up_silu_into(nk, klayers[i % L][0], klayers[i % L][1], Q4_K, hk, num)
+
+        def kq_norm_fused(i):
+            ops.rmsnorm_gate_up_silu_into(xk, gk, 1e-6, klayers[i % L][0], klayers[i % L][1], Q4_K, hk, num)
+
+        kn = max(64, K // 4)
+        wall_ns, _ = run_region(kq_norm_separate, kn, min(W, 16))
+        wall_nf, _ = run_region(kq_norm_fused, kn, min(W, 16))
+        kq["gate_up_M1_with_norm"] = {"separate_rms_norm_us": round(wall_ns / kn * 1e3, 2), "fused_us": round(wall_nf / kn * 1e3, 2)}
         del klayers
         if not args.no_gemm:
             m = 4096

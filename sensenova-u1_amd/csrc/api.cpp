@@ -13,6 +13,9 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
                         float eps);
+int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
+                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
+                        const void* gamma, float eps);
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
 int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
@@ -175,8 +178,8 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
 }
 
 int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K) {
-    // the fused norm works on activations staged in LDS: Q8_0 rows of whole 256-element runs, M (2 K + 64) <= 16 KB
-    return qtype == SNGGUF_TYPE_Q8_0 && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
+    // the fused norm works on activations staged in LDS: rows of whole 256-element runs, M (2 K + 64) <= 16 KB
+    return known_type(qtype) && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
 }
 
 namespace {
@@ -184,7 +187,6 @@ int check_rmsnorm(const void* x, int64_t M, const void* gamma, float eps, const 
                   const void* y, int numerics) {
     const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
     if (rc != SNGGUF_OK) return rc;
-    if (qtype != SNGGUF_TYPE_Q8_0) return SNGGUF_E_BADTYPE;
     if (!(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
     if (M == 0 || N == 0) return SNGGUF_OK;
     if (!sngguf_rmsnorm_fits(qtype, M, K)) return SNGGUF_E_BADSHAPE;
@@ -198,6 +200,9 @@ int sngguf_rmsnorm_linear(const void* x, int64_t M, const void* gamma, float eps
                           int64_t K, const void* bias, void* y, int numerics, void* stream) {
     const int rc = check_rmsnorm(x, M, gamma, eps, q, qtype, N, K, y, numerics);
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    if (qtype != SNGGUF_TYPE_Q8_0)
+        return sngguf::launch_gemv_kq_mfma(x, M, q, nullptr, qtype, N, K, bias, nullptr, y, numerics, false,
+                                           static_cast<hipStream_t>(stream), gamma, eps);
     return sngguf::launch_gemv_q8_mfma(x, M, q, nullptr, N, K, bias, nullptr, y, numerics, false,
                                        static_cast<hipStream_t>(stream), gamma, eps);
 }
@@ -208,6 +213,9 @@ int sngguf_rmsnorm_gate_up_silu(const void* x, int64_t M, const void* gamma, flo
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (!q_up) return SNGGUF_E_NULLPTR;
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
+    if (qtype != SNGGUF_TYPE_Q8_0)
+        return sngguf::launch_gemv_kq_mfma(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true,
+                                           static_cast<hipStream_t>(stream), gamma, eps);
     return sngguf::launch_gemv_q8_mfma(x, M, q_gate, q_up, N, K, nullptr, nullptr, h, numerics, true,
                                        static_cast<hipStream_t>(stream), gamma, eps);
 }

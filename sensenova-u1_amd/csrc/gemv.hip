@@ -250,7 +250,8 @@ int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb
                         const void* gamma = nullptr, float eps = 0.f);
 
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
+                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
+                        const void* gamma = nullptr, float eps = 0.f);
 
 // M in 1..16 (up to 64 when K % 256 == 0 and not gated), N >= 1, K a positive multiple of the block
 // size (checked by the caller).

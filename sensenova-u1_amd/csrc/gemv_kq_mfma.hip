@@ -367,11 +367,16 @@ __device__ __forceinline__ void decode_half(half4_t ident, const uint8_t* row, i
     }
 }
 
-template <int QT, int NUM, int R, bool GATED, int WMAX, int MT>
+// XN (MT = 1 only): RMSNorm(x) with weight `gamma` is what gets contracted (see rmsnorm_piece).  Each wavefront
+// stages the K range it works on (all M rows) in LDS behind the slabs, the workgroup adds up the sums of squares,
+// every wavefront normalizes its own share in place, and the B fragments come from there.
+template <int QT, int NUM, int R, bool GATED, int WMAX, int MT, bool XN = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y) {
+                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
+                                                                 const bf16_t* __restrict__ gamma, float eps) {
+    static_assert(!XN || MT == 1, "the fused norm is for at most 16 rows");
     typedef Slab<QT> S;
     constexpr int kRows = 16 * R;
     constexpr int kPieces = kRows * S::pieces;
@@ -441,12 +446,19 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     // the current super-block on entry; the second half is requested into `xb` before the first is
     // used, and the first half of the next super-block into `xa` before the second is used, so each
     // request has half a step of decode work to cover its latency.
+    // XN: this wavefront's normalized activations, [M][xrow_b bytes]; the fragment of super-block s, half, j of
+    // row m sits at byte ((s - s0) * 8 + 4 * half + j) * 64 + 16 g of row m
+    const int xrow_b = XN ? (int)((nsb + W - 1) / W) * 512 + 16 : 0;
+    uint8_t* xw = lds + waves * kSlab + wave * (M * xrow_b);
+    const uint8_t* xwrow = xw + (r < M ? r : M - 1) * xrow_b + 16 * g;
     auto load_x = [&](int s, int half, u32x4_t (&dstx)[MT][4]) {
 #pragma unroll
         for (int t = 0; t < MT; t++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                dstx[t][j] = *reinterpret_cast<const u32x4_t*>(xrow[t] + ((int64_t)s * 8 + 4 * half + j) * 32);
+            for (int j = 0; j < 4; j++) {
+                if constexpr (XN) dstx[t][j] = *reinterpret_cast<const u32x4_t*>(xwrow + ((s - s0) * 8 + 4 * half + j) * 64);
+                else dstx[t][j] = *reinterpret_cast<const u32x4_t*>(xrow[t] + ((int64_t)s * 8 + 4 * half + j) * 32);
+            }
     };
     u32x4_t xa[MT][4], xb[MT][4];
     auto step = [&](int s) {
@@ -482,7 +494,35 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
             decode_half<QT, NUM, 1>(ident, row, g, emit);
         }
     };
-    if (s0 < s1) {
+    if constexpr (XN) {
+        // the first slab is requested, then the activations are staged and normalized underneath it
+        if (s0 < s1) fetch(s0);
+        float* ssum = reinterpret_cast<float*>(lds + waves * kSlab + waves * (M * xrow_b));  // [M][waves]
+        const int pieces = (s1 - s0) * 32;               // 16-byte pieces per row in this wavefront's K range
+        const int64_t k0 = (int64_t)s0 * 256;
+        for (int m = 0; m < M; m++) {
+            float ss = 0.f;
+            for (int c = lane; c < pieces; c += 64) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + k0 + 8 * c);
+                *reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * c) = v;
+                ss += sumsq_piece(v);
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) ssum[m * waves + wave] = ss;
+        }
+        __syncthreads();
+        for (int m = 0; m < M; m++) {
+            float tot = 0.f;
+            for (int w = 0; w < W; w++) tot += ssum[m * waves + w];   // wavefronts [0, W) cover K once
+            const float rstd = rsqrtf(tot / (float)K + eps);
+            for (int c = lane; c < pieces; c += 64) {
+                u32x4_t* cell = reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * c);
+                const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + k0 + 8 * c);
+                *cell = rmsnorm_piece(*cell, gv, rstd);
+            }
+        }
+        if (s0 < s1) load_x(s0, 0, xa);
+    } else if (s0 < s1) {
         load_x(s0, 0, xa);
         fetch(s0);
     }
@@ -542,7 +582,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
 
 template <int QT, int NUM, int R>
 int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-             const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+             const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
     const int64_t groups = (N + 16 * R - 1) / (16 * R);
     const int nsb = (int)(K >> 8);
     const int mt = (M + 15) / 16;
@@ -557,10 +597,30 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     const int waves = (int)(gated ? 2 * w : w);
     const size_t slab = (size_t)waves * 16 * R * Slab<QT>::stride;
     const size_t red = (size_t)waves * R * mt * 64 * sizeof(f32x4_t);
-    const size_t lds_bytes = slab > red ? slab : red;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
+    if (gamma) {
+        // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares; the
+        // caller keeps M (2 K + 64) within 16 KB
+        if (mt > 1) return SNGGUF_E_BADSHAPE;
+        const size_t xrow_b = (size_t)((nsb + w - 1) / w) * 512 + 16;
+        const size_t staged = slab + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
+        const size_t lds_norm = staged > red ? staged : red;
+        if (lds_norm > 64 * 1024) return SNGGUF_E_BADSHAPE;
+#define SNGGUF_LAUNCH_XN(G, WM) \
+    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, 1, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps)
+        if (gated) {
+            if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
+            else SNGGUF_LAUNCH_XN(true, 8);
+        } else {
+            if (waves <= 4) SNGGUF_LAUNCH_XN(false, 4);
+            else SNGGUF_LAUNCH_XN(false, 8);
+        }
+#undef SNGGUF_LAUNCH_XN
+        return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+    }
+    const size_t lds_bytes = slab > red ? slab : red;
 #define SNGGUF_LAUNCH(G, WM, MT_) \
-    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y)
+    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f)
     if (mt > 1) {
         // more than 16 activation rows: plain projections with one row group per wavefront only
         if constexpr (R == 1) {
@@ -584,19 +644,22 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
 
 template <int QT, int NUM>
 int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-              const bf16_t* residual, bf16_t* y, bool gated, hipStream_t stream) {
+              const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
     // Two row groups per wavefront only when one per wavefront would already give far more
     // wavefronts than the chip holds (a vocabulary-sized projection): otherwise more, smaller
     // workgroups spread more evenly over the 256 compute units.
-    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
-    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, stream);
+    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
+    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
 }
 
 }  // namespace
 
-// 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).
+// 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).  `gamma`
+// (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
-                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream) {
+                        const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
+                        const void* gamma, float eps) {
+    const bf16_t* gp = static_cast<const bf16_t*>(gamma);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
@@ -606,9 +669,9 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
 #define SNGGUF_CASE(QT)                                                                                          \
     if (qtype == QT) {                                                                                           \
         if (numerics == SNGGUF_NUM_GGML_FP32)                                                                    \
-            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);          \
+            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);          \
         if (numerics == SNGGUF_NUM_UPSTREAM_FP16)                                                                \
-            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, stream);      \
+            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);      \
         return SNGGUF_E_BADTYPE;                                                                                 \
     }
     SNGGUF_CASE(SNGGUF_TYPE_Q4_0)

@@ -274,8 +274,8 @@ def test_mlp_forward_under_hip_graph(tmp_path, dev):
 
 
 def test_fused_rmsnorm_through_the_module_helpers(dev):
-    """FusedProjections / gated_mlp with a norm weight: one decode row takes the fused-norm kernels, more rows (or a
-    K-quant) the torch norm in front of the projection; both agree with the oracle's norm + projection."""
+    """FusedProjections / gated_mlp with a norm weight: one decode row takes the fused-norm kernels, more rows the torch
+    norm in front of the projection; both agree with the oracle's norm + projection."""
     from sensenova_u1_amd import FusedProjections, gated_mlp
     from sensenova_u1_amd.quantized_linear import rms_norm
     k, eps = 2048, 1e-6

@@ -63,6 +63,36 @@ def test_rmsnorm_gate_up_silu_parity(dev, c_oracle, shape):
     assert go.rel_l2(h.cpu(), c_oracle.silu_mul(g, u)) <= TOL
 
 
+OTHER_TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K]
+
+
+@pytest.mark.parametrize("qt", OTHER_TYPES)
+def test_rmsnorm_other_formats_parity(dev, c_oracle, qt):
+    """The fused norm in the kernel of the nine other formats: projection with bias (both numerics), a vocabulary-wide
+    one (two row groups per wavefront) and the gated pair."""
+    for m, n, k in [(1, 6144, 4096), (3, 530, 2048), (16, 37, 256)] + ([(1, 40000, 1024)] if qt in (go.Q4_K, go.Q6_K) else []):
+        print(f"case rmsnorm_kq qt={qt} m={m} n={n} k={k}", flush=True)
+        assert ops.rmsnorm_fits(qt, m, k)
+        gate = synthetic.make_packed(qt, n, k, seed=111)
+        up = synthetic.make_packed(qt, n, k, seed=112)
+        x = (synthetic.make_activations(m, k, seed=113 + m).float() * 2.5).to(torch.bfloat16)
+        gamma = _gamma(k, 114)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16)
+        normed = go.qwen3_rms_norm(x, gamma, EPS)
+        gd, ud = gate.to(dev), up.to(dev)
+        for numerics in (0, 1):
+            want = go.gguf_linear_forward(normed, gate, qt, bias, numerics=numerics)
+            y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+            ops.rmsnorm_linear_into(x.to(dev), gamma.to(dev), EPS, gd, qt, bias.to(dev), y, numerics)
+            assert bool(torch.isfinite(y.float()).all())
+            assert go.rel_l2(y.cpu(), want) <= TOL, (m, n, k, numerics)
+        g = go.gguf_linear_forward(normed, gate, qt)
+        u = go.gguf_linear_forward(normed, up, qt)
+        h = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.rmsnorm_gate_up_silu_into(x.to(dev), gamma.to(dev), EPS, gd, ud, qt, h, 1)
+        assert go.rel_l2(h.cpu(), c_oracle.silu_mul(g, u)) <= TOL, (m, n, k)
+
+
 def test_normalized_rows_match_the_oracle_elementwise(dev):
     """An identity-like weight (scale 1.0, one quant of 1 per row) makes the projection return the normalized row itself:
     every element must equal the oracle's, up to one bf16 step in the rare near-tie of the first rounding."""
@@ -89,14 +119,14 @@ def test_rmsnorm_argument_errors(dev):
     x = synthetic.make_activations(2, 4096, seed=3).to(dev)
     y = torch.empty((2, 64), dtype=torch.bfloat16, device=dev)
     assert not ops.rmsnorm_fits(go.Q8_0, 2, 4096)           # two rows of 4096 do not fit the staging area
-    assert not ops.rmsnorm_fits(go.Q4_K, 1, 4096)
+    assert ops.rmsnorm_fits(go.Q4_K, 1, 4096) and not ops.rmsnorm_fits(go.Q4_0, 1, 4096 + 32)
     with pytest.raises(ops.SnGgufError):
         ops.rmsnorm_linear_into(x, gamma, EPS, packed, go.Q8_0, None, y, 1)
     with pytest.raises(ops.SnGgufError):
         ops.rmsnorm_linear_into(x[:1], None, EPS, packed, go.Q8_0, None, y[:1], 1)          # gamma required
-    k4 = synthetic.make_packed(go.Q4_K, 64, 4096, seed=4).to(dev)
+    q40 = synthetic.make_packed(go.Q4_0, 64, 4096 + 32, seed=4).to(dev)
     with pytest.raises(ops.SnGgufError):
-        ops.rmsnorm_linear_into(x[:1], gamma, EPS, k4, go.Q4_K, None, y[:1], 1)             # Q8_0 only
+        ops.rmsnorm_linear_into(synthetic.make_activations(1, 4096 + 32, seed=5).to(dev), gamma, EPS, q40, go.Q4_0, None, y[:1], 1)   # K % 256
     with pytest.raises(ops.SnGgufError):
         ops.rmsnorm_linear_into(x[:1], gamma, -1.0, packed, go.Q8_0, None, y[:1], 1)        # eps < 0
 
