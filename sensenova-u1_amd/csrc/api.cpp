@@ -21,6 +21,8 @@ int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
                          const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
                          const void* gamma = nullptr, float eps = 0.f);
+int launch_gemm_splitk(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                       float* partial, int slices, int numerics, hipStream_t stream);
 int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
                       hipStream_t stream);
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
@@ -160,8 +162,33 @@ int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t
     if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // everything that does not fit the dense route runs as sngguf_linear does
-    const bool two_pass = workspace && workspace_bytes >= 2 * N * K && dense_route_fits(M, N, K);
-    if (!two_pass) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
+    const bool fits = workspace && dense_route_fits(M, N, K);
+    if (!fits) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
+    // Few output tiles (a few hundred rows, or a narrow matrix): a 256 x 256 tile takes as long per K step whether
+    // or not the other compute units have work, so K is split over enough workgroups to occupy them, with the fp32
+    // partial sums in the workspace.  The formats the large-tile kernel decodes itself need no weight pass then and
+    // the whole workspace is free for the sums; the others put them behind the decoded weights if the caller's
+    // workspace is that large.
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const int64_t ksteps = K / 64;
+    const bool tile_type = qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K;
+    const int64_t dense_bytes = tile_type ? 0 : 2 * N * K;
+    if (tiles <= 128 && workspace_bytes > dense_bytes) {
+        int64_t slices = 256 / tiles;
+        const int64_t room = (workspace_bytes - dense_bytes) / (4 * M * N);
+        if (slices > room) slices = room;
+        if (slices > ksteps / 2) slices = ksteps / 2;   // at least two K steps per workgroup
+        if (slices > 64) slices = 64;
+        if (slices >= 2) {
+            float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + dense_bytes);
+            if (tile_type)
+                return sngguf::launch_gemm_splitk(x, M, q, qtype, N, K, bias, y, partial, (int)slices, numerics, s);
+            const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
+            if (rd != SNGGUF_OK) return rd;
+            return sngguf::launch_gemm_splitk(x, M, workspace, 30, N, K, bias, y, partial, (int)slices, numerics, s);
+        }
+    }
+    if (workspace_bytes < 2 * N * K) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
     if (rd != SNGGUF_OK) return rd;
     return sngguf::launch_gemm_dense(x, M, workspace, N, K, bias, y, s);

@@ -261,6 +261,30 @@ int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_
     return launch_gemm_tiles(a, 30, SNGGUF_NUM_GGML_FP32, stream);
 }
 
+int launch_splitk_reduce(const GemmArgs& a, hipStream_t stream);
+
+// y = x W^T (+ bias) on the large-tile kernel with K split over `slices` workgroups per output tile: fp32 partial
+// sums into `partial` (slices * M * N floats), then one pass that adds them.  For problems whose tiles alone leave
+// most of the chip idle.  qtype: Q8_0 (K % 64 == 0), Q4_K, or 30 for weights that are already bf16; 2 <= slices <=
+// K / 64; M K < 2^31 (checked by the caller).
+int launch_gemm_splitk(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                       float* partial, int slices, int numerics, hipStream_t stream) {
+    GemmArgs a{};
+    a.x = static_cast<const bf16_t*>(x);
+    a.y = static_cast<bf16_t*>(y);
+    a.M = M; a.N = N; a.K = K;
+    a.rowmap = nullptr; a.n0_dev = nullptr; a.n0 = M;
+    a.q[0] = a.q[1] = static_cast<const uint8_t*>(q);
+    a.bias[0] = a.bias[1] = static_cast<const bf16_t*>(bias);
+    a.residual = nullptr;
+    a.group_mask = 1;
+    a.partial = partial;
+    a.ksplit = slices;
+    const int rc = launch_gemm_tiles(a, qtype, qtype == 30 ? SNGGUF_NUM_GGML_FP32 : numerics, stream);
+    if (rc != SNGGUF_OK) return rc;
+    return launch_splitk_reduce(a, stream);
+}
+
 int64_t grouped_workspace_bytes(int64_t M) { return 16 + 4 * (M > 0 ? M : 0); }
 
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,

@@ -19,6 +19,11 @@ struct GemmArgs {
     const bf16_t* bias[2];
     const bf16_t* residual; // [M][N] added to the rounded projection output (same rows as y), or NULL
     int group_mask;         // bit g: rows of group g are computed by this launch
+    // Split of K over workgroups (large-tile kernel only): with ksplit > 1 every output tile is computed by ksplit
+    // workgroups, each over its share of the K steps, and written as fp32 partial sums to partial[slice][M][N]
+    // (no bias, no residual, nothing written to y); a second kernel adds the slices up.
+    float* partial;
+    int ksplit;
 };
 
 }  // namespace sngguf

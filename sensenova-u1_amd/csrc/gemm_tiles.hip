@@ -116,13 +116,16 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     const int64_t t0 = (a.group_mask & 1) ? (n0 + TM - 1) / TM : 0;            // row tiles of group 0
     const int64_t t1 = (a.group_mask & 2) ? (a.M - n0 + TM - 1) / TM : 0;      // row tiles of group 1
     const int64_t ntn = (a.N + TN - 1) / TN;
-    const int64_t total = (t0 + t1) * ntn;
+    const int S = a.ksplit > 1 ? a.ksplit : 1;                                 // workgroups per output tile (K slices)
+    const int64_t total = (t0 + t1) * ntn * S;
     const int64_t pid = blockIdx.x;
     if (pid >= total) return;
     // consecutive tile numbers on one XCD: workgroup ids are dealt round-robin over 8 XCDs
     const int64_t per = total >> 3, rem = total & 7;
     const int64_t xcd = pid & 7, idx = pid >> 3;
-    const int64_t tile = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    const int64_t tile_slice = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    const int64_t tile = tile_slice / S;
+    const int slice = (int)(tile_slice - tile * S);
     // The 32 workgroups that run at the same time on one XCD cover a block of 4 row tiles x 8 column
     // tiles when the tile grid divides that way (4 activation tiles + 8 packed weight tiles pass
     // through the XCD's L2 per block instead of 1 + 32), else 32 consecutive column tiles of one row.
@@ -148,7 +151,10 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     const bf16_t* __restrict__ bias = a.bias[g];
     const int64_t nb0 = tn * TN;
     const int64_t row_bytes = kDense ? 2 * a.K : kQ4K ? (a.K >> 8) * 144 : (a.K >> 5) * 34;
-    const int ksteps = (int)(a.K / TK);
+    // this workgroup's K steps: [ks0, ks0 + ksteps) of the K / 64 in all (everything when K is not split)
+    const int ksteps_all = (int)(a.K / TK);
+    const int ks0 = (int)((int64_t)slice * ksteps_all / S);
+    const int ksteps = (int)((int64_t)(slice + 1) * ksteps_all / S) - ks0;
 
     // ---- LDS: two stages of (activation tile, weight tile) + one raw-weight slab per wavefront ------------
     // A tile is 256 rows of 64 bf16 (128 bytes, no padding); the eight 16-byte chunks of a row are
@@ -237,14 +243,14 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 #define SNGGUF_FETCH_W(kb, I0, I1)                                                                           \
     do {                                                                                                     \
         if constexpr (kQ4K) {                                                                                \
-            const uint8_t* ph_ = scalar_ptr(wbase + (int64_t)((kb) >> 2) * 144);                             \
-            const uint8_t* pq_ = ph_ + 32 * ((kb) & 3);                                                      \
+            const uint8_t* ph_ = scalar_ptr(wbase + (int64_t)(((kb) + ks0) >> 2) * 144);                     \
+            const uint8_t* pq_ = ph_ + 32 * (((kb) + ks0) & 3);                                              \
             _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
                 __builtin_amdgcn_global_load_lds(                                                            \
                     (const __attribute__((address_space(1))) void*)((head_piece[i_] ? ph_ : pq_) + goff[i_]),\
                     (__attribute__((address_space(3))) void*)(raw + 256 * i_), 16, 0, 0);                    \
         } else {                                                                                             \
-            const uint8_t* p_ = scalar_ptr(wbase + (int64_t)(kb) * 68);                                      \
+            const uint8_t* p_ = scalar_ptr(wbase + (int64_t)((kb) + ks0) * 68);                              \
             _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
                 __builtin_amdgcn_global_load_lds(                                                            \
                     (const __attribute__((address_space(1))) void*)(p_ + goff[i_]),                          \
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     } while (0)
 #define SNGGUF_LOAD_X(kb, stage, I0, I1)                                                                     \
     do {                                                                                                     \
-        const uint8_t* xb_ = scalar_ptr(a.x + (int64_t)(kb) * TK);                                           \
+        const uint8_t* xb_ = scalar_ptr(a.x + (int64_t)((kb) + ks0) * TK);                                   \
         _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
             __builtin_amdgcn_global_load_lds(                                                                \
                 (const __attribute__((address_space(1))) void*)(xb_ + xoff[i_]),                             \
@@ -269,7 +275,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     } while (0)
 #define SNGGUF_LOAD_WD(kb, stage, I0, I1)                                                                    \
     do {                                                                                                     \
-        const uint8_t* wb_ = scalar_ptr(wbase + (int64_t)(kb) * (2 * TK));                                   \
+        const uint8_t* wb_ = scalar_ptr(wbase + (int64_t)((kb) + ks0) * (2 * TK));                           \
         _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
             __builtin_amdgcn_global_load_lds(                                                                \
                 (const __attribute__((address_space(1))) void*)(wb_ + woff[i_]),                             \
@@ -280,7 +286,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 // half); Q4_K (D, DM) of sub-block 2 (kbn % 4) + wblk.
 #define SNGGUF_SCALES_W(kbn)                                                                                 \
     do {                                                                                                     \
-        if constexpr (kQ4K) q4k_sub_block_scales<NUM>(rw[0], rw[1], rw[2], rw[3], 2 * ((kbn) & 3) + wblk, sc_a, sc_b); \
+        if constexpr (kQ4K) q4k_sub_block_scales<NUM>(rw[0], rw[1], rw[2], rw[3], 2 * (((kbn) + ks0) & 3) + wblk, sc_a, sc_b); \
         else sc_a = __builtin_amdgcn_perm(rw[0], rw[0], sel_d);                                              \
     } while (0)
 // decode quarter `part` (8 elements) of this thread's 32 into LDS.  Q8_0: quant dwords 2 part,
@@ -471,6 +477,33 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 
     // ---- epilogue: D[i][j], i = weight row (n), j = activation row (m) ----------------------------------------
     // lane: j = lane % 32; register v: i = 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    if (a.partial) {
+        // K split over workgroups: this slice's sums go out as fp32, to be added up by splitk_reduce_kernel
+        float* part = a.partial + (int64_t)slice * a.M * a.N;
+        const bool vec = (a.N & 3) == 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                const int64_t n = nb0 + wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int64_t rr = row_begin + wm * 64 + j * 32 + (lane & 31);
+                    if (rr >= row_end || n >= a.N) continue;
+                    const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+                    float* pp = part + gr * a.N + n;
+                    if (vec) {
+                        *reinterpret_cast<f32x4_t*>(pp) = f32x4_t{acc[i][j][4 * vg], acc[i][j][4 * vg + 1], acc[i][j][4 * vg + 2], acc[i][j][4 * vg + 3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < a.N) pp[e] = acc[i][j][4 * vg + e];
+                    }
+                }
+            }
+        }
+        return;
+    }
     if ((a.N & 7) == 0) {
         // Rows of y are 16-byte aligned: stage the tile in LDS as bf16 [256 m][256 n] (all K-loop
         // buffers are dead after the last barrier) and write it out as 16-byte pieces, 32 lanes
@@ -562,8 +595,38 @@ int launch_tiles(const GemmArgs& a, hipStream_t stream) {
     if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
     const int64_t row_tiles = (a.M + TM - 1) / TM + 1;  // a split adds at most one partial tile
     const int64_t ntn = (a.N + TN - 1) / TN;
-    gemm_tile_kernel<QT, NUM><<<dim3((unsigned)(row_tiles * ntn)), dim3(512), kLdsBytes, stream>>>(a);
+    const int64_t slices = a.ksplit > 1 ? a.ksplit : 1;
+    gemm_tile_kernel<QT, NUM><<<dim3((unsigned)(row_tiles * ntn * slices)), dim3(512), kLdsBytes, stream>>>(a);
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
+// y[m][n] = bf16(sum over slices of partial[s][m][n] + bias[n]), slices added in ascending order; one thread per
+// four consecutive outputs.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t M, int64_t N,
+                                                            const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+    const int64_t total = M * N;
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i0 >= total) return;
+    if ((N & 3) == 0) {
+        f32x4_t s = *reinterpret_cast<const f32x4_t*>(partial + i0);
+        for (int k = 1; k < slices; k++) {
+            const f32x4_t t = *reinterpret_cast<const f32x4_t*>(partial + (int64_t)k * total + i0);
+            s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+        }
+        if (bias) {
+            const int64_t n = i0 % N;
+#pragma unroll
+            for (int e = 0; e < 4; e++) s[e] += bf16_to_f32(bias[n + e]);
+        }
+        *reinterpret_cast<u32x2_t*>(y + i0) = u32x2_t{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3])};
+    } else {
+        for (int e = 0; e < 4 && i0 + e < total; e++) {
+            float s = partial[i0 + e];
+            for (int k = 1; k < slices; k++) s += partial[(int64_t)k * total + i0 + e];
+            if (bias) s += bf16_to_f32(bias[(i0 + e) % N]);
+            y[i0 + e] = f32_to_bf16(s);
+        }
+    }
 }
 
 }  // namespace
@@ -579,6 +642,13 @@ int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t st
     if (qtype == kTypeBF16) return launch_tiles<kTypeBF16, SNGGUF_NUM_GGML_FP32>(a, stream);
 #undef SNGGUF_CASE
     return SNGGUF_E_BADTYPE;
+}
+
+// The partial sums of a launch with a.ksplit > 1 -> a.y (+ bias of group 0).
+int launch_splitk_reduce(const GemmArgs& a, hipStream_t stream) {
+    const int64_t quads = (a.M * a.N + 3) / 4;
+    splitk_reduce_kernel<<<dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream>>>(a.partial, a.ksplit, a.M, a.N, a.bias[0], a.y);
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
 }  // namespace sngguf

@@ -19,6 +19,28 @@ def _check(got, want, tol=TOL):
 
 
 @pytest.mark.parametrize("qt", TYPES)
+def test_linear_with_workspace_split_k(dev, qt):
+    """sngguf_linear_ws on problems with few output tiles (some hundred rows, or a narrow matrix): K is split over
+    several workgroups per tile and the fp32 partial sums are added in a second pass.  Q8_0 / Q4_K keep the sums in
+    the plain 2 N K workspace, the other formats behind the decoded weights when the workspace is larger."""
+    print(f"case linear_ws_splitk qt={qt}", flush=True)
+    for numerics, (m, n, k) in [(1, (128, 1024, 4096)), (0, (300, 2050, 1024)), (1, (65, 37, 512)), (1, (512, 4096, 2048)),
+                                (0, (1000, 515, 768))]:
+        packed = synthetic.make_packed(qt, n, k, seed=m + n + k + qt)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(k)) * 0.5).to(torch.bfloat16) if n % 2 else None
+        want = go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics)
+        xd, pd = x.to(dev), packed.to(dev)
+        bd = bias.to(dev) if bias is not None else None
+        for extra in (0, 4 * 16 * m * n):
+            ws = torch.full(((ops.linear_workspace_bytes(n, k) + extra) // 2,), float("nan"), dtype=torch.bfloat16, device=dev)
+            y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+            ops.linear_ws_into(xd, pd, qt, bd, y, ws, numerics)
+            assert bool(torch.isfinite(y.float()).all())
+            _check(y.cpu(), want)
+
+
+@pytest.mark.parametrize("qt", TYPES)
 @pytest.mark.parametrize("numerics", [0, 1])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 16])
 def test_gemv_parity(dev, qt, numerics, m):
