@@ -442,6 +442,21 @@ def main() -> None:
             for j, n, k in rest:
                 ops.linear_ws_into(xs[k], tower[i % 2][j], Q8_0, None, ys[n], wtmp, num)
 
+        # a few hundred rows (a text prompt): few output tiles, so the workspace route splits K over workgroups
+        mid = {}
+        for mm in (128, 512):
+            xm = {k: synthetic.make_activations(mm, k, seed=40 + k, device=dev) for k in (HIDDEN, INTER)}
+            ym = {n: torch.empty((mm, n), dtype=torch.bfloat16, device=dev) for n in (HIDDEN, KV, INTER)}
+            row = {}
+            for j, (nm, n, k) in enumerate(shapes):
+                if nm in ("v", "o", "up"):
+                    continue
+                _, e_f = run_region(lambda i: ops.linear_into(xm[k], tower[i % 2][j], Q8_0, None, ym[n], num), 16, 4)
+                _, e_w = run_region(lambda i: ops.linear_ws_into(xm[k], tower[i % 2][j], Q8_0, None, ym[n], wtmp, num), 16, 4)
+                _, e_t = run_region(lambda i: two_pass(xm[k], tower[i % 2][j], n, k, ym[n]), 16, 4)
+                row[nm] = {"linear_us": round(e_f / 16 * 1e3, 1), "workspace_us": round(e_w / 16 * 1e3, 1),
+                           "two_pass_us": round(e_t / 16 * 1e3, 1)}
+            mid[f"M{mm}"] = row
         wall_st, _ = run_region(tower_stacked, gs, args.gemm_warmup)
         wall_st_ws, _ = run_region(tower_stacked_ws, gs, args.gemm_warmup)
         del qkv, y_qkv
@@ -493,6 +508,12 @@ def main() -> None:
                 "workspace_value": round(flops / (wall_st_ws / gs * 1e-3) / 1e12, 2),
                 "workspace_ms_per_step": round(wall_st_ws / gs, 4),
                 "workspace_pct_of_bf16_mfma_peak": round(100 * flops / (wall_st_ws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            },
+            "mid_rows": {
+                "what": "one projection at 128 and 512 rows (q 4096^2, k 4096->1024, gate 4096->12288, down 12288->4096): "
+                        "sngguf_linear (large-tile kernel, few tiles), sngguf_linear_ws (K split over workgroups, fp32 partial "
+                        "sums in the workspace) and dequantize + device-library GEMM",
+                **mid,
             },
             "resident": {
                 "what": "gemm_policy 'resident': the bf16 weights written once by sngguf dequantize and kept "

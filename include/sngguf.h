@@ -131,8 +131,11 @@ int sngguf_linear_residual(const void* x, int64_t M, const void* q, int qtype, i
  * workspace (device memory, 16-byte aligned) of at least sngguf_linear_workspace_bytes(N, K) = 2 N K bytes
  * and a problem it fits (M >= 65, K % 64 == 0, M K < 2^31) the weights are decoded once into the workspace as bf16 - the same values, same rounding chain,
  * as the fused kernels decode on the fly - and a dense bf16 tile GEMM consumes them; any of the ten types then
- * runs at the rate of that GEMM.  Otherwise (workspace NULL or too small included) it behaves exactly as
- * sngguf_linear.  The workspace holds nothing the caller needs afterwards; calls sharing one workspace must
+ * runs at the rate of that GEMM.  A problem with at most 128 output tiles of 256 x 256 (a few hundred rows, or a
+ * narrow matrix) is split along K over floor(256 / tiles) workgroups per tile, with fp32 partial sums in the
+ * workspace and a second pass that adds them: Q8_0 and Q4_K then skip the weight pass and use the 2 N K bytes
+ * for the sums, the other types need 4 S M N bytes more than 2 N K for it.  Otherwise (workspace NULL or too
+ * small included) it behaves exactly as sngguf_linear.  The workspace holds nothing the caller needs afterwards; calls sharing one workspace must
  * be ordered on one stream.  Never allocates.
  */
 int64_t sngguf_linear_workspace_bytes(int64_t N, int64_t K);

@@ -308,3 +308,23 @@ def test_fused_rmsnorm_through_the_module_helpers(dev):
             want, _ = go.mlp_forward(normed, gate.weight.as_tensor().cpu(), up.weight.as_tensor().cpu(),
                                      down.weight.as_tensor().cpu(), (qt, qt, qt))
             assert go.rel_l2(got.cpu(), want) <= 2e-3     # two chained projections
+
+
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K, go.Q6_K])
+def test_auto_policy_between_65_and_256_rows(dev, qt):
+    """65 ... 256 rows under gemm_policy 'auto': Q8_0 / Q4_K through the library's split-K route, other formats
+    through the weight pass + dense GEMM; every policy agrees with the oracle."""
+    n, k = 1000, 2048
+    mod = GGUFLinear(k, n, bias=True, compute_dtype=torch.bfloat16, device="meta")
+    packed = synthetic.make_packed(qt, n, k, seed=31)
+    mod.weight = GGUFParameter(packed.to(dev), quant_type=qt)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(32)) * 0.5).to(torch.bfloat16)
+    mod.bias = torch.nn.Parameter(bias.to(dev), requires_grad=False)
+    for rows in (65, 200, 256, 300):
+        print(f"case module_mid_rows qt={qt} rows={rows}", flush=True)
+        x = synthetic.make_activations(rows, k, seed=rows)
+        want = go.gguf_linear_forward(x, packed, qt, bias)
+        for policy in ("auto", "two_pass", "fused"):
+            mod.gemm_policy = policy
+            got = mod(x.to(dev))
+            assert go.rel_l2(got.cpu(), want) <= TOL, (rows, policy)
