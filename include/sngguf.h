@@ -232,6 +232,9 @@ int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, in
  * decoded into it once as bf16 and ONE dense tile-GEMM launch serves both row groups - whatever the two quant
  * types are.  Otherwise it is sngguf_grouped_linear.  workspace is the row-map scratch of
  * sngguf_grouped_linear (needed with an indicator).  Never allocates.
+ * Two weight sets of one type among Q8_0 / Q4_K with at most 128 output tiles (narrow matrices such as k / v, or a
+ * few hundred rows) are split along K as sngguf_linear_ws does, the fp32 partial sums in dense_workspace (room for
+ * at least two slices of M N floats enables it; the weights are then decoded on the fly).
  */
 int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text,
                              const void* q_und, int qtype_und, const void* q_gen, int qtype_gen,

@@ -31,7 +31,8 @@ int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, i
 int64_t grouped_workspace_bytes(int64_t M);
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
                         int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
-                        const void* bias_gen, void* y, void* workspace, int numerics, hipStream_t stream);
+                        const void* bias_gen, void* y, void* workspace, int numerics, hipStream_t stream,
+                        float* partial = nullptr, int slices = 0);
 }  // namespace sngguf
 
 namespace {
@@ -346,6 +347,34 @@ int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator,
                              const void* bias_gen, void* y, void* workspace, void* dense_workspace,
                              int64_t dense_workspace_bytes, int numerics, void* stream) {
     const bool two_pass = dense_workspace && dense_workspace_bytes >= 4 * N * K && K > 0 && N > 0 && grouped_dense_route_fits(M, N, K);
+    // Few output tiles (narrow matrices such as k / v, or a few hundred rows) of one type the large-tile kernel decodes
+    // itself: K split over workgroups, the fp32 partial sums in the dense workspace (as sngguf_linear_ws does)
+    const bool tile_types = qtype_und == qtype_gen && (qtype_und == SNGGUF_TYPE_Q8_0 || qtype_und == SNGGUF_TYPE_Q4_K);
+    if (!two_pass && dense_workspace && tile_types && M >= 65 && N > 0 && K > 0 && K % 64 == 0 && M < kMaxDim && N < kMaxDim
+        && K < kMaxDim && M * K < ((int64_t)1 << 31)) {
+        const int64_t tiles = ((M + 255) / 256 + 1) * ((N + 255) / 256);   // a split into two groups adds one partial row tile
+        int64_t slices = tiles <= 128 ? 256 / tiles : 0;
+        const int64_t room = dense_workspace_bytes / (4 * M * N);
+        if (slices > room) slices = room;
+        if (slices > K / 128) slices = K / 128;   // at least two K steps per workgroup
+        if (slices > 64) slices = 64;
+        if (slices >= 2) {
+            int rc = check_matmul(x, M, q_und, qtype_und, N, K, y, numerics);
+            if (rc != SNGGUF_OK) return rc;
+            rc = check_matmul(x, M, q_gen, qtype_gen, N, K, y, numerics);
+            if (rc != SNGGUF_OK) return rc;
+            if (!aligned(dense_workspace, 16)) return SNGGUF_E_ALIGN;
+            if (indicator) {
+                if (!workspace) return SNGGUF_E_NULLPTR;
+                if (!aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+            } else if (n_text < 0 || n_text > M) {
+                return SNGGUF_E_BADSHAPE;
+            }
+            return sngguf::launch_grouped_gemm(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und,
+                                               bias_gen, y, workspace, numerics, static_cast<hipStream_t>(stream),
+                                               static_cast<float*>(dense_workspace), (int)slices);
+        }
+    }
     if (!two_pass)
         return sngguf_grouped_linear(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und, bias_gen, y,
                                      workspace, numerics, stream);

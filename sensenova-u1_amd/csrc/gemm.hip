@@ -261,7 +261,7 @@ int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_
     return launch_gemm_tiles(a, 30, SNGGUF_NUM_GGML_FP32, stream);
 }
 
-int launch_splitk_reduce(const GemmArgs& a, hipStream_t stream);
+int launch_splitk_reduce(const GemmArgs& a, const uint8_t* indicator, int64_t n_text, hipStream_t stream);
 
 // y = x W^T (+ bias) on the large-tile kernel with K split over `slices` workgroups per output tile: fp32 partial
 // sums into `partial` (slices * M * N floats), then one pass that adds them.  For problems whose tiles alone leave
@@ -282,14 +282,17 @@ int launch_gemm_splitk(const void* x, int64_t M, const void* q, int qtype, int64
     a.ksplit = slices;
     const int rc = launch_gemm_tiles(a, qtype, qtype == 30 ? SNGGUF_NUM_GGML_FP32 : numerics, stream);
     if (rc != SNGGUF_OK) return rc;
-    return launch_splitk_reduce(a, stream);
+    return launch_splitk_reduce(a, nullptr, M, stream);
 }
 
 int64_t grouped_workspace_bytes(int64_t M) { return 16 + 4 * (M > 0 ? M : 0); }
 
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
                         int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
-                        const void* bias_gen, void* y, void* workspace, int numerics, hipStream_t stream) {
+                        const void* bias_gen, void* y, void* workspace, int numerics, hipStream_t stream, float* partial,
+                        int slices) {
+    // partial / slices: K split over `slices` workgroups per tile with fp32 partial sums (slices * M * N floats);
+    // only for two weight sets of one type that the large-tile kernel takes (checked by the caller)
     GemmArgs a{};
     a.x = static_cast<const bf16_t*>(x);
     a.y = static_cast<bf16_t*>(y);
@@ -310,6 +313,15 @@ int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int6
         a.rowmap = nullptr;
         a.n0_dev = nullptr;
         a.n0 = n_text;
+    }
+    if (partial && slices > 1) {
+        if (qtype_und != qtype_gen) return SNGGUF_E_BADTYPE;
+        a.group_mask = 3;
+        a.partial = partial;
+        a.ksplit = slices;
+        const int rc = launch_gemm_tiles(a, qtype_und, numerics, stream);
+        if (rc != SNGGUF_OK) return rc;
+        return launch_splitk_reduce(a, indicator, n_text, stream);
     }
     if (qtype_und == qtype_gen) {
         a.group_mask = 3;

@@ -600,21 +600,26 @@ int launch_tiles(const GemmArgs& a, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
-// y[m][n] = bf16(sum over slices of partial[s][m][n] + bias[n]), slices added in ascending order; one thread per
-// four consecutive outputs.
+// y[m][n] = bf16(sum over slices of partial[s][m][n] + bias_g[n]), slices added in ascending order; one thread per
+// four consecutive outputs.  Row m belongs to group 1 (bias1) when indicator[m] != 0, or without an indicator when
+// m >= n_text.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t M, int64_t N,
-                                                            const bf16_t* __restrict__ bias, bf16_t* __restrict__ y) {
+                                                            const uint8_t* __restrict__ indicator, int64_t n_text,
+                                                            const bf16_t* __restrict__ bias0, const bf16_t* __restrict__ bias1,
+                                                            bf16_t* __restrict__ y) {
     const int64_t total = M * N;
     const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i0 >= total) return;
+    auto bias_of = [&](int64_t m) { return (indicator ? indicator[m] != 0 : m >= n_text) ? bias1 : bias0; };
     if ((N & 3) == 0) {
         f32x4_t s = *reinterpret_cast<const f32x4_t*>(partial + i0);
         for (int k = 1; k < slices; k++) {
             const f32x4_t t = *reinterpret_cast<const f32x4_t*>(partial + (int64_t)k * total + i0);
             s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
         }
+        const int64_t m = i0 / N, n = i0 - m * N;
+        const bf16_t* bias = bias_of(m);
         if (bias) {
-            const int64_t n = i0 % N;
 #pragma unroll
             for (int e = 0; e < 4; e++) s[e] += bf16_to_f32(bias[n + e]);
         }
@@ -623,7 +628,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
         for (int e = 0; e < 4 && i0 + e < total; e++) {
             float s = partial[i0 + e];
             for (int k = 1; k < slices; k++) s += partial[(int64_t)k * total + i0 + e];
-            if (bias) s += bf16_to_f32(bias[(i0 + e) % N]);
+            const int64_t m = (i0 + e) / N;
+            const bf16_t* bias = bias_of(m);
+            if (bias) s += bf16_to_f32(bias[(i0 + e) - m * N]);
             y[i0 + e] = f32_to_bf16(s);
         }
     }
@@ -644,10 +651,12 @@ int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t st
     return SNGGUF_E_BADTYPE;
 }
 
-// The partial sums of a launch with a.ksplit > 1 -> a.y (+ bias of group 0).
-int launch_splitk_reduce(const GemmArgs& a, hipStream_t stream) {
+// The partial sums of a launch with a.ksplit > 1 -> a.y (+ the bias of each row's group: group 1 where indicator[m] != 0,
+// or from row n_text on without an indicator).
+int launch_splitk_reduce(const GemmArgs& a, const uint8_t* indicator, int64_t n_text, hipStream_t stream) {
     const int64_t quads = (a.M * a.N + 3) / 4;
-    splitk_reduce_kernel<<<dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream>>>(a.partial, a.ksplit, a.M, a.N, a.bias[0], a.y);
+    splitk_reduce_kernel<<<dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream>>>(a.partial, a.ksplit, a.M, a.N, indicator, n_text,
+                                                                                          a.bias[0], a.bias[1], a.y);
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 

@@ -290,6 +290,37 @@ def _grouped_large_tiles(dev, m, n, k):
     assert torch.equal(got[~split], yu[~split]) and torch.equal(got[split], yg[split])
 
 
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K])
+def test_grouped_linear_split_k(dev, qt):
+    """sngguf_grouped_linear_ws on a narrow matrix (few output tiles) of a type the large-tile kernel decodes: K split over
+    workgroups, partial sums in the dense workspace, the reduce pass adding each row's own group bias - with a row map
+    and with the contiguous split, ragged N, an empty group."""
+    print(f"case grouped_splitk qt={qt}", flush=True)
+    for m, n, k, n_text in [(700, 1024, 1024, 300), (4608, 1030, 512, 512), (130, 257, 2048, 0), (1000, 515, 768, 1000)]:
+        und = synthetic.make_packed(qt, n, k, seed=61)
+        gen = synthetic.make_packed(qt, n, k, seed=62)
+        x = synthetic.make_activations(m, k, seed=63)
+        g = torch.Generator().manual_seed(64)
+        ind = torch.rand(m, generator=g) < 0.6
+        bu = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16)
+        bg = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16)
+        want = torch.empty((m, n), dtype=torch.bfloat16)
+        want[~ind] = go.gguf_linear_forward(x[~ind], und, qt, bu)
+        want[ind] = go.gguf_linear_forward(x[ind], gen, qt, bg)
+        xd, ud, gd, bud, bgd = x.to(dev), und.to(dev), gen.to(dev), bu.to(dev), bg.to(dev)
+        ws = torch.empty(ops.grouped_workspace_bytes(m), dtype=torch.uint8, device=dev)
+        dw = torch.full((4 * 16 * m * n // 2,), float("nan"), dtype=torch.bfloat16, device=dev)   # room for 16 slices
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.grouped_linear_ws_into(xd, ind.to(torch.uint8).to(dev), 0, ud, qt, gd, qt, bud, bgd, y, ws, dw, 1)
+        assert bool(torch.isfinite(y.float()).all())
+        _check(y.cpu(), want)
+        want2 = torch.cat([go.gguf_linear_forward(x[:n_text], und, qt, bu), go.gguf_linear_forward(x[n_text:], gen, qt, bg)])
+        y2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.grouped_linear_ws_into(xd, None, n_text, ud, qt, gd, qt, bud, bgd, y2, None, dw, 0)
+        want2 = torch.cat([go.gguf_linear_forward(x[:n_text], und, qt, bu, numerics=0), go.gguf_linear_forward(x[n_text:], gen, qt, bg, numerics=0)])
+        _check(y2.cpu(), want2)
+
+
 @pytest.mark.parametrize("qt_pair", [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q6_K), (go.Q5_0, go.Q3_K)])
 def test_grouped_linear_with_dense_workspace(dev, qt_pair):
     """sngguf_grouped_linear_ws: both weight sets decoded once into the workspace, one dense launch over both row
