@@ -529,3 +529,42 @@ def test_linear_errors(dev):
         ops.linear(torch.zeros(2, 64, dtype=torch.bfloat16), packed.cpu(), go.Q8_0)       # CPU
     y = ops.linear(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16), packed, go.Q8_0)
     assert y.shape == (0, 8)
+
+
+def test_workspace_routes_replay_in_a_graph(dev):
+    """The multi-launch routes (split-K + reduce pass; weight pass + dense kernel; row partition + grouped launch)
+    captured in a HIP graph: every replay, with eager launches and new inputs in between, equals the eager result."""
+    print("case ws_graph", flush=True)
+    qt, n, k = go.Q8_0, 1024, 2048
+    packed = synthetic.make_packed(qt, n, k, seed=5).to(dev)
+    gen = synthetic.make_packed(qt, n, k, seed=6).to(dev)
+    big = synthetic.make_packed(qt, 8192, 512, seed=7).to(dev)
+    ws = torch.empty(4 * 16 * 700 * n, dtype=torch.uint8, device=dev)
+    rowws = torch.empty(ops.grouped_workspace_bytes(700), dtype=torch.uint8, device=dev)
+    sx = synthetic.make_activations(700, k, seed=1).to(dev)
+    sx_big = synthetic.make_activations(4096, 512, seed=2).to(dev)
+    sind = torch.zeros(700, dtype=torch.uint8, device=dev)
+    y1 = torch.empty((128, n), dtype=torch.bfloat16, device=dev)
+    y2 = torch.empty((700, n), dtype=torch.bfloat16, device=dev)
+    y3 = torch.empty((4096, 8192), dtype=torch.bfloat16, device=dev)
+
+    def run(o1, o2, o3):
+        ops.linear_ws_into(sx[:128], packed, qt, None, o1, ws, 1)                                   # split-K
+        ops.grouped_linear_ws_into(sx, sind, 0, packed, qt, gen, qt, None, None, o2, rowws, ws, 1)  # partition + split-K
+        ops.linear_ws_into(sx_big, big, qt, None, o3, ws, 1)                                        # weight pass + dense
+
+    run(y1, y2, y3)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(y1, y2, y3)
+    for seed in (21, 22, 23):
+        sx.copy_(synthetic.make_activations(700, k, seed=seed).to(dev))
+        sx_big.copy_(synthetic.make_activations(4096, 512, seed=seed + 10).to(dev))
+        sind.copy_((torch.rand(700, generator=torch.Generator().manual_seed(seed)) < 0.5).to(torch.uint8).to(dev))
+        e1, e2, e3 = torch.empty_like(y1), torch.empty_like(y2), torch.empty_like(y3)
+        run(e1, e2, e3)                      # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y1, e1) and torch.equal(y2, e2) and torch.equal(y3, e3), seed
