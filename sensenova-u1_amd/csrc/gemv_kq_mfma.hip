@@ -605,9 +605,18 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
         const size_t xrow_b = (size_t)((nsb + w - 1) / w) * 512 + 16;
         const size_t staged = slab + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
         const size_t lds_norm = staged > red ? staged : red;
-        if (lds_norm > 64 * 1024) return SNGGUF_E_BADSHAPE;
-#define SNGGUF_LAUNCH_XN(G, WM) \
-    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, 1, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps)
+        if (lds_norm > 160 * 1024) return SNGGUF_E_BADSHAPE;
+        // slabs of two row groups per wavefront plus the staged activations can pass the default dynamic-LDS limit:
+        // raise it once per kernel instance
+#define SNGGUF_LAUNCH_XN(G, WM)                                                                                        \
+    do {                                                                                                               \
+        static const hipError_t attr = hipFuncSetAttribute(                                                            \
+            reinterpret_cast<const void*>(&gemv_kq_mfma_kernel<QT, NUM, R, G, WM, 1, true>),                            \
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                                    \
+        if (attr != hipSuccess) return SNGGUF_E_LAUNCH;                                                                 \
+        gemv_kq_mfma_kernel<QT, NUM, R, G, WM, 1, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias,    \
+                                                                                           residual, y, gamma, eps);   \
+    } while (0)
         if (gated) {
             if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
             else SNGGUF_LAUNCH_XN(true, 8);

@@ -70,7 +70,8 @@ OTHER_TYPES = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q2_K, go.Q3_K, go.Q4_K, go
 def test_rmsnorm_other_formats_parity(dev, c_oracle, qt):
     """The fused norm in the kernel of the nine other formats: projection with bias (both numerics), a vocabulary-wide
     one (two row groups per wavefront) and the gated pair."""
-    for m, n, k in [(1, 6144, 4096), (3, 530, 2048), (16, 37, 256)] + ([(1, 40000, 1024)] if qt in (go.Q4_K, go.Q6_K) else []):
+    for m, n, k in [(1, 6144, 4096), (3, 530, 2048), (16, 37, 256)] + ([(1, 40000, 1024)] if qt in (go.Q4_K, go.Q6_K) else []) \
+            + ([(1, 33000, 4096)] if qt in (go.Q6_K, go.Q5_1) else []):   # lm_head-like: the largest slabs + staged activations
         print(f"case rmsnorm_kq qt={qt} m={m} n={n} k={k}", flush=True)
         assert ops.rmsnorm_fits(qt, m, k)
         gate = synthetic.make_packed(qt, n, k, seed=111)
