@@ -554,12 +554,21 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     const int waves = gated ? 2 * w : w;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     if (gamma) {
-        // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares;
-        // the caller keeps M (2 K + 64) within 16 KB, so this stays below the default dynamic-LDS limit
+        // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares.
+        // The caller keeps M (2 K + 64) within 16 KB; a gated pair stages the rows twice (gate and up wavefronts),
+        // so with the slabs this can pass the default dynamic-LDS limit: raise it once per kernel instance
         const size_t xrow_b = (size_t)((steps + w - 1) / w) * CB * 64 + 16;
         const size_t lds_norm = (size_t)waves * 16 * CB * 34 + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
-        if (lds_norm > 64 * 1024) return SNGGUF_E_BADSHAPE;
-#define SNGGUF_LAUNCH_XN(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps)
+        if (lds_norm > 160 * 1024) return SNGGUF_E_BADSHAPE;
+#define SNGGUF_LAUNCH_XN(G, WM)                                                                                         \
+    do {                                                                                                                \
+        static const hipError_t attr = hipFuncSetAttribute(                                                             \
+            reinterpret_cast<const void*>(&gemv_q8_mfma_kernel<NUM, CB, G, WM, true>),                                   \
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                                     \
+        if (attr != hipSuccess) return SNGGUF_E_LAUNCH;                                                                  \
+        gemv_q8_mfma_kernel<NUM, CB, G, WM, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, \
+                                                                                     y, gamma, eps);                    \
+    } while (0)
         if (gated) {
             if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
             else SNGGUF_LAUNCH_XN(true, 8);

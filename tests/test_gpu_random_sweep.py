@@ -123,3 +123,45 @@ def test_random_grouped_cases(dev, seed):
             ops.grouped_linear_ws_into(put(x), put(ind.to(torch.uint8)), 0, put(und), qu, put(gen), qg, put(bu), put(bg), y,
                                        row_ws, dense_ws, numerics)
         _ok(y.cpu(), want, tag)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_rmsnorm_cases(dev, seed):
+    """RMSNorm folded into the projection / the gated pair: every type (and the tiled Q8_0 copy), row counts up to what
+    the staging area takes for the drawn K, ragged N, wide N, both numerics, against oracle norm + oracle projection."""
+    rnd = random.Random(seed)
+    for it in range(40):
+        qt = rnd.choice(TYPES)
+        k = 256 * rnd.randint(1, 24)
+        m = rnd.randint(1, min(16, 16384 // (2 * k + 64)))
+        n = rnd.choice([rnd.randint(1, 2500), rnd.randint(1, 2500), 6144, 33000 + rnd.randint(0, 40)])
+        numerics = rnd.choice([0, 1])
+        kind = rnd.choice(["linear", "gate_up", "tiled", "tiled_gate_up"])
+        if kind.startswith("tiled"):
+            qt = go.Q8_0
+        eps = rnd.choice([1e-6, 1e-5, 0.0])
+        tag = f"seed={seed} it={it} kind={kind} qt={qt} m={m} n={n} k={k} numerics={numerics} eps={eps}"
+        print("case", tag, flush=True)
+        assert ops.rmsnorm_fits(qt, m, k), tag
+        packed = synthetic.make_packed(qt, n, k, seed=it)
+        x = (synthetic.make_activations(m, k, seed=2000 + it).float() * rnd.choice([0.05, 1.0, 7.0])).to(torch.bfloat16)
+        gamma = (torch.rand(k, generator=torch.Generator().manual_seed(it)) * 1.5 + 0.25).to(torch.bfloat16)
+        use_bias = kind in ("linear", "tiled") and rnd.random() < 0.4
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(it)) * 0.5).to(torch.bfloat16) if use_bias else None
+        normed = go.qwen3_rms_norm(x, gamma, eps)
+        want = go.gguf_linear_forward(normed, packed, qt, bias, numerics=numerics)
+        xd, gd, pd = x.to(dev), gamma.to(dev), packed.to(dev)
+        bd = bias.to(dev) if bias is not None else None
+        got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        if kind == "linear":
+            ops.rmsnorm_linear_into(xd, gd, eps, pd, qt, bd, got, numerics)
+        elif kind == "tiled":
+            ops.rmsnorm_linear_tiled_into(xd, gd, eps, ops.q8_0_tile(pd), bd, got, numerics)
+        else:
+            up = synthetic.make_packed(qt, n, k, seed=9000 + it)
+            want = torch.nn.functional.silu(want) * go.gguf_linear_forward(normed, up, qt, None, numerics=numerics)
+            if kind == "gate_up":
+                ops.rmsnorm_gate_up_silu_into(xd, gd, eps, pd, up.to(dev), qt, got, numerics)
+            else:
+                ops.rmsnorm_gate_up_silu_tiled_into(xd, gd, eps, ops.q8_0_tile(pd), ops.q8_0_tile(up.to(dev)), got, numerics)
+        _ok(got.cpu(), want, tag)
