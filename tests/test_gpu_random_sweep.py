@@ -165,3 +165,52 @@ def test_random_rmsnorm_cases(dev, seed):
             else:
                 ops.rmsnorm_gate_up_silu_tiled_into(xd, gd, eps, ops.q8_0_tile(pd), ops.q8_0_tile(up.to(dev)), got, numerics)
         _ok(got.cpu(), want, tag)
+
+
+@pytest.mark.parametrize("seed", [41])
+def test_random_split_k_cases(dev, seed):
+    """The K-split routes on random shapes with few output tiles: plain (all ten types, the partial sums behind the decoded
+    weights where the kernel does not decode the type itself) and grouped (Q8_0 / Q4_K, all four row-group forms)."""
+    rnd = random.Random(seed)
+    for it in range(40):
+        grouped = rnd.random() < 0.5
+        qt = rnd.choice([go.Q8_0, go.Q4_K]) if grouped else rnd.choice(TYPES)
+        m = rnd.choice([65, 66, 100, 255, 256, 257, 511, 700, 1500])
+        n = rnd.randint(1, 1500)
+        k = 256 * rnd.randint(1, 10) if rnd.random() < 0.7 else 64 * rnd.randint(2, 40) if qt == go.Q8_0 else 256
+        numerics = rnd.choice([0, 1])
+        tag = f"seed={seed} it={it} grouped={grouped} qt={qt} m={m} n={n} k={k} numerics={numerics}"
+        print("case", tag, flush=True)
+        g = torch.Generator().manual_seed(it)
+        x = synthetic.make_activations(m, k, seed=300 + it)
+        und = synthetic.make_packed(qt, n, k, seed=it)
+        bu = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if rnd.random() < 0.5 else None
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(2 * n * k + 4 * 16 * m * n, dtype=torch.uint8, device=dev)
+
+        def put(t):
+            return t.to(dev) if t is not None else None
+
+        if not grouped:
+            want = go.gguf_linear_forward(x, und, qt, bu, numerics=numerics)
+            ops.linear_ws_into(put(x), put(und), qt, put(bu), y, ws, numerics)
+        else:
+            gen = synthetic.make_packed(qt, n, k, seed=7000 + it)
+            bg = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if rnd.random() < 0.5 else None
+            form = rnd.choice(["indicator", "split", "all_text", "all_image"])
+            n_text = rnd.randint(0, m)
+            ind = {"indicator": torch.rand(m, generator=g) < rnd.random(), "split": torch.arange(m) >= n_text,
+                   "all_text": torch.zeros(m, dtype=torch.bool), "all_image": torch.ones(m, dtype=torch.bool)}[form]
+            want = torch.empty((m, n), dtype=torch.bfloat16)
+            if bool((~ind).any()):
+                want[~ind] = go.gguf_linear_forward(x[~ind], und, qt, bu, numerics=numerics)
+            if bool(ind.any()):
+                want[ind] = go.gguf_linear_forward(x[ind], gen, qt, bg, numerics=numerics)
+            row_ws = torch.empty(ops.grouped_workspace_bytes(m), dtype=torch.uint8, device=dev)
+            if form == "split":
+                ops.grouped_linear_ws_into(put(x), None, n_text, put(und), qt, put(gen), qt, put(bu), put(bg), y, None, ws, numerics)
+            else:
+                ops.grouped_linear_ws_into(put(x), put(ind.to(torch.uint8)), 0, put(und), qt, put(gen), qt, put(bu), put(bg), y,
+                                           row_ws, ws, numerics)
+            tag += f" form={form}"
+        _ok(y.cpu(), want, tag)
