@@ -48,7 +48,9 @@ __global__ __launch_bounds__(256) void q8_0_tile_kernel(const uint8_t* __restric
 // grid: row groups; block: W wavefronts that split the K range (GATED: 2 W, the second half on the up matrix).
 // XLDS: the activations (M K bf16) are copied into LDS once per workgroup; otherwise each lane fetches its fragments
 // from global memory one run ahead.
-template <int NUM, bool GATED, int WMAX, bool XLDS>
+// PAIRED (gated): one wavefront works on the gate AND the up matrix of its K range, so that each activation fragment is
+// fetched once for both - with several activation rows those fetches, not the weights, fill the vector memory path.
+template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* __restrict__ x, int M,
                                                                   const uint8_t* __restrict__ ta, const uint8_t* __restrict__ tb,
                                                                   int64_t N, int64_t K, const bf16_t* __restrict__ bias,
@@ -56,10 +58,12 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
                                                                   const bf16_t* __restrict__ gamma, float eps) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
+    constexpr int NQ = PAIRED ? 2 : 1;   // matrices per wavefront
     const int waves = blockDim.x >> 6;
-    const int W = GATED ? waves >> 1 : waves;
-    const int kw = GATED ? (wave >= W ? wave - W : wave) : wave;
-    const uint8_t* __restrict__ t = (GATED && wave >= W) ? tb : ta;
+    const int W = (GATED && !PAIRED) ? waves >> 1 : waves;
+    const int kw = (GATED && !PAIRED) ? (wave >= W ? wave - W : wave) : wave;
+    const uint8_t* __restrict__ t = (GATED && !PAIRED && wave >= W) ? tb : ta;
     const int r = lane & 15, g = lane >> 4;
     const int64_t rg = blockIdx.x, G = (N + 15) >> 4;
     const int runs = (int)(K >> 8);                       // runs of eight blocks
@@ -68,6 +72,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     // checked by the launcher): with 64-bit index arithmetic per request the kernel measured 14.6 instead of 12.6 us.
     const uint8_t* __restrict__ qp = t + rg * (K >> 5) * 512 + 16 * lane;                  // + run * 4096 + pair * 1024
     const uint8_t* __restrict__ sp = t + 16 * G * K + rg * runs * 256 + 16 * r;            // + run * 256
+    const int64_t pair_delta = PAIRED ? tb - ta : 0;                                       // the up matrix, same offsets
 
     const bool has_x = r < M;
     const int xr = has_x ? r : M - 1;   // columns >= M are never stored: those lanes re-read the last activation row
@@ -75,11 +80,16 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     const int xs_stride = 2 * (int)K + 64;                // bytes per activation row in LDS (+64: rows on different banks)
     const uint8_t* xsrow = lds + xr * xs_stride + 16 * g;
 
-    u32x4_t wq[2][4], ws[2], xf[2][8];
+    u32x4_t wq[2][NQ][4], ws[2][NQ], xf[2][8];
     auto fetch = [&](int run, int buf) {
 #pragma unroll
-        for (int p = 0; p < 4; p++) wq[buf][p] = *reinterpret_cast<const u32x4_t*>(qp + (uint32_t)(run * 4096 + p * 1024));
-        ws[buf] = *reinterpret_cast<const u32x4_t*>(sp + (uint32_t)(run * 256));
+        for (int h = 0; h < NQ; h++) {
+            const uint8_t* qh = qp + h * pair_delta;
+            const uint8_t* sh = sp + h * pair_delta;
+#pragma unroll
+            for (int p = 0; p < 4; p++) wq[buf][h][p] = *reinterpret_cast<const u32x4_t*>(qh + (uint32_t)(run * 4096 + p * 1024));
+            ws[buf][h] = *reinterpret_cast<const u32x4_t*>(sh + (uint32_t)(run * 256));
+        }
         if constexpr (!XLDS) {
 #pragma unroll
             for (int b = 0; b < 8; b++) xf[buf][b] = *reinterpret_cast<const u32x4_t*>(xrow + (uint32_t)((run * 8 + b) * 32));
@@ -121,7 +131,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
         __syncthreads();
     }
 
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; q++) acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     auto step = [&](int run, int buf) {
         if (run + 1 < r1) fetch(run + 1, buf ^ 1);
 #pragma unroll
@@ -129,17 +141,20 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const int b = 2 * p + h;
-                const uint32_t sdw = ws[buf][b >> 1];
-                const uint16_t d = (uint16_t)((b & 1) ? (sdw >> 16) : (sdw & 0xFFFFu));
-                uint32_t a0, a1, a2, a3;
-                q8_dword_bf16<NUM>(d, wq[buf][p][2 * h], a0, a1);
-                q8_dword_bf16<NUM>(d, wq[buf][p][2 * h + 1], a2, a3);
-                const u32x4_t a = {a0, a1, a2, a3};
                 u32x4_t xb;
                 if constexpr (XLDS) xb = *reinterpret_cast<const u32x4_t*>(xsrow + (run * 8 + b) * 64);
                 else xb = xf[buf][b];
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                              __builtin_bit_cast(bf16x8_t, xb), acc, 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < NQ; q++) {
+                    const uint32_t sdw = ws[buf][q][b >> 1];
+                    const uint16_t d = (uint16_t)((b & 1) ? (sdw >> 16) : (sdw & 0xFFFFu));
+                    uint32_t a0, a1, a2, a3;
+                    q8_dword_bf16<NUM>(d, wq[buf][q][p][2 * h], a0, a1);
+                    q8_dword_bf16<NUM>(d, wq[buf][q][p][2 * h + 1], a2, a3);
+                    const u32x4_t a = {a0, a1, a2, a3};
+                    acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                                     __builtin_bit_cast(bf16x8_t, xb), acc[q], 0, 0, 0);
+                }
             }
         }
     };
@@ -153,7 +168,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     // ---- add the wavefronts' partial sums (the staged activations are dead: reuse the space) -------------------
     __syncthreads();
     f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [gate partial sums of the W K ranges | up partial sums][64]
-    red[wave * 64 + lane] = acc;
+    red[wave * 64 + lane] = acc[0];
+    if constexpr (PAIRED) red[(W + wave) * 64 + lane] = acc[1];
     __syncthreads();
     if (wave != 0 || !has_x) return;
     // D[i][j]: j = lane % 16 is the activation row, register v holds weight row 4 * (lane / 16) + v
@@ -193,6 +209,11 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
     }
 }
 
+// Rows from which the gated pair runs in the paired mode; measured 12288 x 4096 gate/up, unpaired / paired us:
+// M=1 23.0 / 23.7, M=2 25.9 / 23.7, M=4 26.3 / 23.1, M=8 28.4 / 23.3, M=16 35.0 / 25.4 (8 instead of 4 wavefronts per
+// workgroup in the paired mode: 27.6 - 31.3).
+constexpr int kTiledPairedMinM = 2;
+
 template <int NUM>
 int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, int64_t N, int64_t K, const bf16_t* bias,
                  const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
@@ -203,16 +224,21 @@ int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, i
     int w = gated ? 4 : 8;
     while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 24) w >>= 1;
     if (w > runs) w = runs;
-    const int waves = gated ? 2 * w : w;
     const size_t x_bytes = (size_t)M * (2 * K + 64);
     const bool xlds = x_bytes <= 16 * 1024;
-    const size_t red_bytes = (size_t)waves * 1024;
+    // a gated pair with two activation rows or more: one wavefront takes both matrices
+    const bool paired = gated && M >= kTiledPairedMinM;
+    const int waves = (gated && !paired) ? 2 * w : w;
+    const size_t red_bytes = (size_t)(gated ? 2 * w : w) * 1024;
     if (gamma && !xlds) return SNGGUF_E_BADSHAPE;   // the norm is applied to activations staged in LDS
     const size_t stage_bytes = x_bytes + (gamma ? (((size_t)4 * M * waves + 15) & ~(size_t)15) : 0);
     const size_t lds_bytes = xlds && stage_bytes > red_bytes ? stage_bytes : red_bytes;
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
 #define SNGGUF_LAUNCH(G, XL) gemv_q8_tiled_kernel<NUM, G, 8, XL><<<grid, block, lds_bytes, stream>>>(x, M, ta, tb, N, K, bias, residual, y, gamma, eps)
-    if (gated) {
+    if (paired) {
+        if (xlds) gemv_q8_tiled_kernel<NUM, true, 4, true, true><<<grid, block, lds_bytes, stream>>>(x, M, ta, tb, N, K, bias, residual, y, gamma, eps);
+        else gemv_q8_tiled_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, ta, tb, N, K, bias, residual, y, gamma, eps);
+    } else if (gated) {
         if (xlds) SNGGUF_LAUNCH(true, true);
         else SNGGUF_LAUNCH(true, false);
     } else {

@@ -151,8 +151,7 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
                                               gate_proj.numerics)
             return down_proj(h)
         x = rms_norm(x, norm_weight, eps)
-    # the tiled gated kernel has no paired mode: beyond 8 rows the GGUF-native pair kernel is the faster one
-    tg = gate_proj.tiled_weight() if decode and rows <= 8 else None
+    tg = gate_proj.tiled_weight() if decode else None
     tu = up_proj.tiled_weight() if decode and tg is not None else None
     if tu is not None:
         x2d = x.reshape(-1, gate_proj.in_features)
