@@ -486,7 +486,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     const int spans = (int)(K >> 11);
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
     if (gated && w > 4) w = 4;
-    while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 16) w--;   // plenty of row groups: fewer, longer wavefronts
+    // (no cap for many row groups: a 151936-row projection runs 3 - 5 % faster with two wavefronts per group than with one)
     // stage the activations in LDS when they are small enough to leave room for three workgroups
     // per compute unit (or, for few row groups, one)
     const size_t x_bytes = (size_t)M * (2 * K + 64);

@@ -219,13 +219,16 @@ int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, i
                  const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
     const int64_t groups = (N + 15) / 16;
     const int runs = (int)(K >> 8);
-    // wavefronts per matrix and row group: measured best at 8 (4 for the gated pair, which doubles them); fewer when
-    // the row groups alone fill the chip several times over, never more than there are runs
-    int w = gated ? 4 : 8;
-    while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 24) w >>= 1;
-    if (w > runs) w = runs;
     const size_t x_bytes = (size_t)M * (2 * K + 64);
     const bool xlds = x_bytes <= 16 * 1024;
+    // wavefronts per matrix and row group: measured best at 8 (4 for the gated pair, which doubles them), never more
+    // than there are runs.  With the activations fetched from global memory, fewer when the row groups alone fill the
+    // chip several times over (a 151936-row projection at M = 4: 128 us with one wavefront per group, 159 us with eight);
+    // with them staged in LDS the full count also there (the same projection at M = 1: 109 against 127 us).
+    int w = gated ? 4 : 8;
+    if (!xlds)
+        while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 24) w >>= 1;
+    if (w > runs) w = runs;
     // a gated pair with two activation rows or more: one wavefront takes both matrices
     const bool paired = gated && M >= kTiledPairedMinM;
     const int waves = (gated && !paired) ? 2 * w : w;
