@@ -600,8 +600,11 @@ static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     // The line-aligned variant needs whole 2048-element spans per wavefront; with few row groups
     // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
     // every 256 elements) is the better fit.
+    // (12288 -> 4096, 1536 such wavefronts, block-aligned / line-aligned us: M=1 15.0 / 17.4, M=4 15.9 / 16.3,
+    // M=16 21.6 / 19.3 - with a dozen rows the fewer, longer wavefronts of the line-aligned variant fetch fewer
+    // activation fragments per weight byte in flight, so the bar is lower there; 4096 -> 4096 loses at every M)
     const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
-    if (K % 2048 == 0 && span_waves >= 2048)
+    if (K % 2048 == 0 && span_waves >= (M >= 12 ? 1536 : 2048))
         return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
     return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
 }
