@@ -355,15 +355,15 @@ def main() -> None:
         heads = [synthetic.make_packed(Q8_0, vocab, HIDDEN, seed=9500 + i, device=dev) for i in range(2)]
         xh = synthetic.make_activations(1, HIDDEN, seed=14, device=dev)
         logits = torch.empty((1, vocab), dtype=torch.bfloat16, device=dev)
-        n_h = 32
-        _, ev_h = run_region(lambda i: ops.linear_into(xh, heads[i % 2], Q8_0, None, logits, num), n_h, 4)
+        n_h = 64
+        _, ev_h = run_region(lambda i: ops.linear_into(xh, heads[i % 2], Q8_0, None, logits, num), n_h, 32)
         hb = linear_bytes(1, vocab, HIDDEN)
         t_heads = [ops.q8_0_tile(w) for w in heads]
-        _, ev_ht = run_region(lambda i: ops.linear_tiled_into(xh, t_heads[i % 2], None, None, logits, num), n_h, 4)
+        _, ev_ht = run_region(lambda i: ops.linear_tiled_into(xh, t_heads[i % 2], None, None, logits, num), n_h, 32)
         del t_heads
         gh = (torch.rand(HIDDEN, generator=torch.Generator().manual_seed(15)) + 0.5).to(torch.bfloat16).to(dev)
         # the model's final RMSNorm (modeling_qwen3.py:1183; lm_head at :1264 reads its output) folded into the same launch
-        _, ev_hn = run_region(lambda i: ops.rmsnorm_linear_into(xh, gh, 1e-6, heads[i % 2], Q8_0, None, logits, num), n_h, 4)
+        _, ev_hn = run_region(lambda i: ops.rmsnorm_linear_into(xh, gh, 1e-6, heads[i % 2], Q8_0, None, logits, num), n_h, 32)
         result["lm_head"] = {"workload": "Q8_0 lm_head 4096 -> 151936 at M=1, two weight copies alternating",
                              "bytes_per_launch": hb, "avg_launch_us": round(ev_h / n_h * 1e3, 2),
                              "with_final_norm_fused_us": round(ev_hn / n_h * 1e3, 2),
