@@ -115,6 +115,25 @@ int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
 
 namespace {
 
+// Between the decode kernels' 64 rows and a few hundred, a matrix with few 256 x 256 output tiles keeps only a few
+// compute units busy in the tile kernels, each for K / 64 steps of about 1.6 us, while the decode kernel streams the
+// whole matrix in 10 us + N K / 1.25e12 s per 64 rows (measured: 12288 x 4096 50 us, 4096 x 4096 20 us, 1024 x 4096 19 us) and less for a
+// short last chunk.  Row chunks through the decode kernel win where the sum of those stays below the tile kernel's time:
+// 4096 x 12288 at 128 rows 102 against 292 us, 4096 x 4096 41 against 102 us; 12288 x 4096 only up to 65 rows or so.
+// (Chunks start at multiples of 64 rows, so x, y and the residual keep their 16-byte alignment.)
+bool row_chunks_win(int64_t M, int64_t N, int64_t K, int qtype) {
+    if (K % 256 != 0 || M > 512) return false;
+    const double weights = (double)N * (double)K;
+    const double t16 = 8.0 + weights * (double)sngguf_type_size(qtype) / (double)sngguf_block_size(qtype) / 6.2e6;   // us
+    const double t64_w = 10.0 + weights / 1.25e6;
+    const double t64 = t64_w > 19.0 ? t64_w : 19.0;   // 64 activation rows per 16 weight rows: never below 19 us
+    const int64_t full = M / 64, rem = M % 64;
+    const double last = rem == 0 ? 0.0 : rem <= 16 ? t16 : t16 + (t64 - t16) * (double)(rem - 16) / 48.0;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const double t_tile = (double)((tiles + 255) / 256) * (double)(K / 64) * 1.6;
+    return (double)full * t64 + last < 0.9 * t_tile;
+}
+
 int linear_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
                 const void* residual, void* y, int numerics, void* stream) {
     const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
@@ -125,6 +144,19 @@ int linear_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N, i
     // rows are whole 256-element runs
     if (M <= 16 || (M <= 64 && K % 256 == 0))
         return sngguf::launch_gemv(x, M, q, nullptr, qtype, N, K, bias, residual, y, numerics, false, s);
+    if (row_chunks_win(M, N, K, qtype)) {
+        // a few hundred rows on a matrix with few output tiles: the decode kernel on 64 rows at a time
+        const char* xp = static_cast<const char*>(x);
+        const char* rp = static_cast<const char*>(residual);
+        char* yp = static_cast<char*>(y);
+        for (int64_t r0 = 0; r0 < M; r0 += 64) {
+            const int64_t rows = M - r0 < 64 ? M - r0 : 64;
+            const int rc = sngguf::launch_gemv(xp + 2 * r0 * K, rows, q, nullptr, qtype, N, K, bias,
+                                               rp ? rp + 2 * r0 * N : nullptr, yp + 2 * r0 * N, numerics, false, s);
+            if (rc != SNGGUF_OK) return rc;
+        }
+        return SNGGUF_OK;
+    }
     return sngguf::launch_gemm(x, M, q, qtype, N, K, bias, residual, y, numerics, s);
 }
 
@@ -189,7 +221,9 @@ int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t
             return sngguf::launch_gemm_splitk(x, M, workspace, 30, N, K, bias, y, partial, (int)slices, numerics, s);
         }
     }
-    if (workspace_bytes < 2 * N * K) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
+    // no room for a K split: row chunks through the decode kernel where they beat the few tiles of the dense kernel too
+    if (workspace_bytes < 2 * N * K || row_chunks_win(M, N, K, qtype))
+        return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
     if (rd != SNGGUF_OK) return rd;
     return sngguf::launch_gemm_dense(x, M, workspace, N, K, bias, y, s);

@@ -568,3 +568,28 @@ def test_workspace_routes_replay_in_a_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y1, e1) and torch.equal(y2, e2) and torch.equal(y3, e3), seed
+
+
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K, go.Q6_K, go.Q5_0])
+def test_linear_row_chunks_between_65_and_512_rows(dev, c_oracle, qt):
+    """A few hundred rows on matrices with few output tiles run as 64-row chunks through the decode kernel (no
+    workspace): whole and partial last chunks, bias, residual, ragged N, both numerics."""
+    print(f"case row_chunks qt={qt}", flush=True)
+    for numerics, (m, n, k) in [(1, (65, 1024, 4096)), (0, (128, 4096, 4096)), (1, (200, 515, 2048)), (1, (256, 1030, 12288)),
+                                (0, (321, 64, 4096))]:
+        packed = synthetic.make_packed(qt, n, k, seed=m + n + qt)
+        x = synthetic.make_activations(m, k, seed=m)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16) if n % 2 else None
+        res = synthetic.make_activations(m, n, seed=m + 1)
+        want = go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics)
+        xd, pd = x.to(dev), packed.to(dev)
+        bd = bias.to(dev) if bias is not None else None
+        got = ops.linear(xd, pd, qt, bd, numerics)
+        _check(got.cpu(), want)
+        got_r = ops.linear_residual(xd, pd, qt, res.to(dev), bd, numerics)
+        _check(got_r.cpu(), (res.float() + want.float()).to(torch.bfloat16))
+        if (m, n, k) in ((65, 1024, 4096), (128, 4096, 4096)):
+            # these two are chunked for certain (19 - 47 us of decode kernel against ~100 us of tile kernel): the chunks
+            # are the decode kernel's own results on those rows
+            hi = min(m, 128)
+            assert torch.equal(got[64:hi], ops.linear(xd[64:hi].contiguous(), pd, qt, bd, numerics))
