@@ -109,7 +109,7 @@ int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols,
  * fp32, bias is added in fp32 and the sum is rounded once to bf16.  M <= 16 takes the fused
  * dequant-GEMV (packed bytes streamed once, nothing dequantized is written to memory);
  * larger M takes the LDS-staged dequant-GEMM on bf16 MFMA.
-  * Rows beyond the decode kernels' 64 go to the tile GEMM kernels, except that a few hundred rows on a matrix with few
+ * Rows beyond the decode kernels' 64 go to the tile GEMM kernels, except that a few hundred rows on a matrix with few
  * 256 x 256 output tiles (K % 256 == 0) run as 64-row chunks through the decode kernel where that is faster.
  */
 int sngguf_linear(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
