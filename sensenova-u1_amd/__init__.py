@@ -9,6 +9,7 @@ from .quantized_linear import (
     GGUFLinear,
     GGUFParameter,
     dequantize_gguf_tensor,
+    set_decode_layout,
 )
 
 __all__ = [
@@ -16,5 +17,5 @@ __all__ = [
     "load_gguf_checkpoint", "set_gguf2meta_model", "match_state_dict", "count_gguf_linear",
     "GGUFLinear", "GGUFParameter", "SUPPORTED_GGUF_QUANT_TYPES", "dequantize_gguf_tensor",
     "grouped_linear", "find_mot_pairs", "gated_mlp", "FusedProjections", "NativeGGUFReader",
-    "LayerOffloadWrapper", "PackedLayerStore", "AsyncPrefetcher",
+    "LayerOffloadWrapper", "PackedLayerStore", "AsyncPrefetcher", "set_decode_layout",
 ]

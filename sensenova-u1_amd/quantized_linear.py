@@ -123,6 +123,27 @@ def dequantize_gguf_tensor(tensor: torch.Tensor, dtype: Optional[torch.dtype] = 
     return ops.dequantize(tensor, int(tensor.quant_type), dtype, numerics)
 
 
+def set_decode_layout(model: nn.Module, layout: str = "tiled", build_now: bool = False) -> int:
+    """Set ``decode_layout`` on every ``GGUFLinear`` below ``model`` (including ``model`` itself) and return how many
+    were switched.  ``"tiled"`` makes the decode path (at most 16 rows) of Q8_0 modules whose ``in_features`` is a
+    multiple of 256 read an operand-order copy of the weight, built on first use - or right away with ``build_now``
+    for weights that are already on the device - and kept beside the GGUF rows (the same number of bytes again);
+    ``"native"`` switches back and releases the copies."""
+    if layout not in ("native", "tiled"):
+        raise ValueError(f"decode layout is {layout!r}; expected 'native' or 'tiled'")
+    count = 0
+    for mod in model.modules():
+        if type(mod).__name__ != "GGUFLinear":
+            continue
+        mod.decode_layout = layout
+        if layout == "native":
+            mod.drop_tiled_cache()
+        elif build_now:
+            mod.tiled_weight()
+        count += 1
+    return count
+
+
 def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMSNorm as the decoder layers compute it (``Qwen3RMSNorm.forward``, ``modeling_qwen3.py:192-197``): statistic
     and scaling in fp32, one rounding to the input dtype, then the product with the weight in that dtype."""

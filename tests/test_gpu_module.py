@@ -328,3 +328,22 @@ def test_auto_policy_between_65_and_256_rows(dev, qt):
             mod.gemm_policy = policy
             got = mod(x.to(dev))
             assert go.rel_l2(got.cpu(), want) <= TOL, (rows, policy)
+
+
+def test_set_decode_layout_on_a_loaded_model(tmp_path, dev):
+    """The whole model switched to the tiled decode layout: copies built at once, decode outputs as on the GGUF rows up
+    to the summation order, larger inputs untouched."""
+    from sensenova_u1_amd import set_decode_layout
+    model, _ = _load(tmp_path, dev, 8)
+    x = synthetic.make_activations(3, H, seed=5).to(dev)
+    big = synthetic.make_activations(70, H, seed=6).to(dev)
+    mods = [m for m in model.modules() if type(m).__name__ == "GGUFLinear" and m.in_features == H]
+    before = [m(x) for m in mods]
+    before_big = [m(big) for m in mods]
+    assert set_decode_layout(model, "tiled", build_now=True) >= len(mods)
+    assert any(m.tiled_weight() is not None for m in mods) == (H % 256 == 0)
+    for m, want, want_big in zip(mods, before, before_big):
+        assert go.rel_l2(m(x).cpu(), want.cpu()) <= 2e-4
+        assert torch.equal(m(big), want_big)
+    set_decode_layout(model, "native")
+    assert all(m._tiled_cache is None for m in mods)

@@ -219,3 +219,21 @@ def test_find_mot_pairs(tmp_path):
                           ("q_proj", "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")}
     und, gen = pairs["layers.1.mlp.down_proj"]
     assert und is model.layers[1].mlp.down_proj and gen is model.layers[1].mlp.down_proj_mot_gen
+
+
+def test_set_decode_layout_walks_the_model(tmp_path):
+    """set_decode_layout switches every GGUFLinear (and nothing else); on a CPU host nothing is built."""
+    from sensenova_u1_amd import set_decode_layout
+    path = str(tmp_path / "m.gguf")
+    _make_file(path, 8)
+    sd = load_gguf_checkpoint(path)
+    with torch.device("meta"):
+        model = TinyModel()
+    model = set_gguf2meta_model(model, sd, torch.bfloat16, "cpu")
+    n = count_gguf_linear(model)
+    assert set_decode_layout(model, "tiled") == n > 0
+    assert all(m.decode_layout == "tiled" for m in model.modules() if type(m).__name__ == "GGUFLinear")
+    assert all(m.tiled_weight() is None for m in model.modules() if type(m).__name__ == "GGUFLinear")   # weights on the CPU
+    assert set_decode_layout(model, "native") == n
+    with pytest.raises(ValueError):
+        set_decode_layout(model, "blocked")
