@@ -228,6 +228,9 @@ int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, i
     int w = gated ? 4 : 8;
     if (!xlds)
         while (w > 1 && groups * w * (gated ? 2 : 1) > 256 * 24) w >>= 1;
+    // a dozen rows or more on a long K (12288 -> 4096 at M = 16: 17.4 us with four wavefronts per group, 18.5 with eight,
+    // 22.5 with two): fewer wavefronts fetch the activation fragments of fewer K ranges at a time
+    if (!gated && !xlds && M >= 12 && runs >= 32 && w > 4) w = 4;
     if (w > runs) w = runs;
     // a gated pair with two activation rows or more: one wavefront takes both matrices
     const bool paired = gated && M >= kTiledPairedMinM;
