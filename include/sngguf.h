@@ -35,7 +35,11 @@ enum {
     SNGGUF_TYPE_Q3_K = 11, /* 256 elements / 110 bytes: u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d */
     SNGGUF_TYPE_Q4_K = 12, /* 256 elements / 144 bytes: f16 d, dmin; u8 scales[12]; u8 qs[128]  */
     SNGGUF_TYPE_Q5_K = 13, /* 256 elements / 176 bytes: f16 d, dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] */
-    SNGGUF_TYPE_Q6_K = 14  /* 256 elements / 210 bytes: u8 ql[128]; u8 qh[64]; i8 sc[16]; f16 d */
+    SNGGUF_TYPE_Q6_K = 14, /* 256 elements / 210 bytes: u8 ql[128]; u8 qh[64]; i8 sc[16]; f16 d */
+    SNGGUF_TYPE_BF16 = 30  /* 1 element / 2 bytes: plain bfloat16 rows (upstream wraps BF16 tensors in a GGUFParameter
+                              too and decodes them with dequantize_blocks_BF16: exact in either numerics mode).  Taken by
+                              sngguf_dequantize, sngguf_linear[_residual | _ws], sngguf_gate_up_silu and, with
+                              K % 64 == 0, the grouped launchers; not by the fused-norm and tiled-layout entry points */
 };
 
 /* element type of the `out` buffer of sngguf_dequantize */

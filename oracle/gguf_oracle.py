@@ -33,13 +33,14 @@ import numpy as np
 import torch
 
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 2, 3, 6, 7, 8, 10, 11, 12, 13, 14
+BF16 = 30
 QK_K = 256
 K_SCALE_SIZE = 12
 # gguf.GGML_QUANT_SIZES: type -> (elements per block, bytes per block)
 GGML_QUANT_SIZES = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
-                    Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
+                    Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), BF16: (1, 2)}
 TYPE_NAMES = {Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q8_0", Q2_K: "Q2_K", Q3_K: "Q3_K",
-              Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
+              Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", BF16: "BF16"}
 
 NUM_GGML_FP32 = 0
 NUM_UPSTREAM_FP16 = 1
@@ -209,7 +210,12 @@ def dequantize_blocks_Q6_K(blocks, block_size, type_size, dtype=None):
     return (d * q).reshape((n_blocks, QK_K))
 
 
-dequantize_functions = {Q4_0: dequantize_blocks_Q4_0, Q4_1: dequantize_blocks_Q4_1, Q5_0: dequantize_blocks_Q5_0,
+def dequantize_blocks_BF16(blocks, block_size, type_size, dtype=None):
+    """bf16 bit patterns widened to fp32 (exact): the result is fp32 whatever ``dtype`` says, as upstream's is."""
+    return (blocks.contiguous().view(torch.int16).to(torch.int32) << 16).view(torch.float32)
+
+
+dequantize_functions = {BF16: dequantize_blocks_BF16, Q4_0: dequantize_blocks_Q4_0, Q4_1: dequantize_blocks_Q4_1, Q5_0: dequantize_blocks_Q5_0,
                         Q5_1: dequantize_blocks_Q5_1, Q8_0: dequantize_blocks_Q8_0, Q2_K: dequantize_blocks_Q2_K,
                         Q3_K: dequantize_blocks_Q3_K, Q4_K: dequantize_blocks_Q4_K, Q5_K: dequantize_blocks_Q5_K,
                         Q6_K: dequantize_blocks_Q6_K}

@@ -372,11 +372,20 @@ void sno_dequantize_row_q3_K(const uint8_t* src, float* y, int64_t k, int numeri
 }
 
 
+/* BF16 (type 30; upstream dequantize_blocks_BF16): "blocks" of one element, two bytes; the
+ * value is the bf16 bit pattern shifted into the upper half of an fp32 word - exact, no
+ * rounding in either numerics mode. */
+void sno_dequantize_row_bf16(const uint8_t* src, float* y, int64_t k, int numerics) {
+    (void)numerics;
+    for (int64_t i = 0; i < k; i++) y[i] = u32_as_f32((uint32_t)rd16(src + 2 * i) << 16);
+}
+
 /* ggml type enum -> bytes / elements per block (0: not restated here) */
 int64_t sno_type_size(int qtype) {
     switch (qtype) {
     case 2: return 18; case 3: return 20; case 6: return 22; case 7: return 24; case 8: return 34;
     case 10: return 84; case 11: return 110; case 12: return 144; case 13: return 176; case 14: return 210;
+    case 30: return 2;
     default: return 0;
     }
 }
@@ -384,6 +393,7 @@ int64_t sno_block_size(int qtype) {
     switch (qtype) {
     case 2: case 3: case 6: case 7: case 8: return 32;
     case 10: case 11: case 12: case 13: case 14: return 256;
+    case 30: return 1;
     default: return 0;
     }
 }
@@ -400,6 +410,7 @@ static int dequant_row(const uint8_t* src, int qtype, float* y, int64_t k, int n
     case 12: sno_dequantize_row_q4_K(src, y, k, numerics); return 0;
     case 13: sno_dequantize_row_q5_K(src, y, k, numerics); return 0;
     case 14: sno_dequantize_row_q6_K(src, y, k, numerics); return 0;
+    case 30: sno_dequantize_row_bf16(src, y, k, numerics); return 0;
     default: return -1;
     }
 }

@@ -16,6 +16,9 @@ int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
                         const void* gamma, float eps);
+int launch_dequantize_bf16(const void* q, int64_t rows, int64_t cols, void* out, int out_dtype, hipStream_t stream);
+int launch_gemv_bf16(const void* x, int64_t M, const void* wa, const void* wb, int64_t N, int64_t K, const void* bias,
+                     const void* residual, void* y, bool gated, hipStream_t stream);
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
 int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
@@ -87,6 +90,7 @@ int64_t sngguf_type_size(int qtype) {
     case SNGGUF_TYPE_Q4_K: return 144;
     case SNGGUF_TYPE_Q5_K: return 176;
     case SNGGUF_TYPE_Q6_K: return 210;
+    case SNGGUF_TYPE_BF16: return 2;
     default: return 0;
     }
 }
@@ -97,6 +101,7 @@ int64_t sngguf_block_size(int qtype) {
         return 32;
     case SNGGUF_TYPE_Q2_K: case SNGGUF_TYPE_Q3_K: case SNGGUF_TYPE_Q4_K: case SNGGUF_TYPE_Q5_K: case SNGGUF_TYPE_Q6_K:
         return 256;
+    case SNGGUF_TYPE_BF16: return 1;
     default: return 0;
     }
 }
@@ -110,6 +115,8 @@ int sngguf_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void
     if (rows == 0 || cols == 0) return SNGGUF_OK;
     if (!q || !out) return SNGGUF_E_NULLPTR;
     if (!aligned(q, 16) || !aligned(out, 16)) return SNGGUF_E_ALIGN;
+    if (qtype == SNGGUF_TYPE_BF16)
+        return sngguf::launch_dequantize_bf16(q, rows, cols, out, out_dtype, static_cast<hipStream_t>(stream));
     return sngguf::launch_dequantize(q, qtype, rows, cols, out, out_dtype, numerics, static_cast<hipStream_t>(stream));
 }
 
@@ -140,6 +147,23 @@ int linear_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N, i
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (residual && !aligned(residual, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (qtype == SNGGUF_TYPE_BF16) {
+        // plain bf16 rows: the decode-sized kernel up to 16 rows, the tile kernel's dense form beyond (whole K steps,
+        // 32-bit activation offsets), else 16 rows at a time
+        if (M > 16 && K % 64 == 0 && M * K < ((int64_t)1 << 31))
+            return sngguf::launch_gemm(x, M, q, 30, N, K, bias, residual, y, numerics, s);
+        const char* xp = static_cast<const char*>(x);
+        const char* rp = static_cast<const char*>(residual);
+        char* yp = static_cast<char*>(y);
+        for (int64_t r0 = 0; r0 < M; r0 += 16) {
+            const int64_t rows = M - r0 < 16 ? M - r0 : 16;
+            // (with an odd K the rows of x are only 2-byte aligned; the kernel then reads single elements)
+            const int rc = sngguf::launch_gemv_bf16(xp + 2 * r0 * K, rows, q, nullptr, N, K, bias, rp ? rp + 2 * r0 * N : nullptr,
+                                                    yp + 2 * r0 * N, false, s);
+            if (rc != SNGGUF_OK) return rc;
+        }
+        return SNGGUF_OK;
+    }
     // decode-shaped work (weights streamed and decoded once): up to 16 rows always, up to 64 rows when the
     // rows are whole 256-element runs
     if (M <= 16 || (M <= 64 && K % 256 == 0))
@@ -194,8 +218,8 @@ int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // everything that does not fit the dense route runs as sngguf_linear does
-    const bool fits = workspace && dense_route_fits(M, N, K);
+    // everything that does not fit the dense route runs as sngguf_linear does (plain bf16 rows need no weight pass)
+    const bool fits = workspace && dense_route_fits(M, N, K) && qtype != SNGGUF_TYPE_BF16;
     if (!fits) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     // Few output tiles (a few hundred rows, or a narrow matrix): a 256 x 256 tile takes as long per K step whether
     // or not the other compute units have work, so K is split over enough workgroups to occupy them, with the fp32
@@ -236,12 +260,14 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (!q_up) return SNGGUF_E_NULLPTR;
     if (!aligned(q_up, 16)) return SNGGUF_E_ALIGN;
     if (M > 16) return SNGGUF_E_BADSHAPE;
+    if (qtype == SNGGUF_TYPE_BF16)
+        return sngguf::launch_gemv_bf16(x, M, q_gate, q_up, N, K, nullptr, nullptr, h, true, static_cast<hipStream_t>(stream));
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
 }
 
 int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K) {
     // the fused norm works on activations staged in LDS: rows of whole 256-element runs, M (2 K + 64) <= 16 KB
-    return known_type(qtype) && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
+    return known_type(qtype) && qtype != SNGGUF_TYPE_BF16 && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
 }
 
 namespace {
@@ -372,6 +398,9 @@ int sngguf_grouped_linear(const void* x, int64_t M, const uint8_t* indicator, in
     } else if (n_text < 0 || n_text > M) {
         return SNGGUF_E_BADSHAPE;
     }
+    // plain bf16 rows run on the tile kernel's dense form only: whole K steps, 32-bit activation offsets
+    if ((qtype_und == SNGGUF_TYPE_BF16 || qtype_gen == SNGGUF_TYPE_BF16) && (K % 64 != 0 || M * K >= ((int64_t)1 << 31)))
+        return SNGGUF_E_BADSHAPE;
     return sngguf::launch_grouped_gemm(x, M, indicator, n_text, q_und, qtype_und, q_gen, qtype_gen, N, K, bias_und,
                                        bias_gen, y, workspace, numerics, static_cast<hipStream_t>(stream));
 }
@@ -426,9 +455,11 @@ int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator,
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint8_t* w_und = static_cast<uint8_t*>(dense_workspace);
     uint8_t* w_gen = w_und + 2 * N * K;
-    rc = sngguf::launch_dequantize(q_und, qtype_und, N, K, w_und, SNGGUF_OUT_BF16, numerics, s);
+    rc = qtype_und == SNGGUF_TYPE_BF16 ? sngguf::launch_dequantize_bf16(q_und, N, K, w_und, SNGGUF_OUT_BF16, s)
+                                       : sngguf::launch_dequantize(q_und, qtype_und, N, K, w_und, SNGGUF_OUT_BF16, numerics, s);
     if (rc != SNGGUF_OK) return rc;
-    rc = sngguf::launch_dequantize(q_gen, qtype_gen, N, K, w_gen, SNGGUF_OUT_BF16, numerics, s);
+    rc = qtype_gen == SNGGUF_TYPE_BF16 ? sngguf::launch_dequantize_bf16(q_gen, N, K, w_gen, SNGGUF_OUT_BF16, s)
+                                       : sngguf::launch_dequantize(q_gen, qtype_gen, N, K, w_gen, SNGGUF_OUT_BF16, numerics, s);
     if (rc != SNGGUF_OK) return rc;
     return sngguf::launch_grouped_gemm(x, M, indicator, n_text, w_und, 30, w_gen, 30, N, K, bias_und, bias_gen, y, workspace,
                                        numerics, s);

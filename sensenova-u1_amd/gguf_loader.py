@@ -7,6 +7,9 @@ Same three functions, signatures, tensor-name mapping (identity) and error behav
     load_gguf_checkpoint(path) -> dict[str, Tensor | GGUFParameter]        (reference :17-47)
     set_gguf2meta_model(meta_model, state_dict, dtype, device) -> nn.Module (reference :50-85)
     match_state_dict(meta_model, state_dict, show_num=10) -> dict           (reference :88-114)
+
+plus ``load_gguf_model``, the one-call form of the sequence the reference's model loader runs around them
+(``src/sensenova_u1/utils/checkpoint_loading.py:288-323``).
 """
 from __future__ import annotations
 
@@ -33,7 +36,9 @@ def load_gguf_checkpoint(gguf_checkpoint_path: str, pin_memory: bool = False, th
 
     F32 / F16 tensors come back as plain torch tensors; every other type must be one the HIP
     kernels decode and is wrapped in ``GGUFParameter`` (packed bytes, copied out of the file
-    mapping).  Tensor names are used verbatim: GGUF names are the model's state-dict keys.
+    mapping).  That includes BF16, as in the reference (``gguf_loader.py:37-43``: only F32 and F16
+    are exempt from the supported-types check and the wrapping).  Tensor names are used
+    verbatim: GGUF names are the model's state-dict keys.
 
     The file is parsed by the library's C++ reader and all payloads are copied in one
     multi-threaded pass into freshly allocated host tensors - page-locked ones with
@@ -84,6 +89,11 @@ def _load_state_dict_into_meta(model: nn.Module, state_dict: dict, dtype: torch.
         module, leaf = _split_param_name(model, name)
         is_buffer = leaf in module._buffers
         slot = module._buffers[leaf] if is_buffer else module._parameters[leaf]
+        if isinstance(value, GGUFParameter) and value.quant_type == GGMLQuantizationType.BF16 \
+                and not (type(module).__name__ == GGUFLinear.__name__ and leaf == "weight"):
+            # a BF16 tensor outside a quantized linear (norm weight, embedding, bias ...): nothing would decode it at
+            # forward time, so it is decoded here - a reinterpretation of the two-byte elements, no arithmetic
+            value = value.as_tensor().view(torch.bfloat16)
         if isinstance(value, GGUFParameter):
             block_size, type_size = GGML_QUANT_SIZES[value.quant_type]
             inferred = _quant_shape_from_byte_shape(value.shape, type_size, block_size)
@@ -157,3 +167,51 @@ def count_gguf_linear(model: nn.Module) -> int:
     """Number of active ``GGUFLinear`` modules, found by type name as the reference's sanity
     check does (``src/sensenova_u1/utils/checkpoint_loading.py:315``)."""
     return sum(1 for m in model.modules() if type(m).__name__ == GGUFLinear.__name__)
+
+
+def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.dtype,
+                    device: str | torch.device | None, model_factory=None) -> nn.Module:
+    """The whole GGUF branch of the reference's model loader in one call
+    (``_load_from_gguf``, ``src/sensenova_u1/utils/checkpoint_loading.py:288-323``): build the model without
+    storage, parse the file, swap the quantized linears in and place the tensors on ``device``, report how many
+    ``GGUFLinear`` modules are active - with the reference's warning when there are none - and return the model
+    in eval mode.
+
+    ``config_or_meta_model`` is either a model that already lives on the meta device, or a config: then
+    ``model_factory(config)`` is called under ``torch.device("meta")``, and without a factory the reference's own
+    construction is used (``transformers.AutoModel.from_config`` under ``accelerate.init_empty_weights``).
+    """
+    print(f"[gguf] loading quantized checkpoint from {gguf_checkpoint}")
+    if isinstance(config_or_meta_model, nn.Module):
+        model = config_or_meta_model
+        on_storage = [n for n, p in model.named_parameters() if p.device.type != "meta"]
+        if on_storage:
+            raise ValueError(f"load_gguf_model needs a meta-initialized model; {on_storage[0]} already has storage")
+    elif model_factory is not None:
+        with torch.device("meta"):
+            model = model_factory(config_or_meta_model)
+    else:
+        try:
+            from accelerate import init_empty_weights
+        except ImportError as exc:
+            raise RuntimeError("GGUF loading requires `accelerate`; install it in your environment.") from exc
+        from transformers import AutoModel
+
+        with init_empty_weights():
+            model = AutoModel.from_config(config_or_meta_model)
+
+    state_dict = load_gguf_checkpoint(gguf_checkpoint)
+    print(f"[gguf] parsed {len(state_dict)} tensors")
+    target_device = torch.device(device) if isinstance(device, str) else device
+    set_gguf2meta_model(model, state_dict, dtype, target_device)
+
+    n_gguf_linear = count_gguf_linear(model)
+    print(f"[gguf] {n_gguf_linear} GGUFLinear modules active (HIP dequant-GEMV / dequant-GEMM at forward time)")
+    if n_gguf_linear == 0:
+        print("[gguf] WARNING: no GGUFLinear modules found — no Linear of the model has a quantized weight in the file")
+
+    del state_dict
+    gc.collect()
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+    return model.eval()

@@ -138,8 +138,11 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     if norm_weight is not None:
         if (decode and x.is_cuda and norm_weight.dtype == torch.bfloat16
                 and ops.rmsnorm_fits(int(gate_proj.weight.quant_type), rows, gate_proj.in_features)):
-            x2d = x.reshape(-1, gate_proj.in_features)
-            x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
+            x2d = gate_proj._checked_rows(x, norm_weight)
+            up_proj._checked_rows(x)
+            if (up_proj.in_features, up_proj.out_features) != (gate_proj.in_features, gate_proj.out_features) \
+                    or norm_weight.numel() != gate_proj.in_features:
+                raise ops.SnGgufError("gated_mlp: gate, up and the norm weight differ in shape")
             h = torch.empty((*x.shape[:-1], gate_proj.out_features), dtype=torch.bfloat16, device=x.device)
             tg, tu = gate_proj.tiled_weight(), up_proj.tiled_weight()
             if tg is not None and tu is not None:
@@ -154,10 +157,12 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     tg = gate_proj.tiled_weight() if decode else None
     tu = up_proj.tiled_weight() if decode and tg is not None else None
     if tu is not None:
-        x2d = x.reshape(-1, gate_proj.in_features)
+        x2d = gate_proj._checked_rows(x)
+        up_proj._checked_rows(x)
+        if up_proj.out_features != gate_proj.out_features:
+            raise ops.SnGgufError("gated_mlp: gate and up differ in shape")
         h = torch.empty((*x.shape[:-1], gate_proj.out_features), dtype=torch.bfloat16, device=x.device)
-        ops.gate_up_silu_tiled_into(x2d if x2d.is_contiguous() else x2d.contiguous(), tg, tu,
-                                    h.view(-1, gate_proj.out_features), gate_proj.numerics)
+        ops.gate_up_silu_tiled_into(x2d, tg, tu, h.view(-1, gate_proj.out_features), gate_proj.numerics)
     elif decode and gate_proj.in_features % 64 == 0:
         h = ops.gate_up_silu(x, gate_proj.weight, up_proj.weight, int(gate_proj.weight.quant_type), gate_proj.numerics)
     else:

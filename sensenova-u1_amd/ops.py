@@ -24,10 +24,11 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libsngguf.so")
 
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 2, 3, 6, 7, 8, 10, 11, 12, 13, 14
+BF16 = 30   # plain bfloat16 rows, a GGUF tensor type like the others: blocks of one element, two bytes
 NUM_GGML_FP32, NUM_UPSTREAM_FP16 = 0, 1
 # type -> (block elements, block bytes)
 GGML_QUANT_SIZES = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
-                    Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
+                    Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), BF16: (1, 2)}
 _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
@@ -161,7 +162,7 @@ def _ptr(t: Optional[torch.Tensor]):
 def _packed_2d(packed: torch.Tensor, quant_type: int):
     """View the packed weight as uint8 [N, row_bytes]; returns (tensor, N, K)."""
     if quant_type not in GGML_QUANT_SIZES:
-        raise SnGgufError(f"quant type {quant_type} is not implemented (have Q4_0=2, Q4_1=3, Q5_0=6, Q5_1=7, Q8_0=8, Q2_K=10, Q3_K=11, Q4_K=12, Q5_K=13, Q6_K=14)")
+        raise SnGgufError(f"quant type {quant_type} is not implemented (have Q4_0=2, Q4_1=3, Q5_0=6, Q5_1=7, Q8_0=8, Q2_K=10, Q3_K=11, Q4_K=12, Q5_K=13, Q6_K=14, BF16=30)")
     bs, ts = GGML_QUANT_SIZES[quant_type]
     p = packed.detach()
     if p.dtype != torch.uint8:

@@ -32,6 +32,7 @@ SUPPORTED_GGUF_QUANT_TYPES = (
     GGMLQuantizationType.Q4_K,
     GGMLQuantizationType.Q5_K,
     GGMLQuantizationType.Q6_K,
+    GGMLQuantizationType.BF16,   # upstream lists it too: a BF16 tensor is wrapped and decoded like a quantized one
 )
 
 
@@ -119,7 +120,9 @@ def dequantize_gguf_tensor(tensor: torch.Tensor, dtype: Optional[torch.dtype] = 
     if not hasattr(tensor, "quant_type"):
         return tensor
     if dtype is None:
-        dtype = torch.float16 if numerics == ops.NUM_UPSTREAM_FP16 else torch.float32
+        # (upstream's BF16 decode returns fp32 whatever the mode)
+        plain = int(tensor.quant_type) == ops.BF16
+        dtype = torch.float16 if numerics == ops.NUM_UPSTREAM_FP16 and not plain else torch.float32
     return ops.dequantize(tensor, int(tensor.quant_type), dtype, numerics)
 
 
@@ -172,12 +175,14 @@ class GGUFLinear(nn.Linear):
     * ``"resident"``: as ``"two_pass"``, but the bf16 weight is kept (2 * N * K bytes per module) and
       reused by later calls until the packed bytes move or change: for towers that see thousands of
       rows many times over (the denoising loop) on a device with memory to spare, it removes the
-      weight pass from every call but the first.  Not meant to be combined with layer offloading.
+      weight pass from every call but the first.  Not meant to be combined with layer offloading; after an in-place
+      rewrite of the packed bytes through ``weight.data`` call ``weights_changed()``.
 
     ``decode_layout = "tiled"`` (Q8_0 with ``in_features`` a multiple of 256 only; default ``"native"``) makes the
     decode calls (at most 16 rows) read an operand-order copy of the weight that is built on first use and kept
     beside the GGUF bytes (the same 34 bytes per block again): 8 - 10 % faster on the M = 1 MLP step, for models
-    that stay resident on the device.  The copy follows the packed bytes: it is rebuilt when they move or change.
+    that stay resident on the device.  The copy follows the packed bytes: it is rebuilt when they move, and after
+    ``weights_changed()`` when they were rewritten in place through ``weight.data``.
 
     Other compute dtypes always take dequantize + matmul.
     """
@@ -198,6 +203,19 @@ class GGUFLinear(nn.Linear):
         if not hasattr(w, "quant_type"):
             raise RuntimeError("GGUFLinear.weight is not a GGUFParameter (no quant_type); was the checkpoint loaded?")
         return int(w.quant_type)
+
+    def _checked_rows(self, inputs: torch.Tensor, *others: Optional[torch.Tensor]) -> torch.Tensor:
+        """``inputs`` as contiguous bf16 rows ``[M, in_features]`` for a raw library call, after the checks the custom
+        ops make: every tensor (inputs, weight, bias, ``others``) on one HIP device, the packed weight a whole
+        number of blocks of shape ``[out_features, in_features]``, the input's last dim ``in_features``.  Raises
+        ``SnGgufError`` before anything is launched - a host pointer handed to a kernel is a GPU memory fault."""
+        ops._require_device(inputs, self.weight, self.bias, *others)
+        _, n, k = ops._packed_2d(self.weight, self._weight_type())
+        if (n, k) != (self.out_features, self.in_features):
+            raise ops.SnGgufError(f"GGUFLinear: packed weight decodes to {(n, k)}, the module is {(self.out_features, self.in_features)}")
+        if not self.weight.is_contiguous():
+            raise ops.SnGgufError("GGUFLinear: the packed weight must be contiguous")
+        return ops._as_bf16_rows(inputs, self.in_features, "GGUFLinear")
 
     def tiled_weight(self) -> Optional[torch.Tensor]:
         """The operand-order copy of the weight when ``decode_layout == "tiled"`` applies to this module (Q8_0,
@@ -220,10 +238,11 @@ class GGUFLinear(nn.Linear):
         tiled = self.tiled_weight()
         if tiled is None:
             return None
-        x2d = inputs.reshape(-1, self.in_features)
-        x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
+        x2d = self._checked_rows(inputs, residual)
         out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
         bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
+        if residual is not None and (residual.dtype != torch.bfloat16 or tuple(residual.shape) != tuple(out.shape)):
+            raise ops.SnGgufError(f"GGUFLinear: residual must be bf16 of shape {tuple(out.shape)}")
         res2d = residual.reshape(-1, self.out_features).contiguous() if residual is not None else None
         ops.linear_tiled_into(x2d, tiled, bias, res2d, out.view(-1, self.out_features), self.numerics)
         return out
@@ -239,12 +258,12 @@ class GGUFLinear(nn.Linear):
                 out = self._decode_tiled(inputs, None)
                 if out is not None:
                     return out
-            if rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused":
+            if rows <= 16 or (rows <= 64 and self.in_features % 256 == 0) or self.gemm_policy == "fused" or qtype == ops.BF16:
                 return ops.linear(inputs, self.weight, qtype, self.bias, self.numerics)
             if self.gemm_policy not in ("auto", "two_pass", "resident"):
                 raise ValueError(f"GGUFLinear.gemm_policy is {self.gemm_policy!r}; expected 'auto', 'two_pass', 'fused' or 'resident'")
+            x2d = self._checked_rows(inputs)
             out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
-            x2d = inputs.reshape(-1, self.in_features)
             tiles = (self.out_features + 255) // 256     # output tiles of 256 x 256 for up to 256 rows
             split_k = (self.gemm_policy == "auto" and rows <= 256 and tiles <= 128 and self.in_features >= 256
                        and self.in_features % 64 == 0 and qtype in (ops.Q8_0, ops.Q4_K))
@@ -253,12 +272,11 @@ class GGUFLinear(nn.Linear):
                 nbytes = min(2 * self.out_features * self.in_features, 4 * max(2, 256 // tiles) * rows * self.out_features)
                 workspace = torch.empty(nbytes, dtype=torch.uint8, device=inputs.device)
                 bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
-                ops.linear_ws_into(x2d if x2d.is_contiguous() else x2d.contiguous(), self.weight, qtype, bias,
-                                   out.view(-1, self.out_features), workspace, self.numerics)
+                ops.linear_ws_into(x2d, self.weight, qtype, bias, out.view(-1, self.out_features), workspace, self.numerics)
             else:
                 self.two_pass_into(x2d, out.view(-1, self.out_features))
             return out
-        weight = ops.dequantize(self.weight, qtype, torch.float16 if self.numerics == ops.NUM_UPSTREAM_FP16
+        weight = ops.dequantize(self.weight, qtype, torch.float16 if self.numerics == ops.NUM_UPSTREAM_FP16 and qtype != ops.BF16
                                 else torch.float32, self.numerics).to(compute_dtype)
         bias = self.bias.to(compute_dtype) if self.bias is not None else None
         return torch.nn.functional.linear(inputs, weight, bias)
@@ -274,8 +292,9 @@ class GGUFLinear(nn.Linear):
                  and ops.rmsnorm_fits(int(self.weight.quant_type), rows, self.in_features))
         if not fused:
             return self.forward(rms_norm(inputs, norm_weight, eps))
-        x2d = inputs.reshape(-1, self.in_features)
-        x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
+        x2d = self._checked_rows(inputs, norm_weight)
+        if norm_weight.numel() != self.in_features:
+            raise ops.SnGgufError(f"GGUFLinear: norm weight has {norm_weight.numel()} elements, in_features is {self.in_features}")
         out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
         bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
         tiled = self.tiled_weight() if self.decode_layout != "native" else None
@@ -317,6 +336,14 @@ class GGUFLinear(nn.Linear):
             torch.matmul(x2d, weight.t(), out=out2d)
         else:
             torch.addmm(self.bias.to(torch.bfloat16), x2d, weight.t(), out=out2d)
+
+    def weights_changed(self) -> None:
+        """Tell the module that the packed bytes were rewritten in place.  The kept copies (``"resident"`` bf16 weight,
+        ``"tiled"`` decode layout) follow ``weight.data_ptr()`` and ``weight._version``: rebinding ``weight.data`` or an
+        in-place op on ``weight`` itself is noticed, a write through ``weight.data`` (``weight.data.copy_(...)``, what an
+        offloader's upload into a reused buffer amounts to) is not - it leaves both untouched - so call this after one."""
+        self._dense_cache = None
+        self._tiled_cache = None
 
     def drop_dense_cache(self) -> None:
         """Release the bf16 weight the "resident" policy keeps."""

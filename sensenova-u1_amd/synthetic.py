@@ -12,13 +12,14 @@ in HBM.
 * Q3_K: mask, quant and scale bytes uniform, ``d = fp16(|N(0, 0.01)|)``.
 * Q6_K: 6-bit quants uniform (ql, qh bytes uniform), int8 sub-scales uniform over the signed
   6-bit range [-32, 31], ``d = fp16(|N(0, 0.01)|)``.
+* BF16 (plain rows): bf16(N(0, 0.02)).
 * activations: bf16 N(0, 1).
 """
 from __future__ import annotations
 
 import torch
 
-from .ops import GGML_QUANT_SIZES, Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0
+from .ops import BF16, GGML_QUANT_SIZES, Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0
 
 
 def _gen(seed: int, device) -> torch.Generator:
@@ -37,6 +38,9 @@ def make_packed(quant_type: int, n: int, k: int, seed: int = 0, device="cpu") ->
     if k % bs:
         raise ValueError(f"k={k} is not a multiple of the block size {bs}")
     g = _gen(seed, device)
+    if quant_type == BF16:
+        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+        return w.to(torch.bfloat16).view(torch.uint8).reshape(n, 2 * k)
     nb = k // bs
     blocks = torch.empty((n, nb, ts), dtype=torch.uint8, device=device)
 

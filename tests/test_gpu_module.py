@@ -129,7 +129,11 @@ def test_resident_policy_keeps_the_bf16_weight_until_the_packed_bytes_change(tmp
     other.gemm_policy = "two_pass"
     assert torch.equal(mod(x), other(x)) and mod._dense_cache[1] is not kept
     mod.weight.data = old
-    mod.weight.data.copy_(other.weight.data)                                # in-place change at the same address
+    y_old = mod(x)                                                          # the cache now holds `old`'s address
+    assert torch.equal(y_old, y0)
+    mod.weight.data.copy_(other.weight.data)                                # in-place change at the same address:
+    assert torch.equal(mod(x), y0)                                          # invisible to the key (documented) ...
+    mod.weights_changed()                                                   # ... until the module is told
     assert torch.equal(mod(x), other(x))
     mod.drop_dense_cache()
     assert mod._dense_cache is None
@@ -347,3 +351,39 @@ def test_set_decode_layout_on_a_loaded_model(tmp_path, dev):
         assert torch.equal(m(big), want_big)
     set_decode_layout(model, "native")
     assert all(m._tiled_cache is None for m in mods)
+
+
+def test_module_paths_refuse_host_tensors_and_wrong_widths(dev):
+    """The module routes that hand raw pointers to the library (split-K workspace route, fused norm, tiled decode,
+    fused gated MLP) raise a clean error for a weight / norm weight / residual left on the host and for an input
+    whose last dim is not in_features, instead of launching a kernel on a host pointer or re-rowing the input."""
+    print("case module host-tensor refusal", flush=True)
+    n, k = 512, 256
+    packed = synthetic.make_packed(8, n, k, seed=3)
+    lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    lin.weight = GGUFParameter(packed, quant_type=8)                        # still on the host
+    gamma_dev = torch.ones(k, dtype=torch.bfloat16, device=dev)
+    for rows in (1, 100, 200):
+        x = synthetic.make_activations(rows, k, seed=rows).to(dev)
+        with pytest.raises(ops.SnGgufError):
+            lin(x)
+    with pytest.raises(ops.SnGgufError):
+        lin.forward_normed(synthetic.make_activations(1, k).to(dev), gamma_dev, 1e-6)
+    lin.weight = GGUFParameter(packed.to(dev), quant_type=8)
+    with pytest.raises(ops.SnGgufError):
+        lin.forward_normed(synthetic.make_activations(1, k).to(dev), gamma_dev.cpu(), 1e-6)   # norm weight on the host
+    with pytest.raises(ops.SnGgufError):
+        lin(synthetic.make_activations(100, 2 * k).to(dev))                 # 100 rows of the wrong width, not 200 rows
+    with pytest.raises(ops.SnGgufError):
+        lin.forward_normed(synthetic.make_activations(1, 2 * k).to(dev), gamma_dev, 1e-6)
+    up = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    up.weight = GGUFParameter(synthetic.make_packed(8, n, k, seed=4), quant_type=8)           # host
+    down = GGUFLinear(n, k, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    down.weight = GGUFParameter(synthetic.make_packed(8, k, n, seed=5).to(dev), quant_type=8)
+    with pytest.raises(ops.SnGgufError):
+        gated_mlp(synthetic.make_activations(1, k).to(dev), lin, up, down, gamma_dev, 1e-6)
+    lin.decode_layout = "tiled"
+    lin.tiled_weight()
+    with pytest.raises(ops.SnGgufError):
+        lin.forward_residual(synthetic.make_activations(2, k).to(dev), synthetic.make_activations(2, n))   # residual on the host
+    torch.cuda.synchronize()

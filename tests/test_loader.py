@@ -237,3 +237,86 @@ def test_set_decode_layout_walks_the_model(tmp_path):
     assert set_decode_layout(model, "native") == n
     with pytest.raises(ValueError):
         set_decode_layout(model, "blocked")
+
+
+def _bf16_rows(t: torch.Tensor) -> np.ndarray:
+    """A float tensor as the uint8 rows a GGUF file stores for type BF16 (two bytes per element)."""
+    b = t.detach().to(torch.bfloat16).contiguous()
+    return b.view(torch.uint8).reshape(*b.shape[:-1], 2 * b.shape[-1]).numpy()
+
+
+def test_bf16_tensors_are_wrapped_and_placed(tmp_path):
+    """BF16 is a GGUF tensor type like the quantized ones (only F32 / F16 are exempt in the reference,
+    gguf_loader.py:37-41): a Linear weight stored as BF16 becomes a GGUFLinear of type BF16, a BF16 side tensor
+    (here a norm weight) is decoded into its plain slot."""
+    torch.manual_seed(0)
+    ref = TinyModel()
+    bf = GGMLQuantizationType.BF16
+    skip = ("lm_head.weight", "layers.0.input_layernorm.weight")
+    extra = [("lm_head.weight", _bf16_rows(ref.lm_head.weight), int(bf)),
+             ("layers.0.input_layernorm.weight", _bf16_rows(ref.layers[0].input_layernorm.weight), int(bf))]
+    path = str(tmp_path / "b.gguf")
+    _make_file(path, skip=skip, extra=extra)
+    sd = load_gguf_checkpoint(path)
+    w = sd["lm_head.weight"]
+    assert isinstance(w, GGUFParameter) and w.quant_type == bf and tuple(w.shape) == (32, 2 * H) and tuple(w.quant_shape) == (32, H)
+    g = sd["layers.0.input_layernorm.weight"]
+    assert isinstance(g, GGUFParameter) and tuple(g.quant_shape) == (H,)
+    with torch.device("meta"):
+        model = TinyModel()
+    model = set_gguf2meta_model(model, sd, torch.bfloat16, torch.device("cpu"))
+    assert type(model.lm_head).__name__ == "GGUFLinear" and model.lm_head.weight.quant_type == bf
+    assert torch.equal(model.lm_head.weight.as_tensor().view(torch.bfloat16), ref.lm_head.weight.detach().to(torch.bfloat16))
+    norm = model.layers[0].input_layernorm.weight
+    assert type(norm) is nn.Parameter and norm.dtype == torch.bfloat16
+    assert torch.equal(norm.detach(), ref.layers[0].input_layernorm.weight.detach().to(torch.bfloat16))
+    # the oracle decodes type 30 exactly, in both modes and both restatements
+    want = ref.lm_head.weight.detach().to(torch.bfloat16).float()
+    for numerics in (0, 1):
+        assert torch.equal(go.dequantize_gguf_tensor(w.as_tensor(), go.BF16, numerics), want)
+        assert torch.equal(go.COracle().dequantize(w.as_tensor(), go.BF16, torch.float32, numerics), want)
+
+
+def test_load_gguf_model_one_call(tmp_path, capsys):
+    """The sequence of checkpoint_loading.py:288-323 in one call: meta model (or config + factory) -> parsed file ->
+    swapped and placed -> count reported -> eval mode; and the warning when nothing was quantized."""
+    from sensenova_u1_amd import load_gguf_model
+    path = str(tmp_path / "m.gguf")
+    ref, packed = _make_file(path)
+    with torch.device("meta"):
+        meta = TinyModel()
+    model = load_gguf_model(meta, path, dtype=torch.bfloat16, device="cpu")
+    out = capsys.readouterr().out
+    assert f"[gguf] loading quantized checkpoint from {path}" in out and "[gguf] parsed" in out
+    assert f"[gguf] {2 * (2 + 6) + 1} GGUFLinear modules active" in out and "WARNING" not in out
+    assert model is meta and not model.training
+    assert not any(p.device.type == "meta" for p in model.parameters())
+    # a config and a factory
+    model2 = load_gguf_model({"unused": 1}, path, dtype=torch.bfloat16, device=torch.device("cpu"), model_factory=lambda cfg: TinyModel())
+    assert count_gguf_linear(model2) == count_gguf_linear(model)
+    assert np.array_equal(model2.layers[1].mlp.up_proj.weight.as_tensor().numpy(), packed["layers.1.mlp.up_proj.weight"])
+    # a model that already holds storage is refused
+    with pytest.raises(ValueError, match="meta-initialized"):
+        load_gguf_model(TinyModel(), path, dtype=torch.bfloat16, device="cpu")
+    # a file without quantized tensors: loads, and says so
+    plain_path = str(tmp_path / "p.gguf")
+    torch.manual_seed(0)
+    plain = TinyModel()
+    write_gguf(plain_path, [(n, t.detach().numpy().astype(np.float32), 0) for n, t in plain.state_dict().items()])
+    capsys.readouterr()
+    model3 = load_gguf_model(None, plain_path, dtype=torch.float32, device="cpu", model_factory=lambda cfg: TinyModel())
+    out = capsys.readouterr().out
+    assert "[gguf] 0 GGUFLinear modules active" in out and "WARNING: no GGUFLinear modules found" in out
+    assert torch.equal(model3.lm_head.weight, plain.lm_head.weight)
+
+
+@pytest.mark.parametrize("rows", [1, 100, 300])
+def test_module_with_host_weight_raises_before_any_launch(rows):
+    """Every row count - decode, the split-K workspace route, the weight-pass route - refuses host tensors with the
+    library's own error type; nothing reaches a kernel with a host pointer."""
+    lin = GGUFLinear(256, 512, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    lin.weight = GGUFParameter(synthetic.make_packed(8, 512, 256), quant_type=8)
+    with pytest.raises(ops.SnGgufError):
+        lin(torch.zeros(rows, 256, dtype=torch.bfloat16))
+    with pytest.raises(ops.SnGgufError):
+        lin._checked_rows(torch.zeros(rows, 256, dtype=torch.bfloat16), torch.ones(256, dtype=torch.bfloat16))
