@@ -2,7 +2,7 @@
 GGUF loader over hand-written HIP kernels (libsngguf.so, C ABI in include/sngguf.h)."""
 from .gguf_file import GGML_QUANT_SIZES, GGMLQuantizationType, GGUFReader, GGUFWriter, NativeGGUFReader
 from .gguf_loader import count_gguf_linear, load_gguf_checkpoint, load_gguf_model, match_state_dict, set_gguf2meta_model
-from .layer_offload import AsyncPrefetcher, LayerOffloadWrapper, PackedLayerStore
+from .layer_offload import LayerOffloadWrapper, LayerStreamer, PackedLayerStore
 from .modality import FusedProjections, find_mot_pairs, gated_mlp, grouped_linear
 from .quantized_linear import (
     SUPPORTED_GGUF_QUANT_TYPES,
@@ -17,5 +17,5 @@ __all__ = [
     "load_gguf_checkpoint", "load_gguf_model", "set_gguf2meta_model", "match_state_dict", "count_gguf_linear",
     "GGUFLinear", "GGUFParameter", "SUPPORTED_GGUF_QUANT_TYPES", "dequantize_gguf_tensor",
     "grouped_linear", "find_mot_pairs", "gated_mlp", "FusedProjections", "NativeGGUFReader",
-    "LayerOffloadWrapper", "PackedLayerStore", "AsyncPrefetcher", "set_decode_layout",
+    "LayerOffloadWrapper", "PackedLayerStore", "LayerStreamer", "set_decode_layout",
 ]

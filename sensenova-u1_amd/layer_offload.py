@@ -4,8 +4,8 @@ Keeps the tensors of every layer of an ``nn.ModuleList`` in pinned host memory a
 the GPU for the layer's forward, optionally ahead of time on a second stream.  Interface and
 semantics follow the reference's layer offloader
 (``src/sensenova_u1/utils/layer_offload.py``: tensor groups ``:51-54``, tower partition ``:195-222``,
-group selection from the layer kwargs ``:225-241``, store ``:289-419``, prefetcher ``:422-462``,
-hooks ``:764-843``, wrapper ``:465-999``), the data movement does not:
+group selection from the layer kwargs ``:225-241``, store ``:289-419``; what the prefetcher ``:422-462`` and the
+hooks ``:764-843`` of the wrapper ``:465-999`` achieve is reached differently), the data movement does not:
 
 * every (layer, group) is packed once into ONE contiguous pinned arena, so bringing a tower of a
   layer onto the GPU is a single asynchronous copy of ~100-200 MB instead of one copy per tensor,
@@ -14,7 +14,11 @@ hooks ``:764-843``, wrapper ``:465-999``), the data movement does not:
   prefetch depth), allocated on first use and then reused for the rest of the process, so a
   forward pass allocates nothing and no caching-allocator stream bookkeeping (``record_stream``)
   is involved.  A slot carries the event recorded on the compute stream when its layer was evicted;
-  the stream that next copies into the slot waits for that event first.
+  the stream that next copies into the slot waits for that event first;
+* copying ahead is part of the store (``copy_ahead`` / ``make_ready``): a copy on the store's second stream leaves
+  a "landed" event with the slot, the consumer's stream waits for it, and a slot handed back before anyone consumed
+  its copy takes that event along to its next user.  A change of tower therefore needs no device-wide
+  synchronisation: the slots of the tower that is no longer read simply go back to the ring.
 
 The VRAM-budget residency policy, the prefix/denoise phase callback and the diagnostics of the
 reference wrapper (``:68-116,684-762,863-919``) are control plane and are not rebuilt; the only
@@ -22,7 +26,6 @@ residency option kept is ``keep_generation_resident`` with an explicit byte budg
 """
 from __future__ import annotations
 
-import functools
 import itertools
 from typing import Any, Optional
 
@@ -109,7 +112,11 @@ class PackedLayerStore:
         self._tensor_groups: list[dict[str, str]] = []
         self._resident: list[dict[str, torch.Tensor]] = []
         self._managed: set[int] = set()
-        self._free: dict[str, list[tuple[torch.Tensor, Any]]] = {g: [] for g in ALL_TENSOR_GROUPS}
+        # free slots, each with the events its next user must wait for: the compute-stream event of the eviction and,
+        # if a copy into it was still unconsumed at that point, that copy's event
+        self._free: dict[str, list[tuple[torch.Tensor, list]]] = {g: [] for g in ALL_TENSOR_GROUPS}
+        self._ready: list[dict[str, Any]] = []      # per layer: group -> event of a copy-ahead nobody has waited for yet
+        self._copy_stream = None
         self._slot_bytes = {g: 0 for g in ALL_TENSOR_GROUPS}
         self._slots_allocated = {g: 0 for g in ALL_TENSOR_GROUPS}
         self._bytes_moved = 0
@@ -135,6 +142,7 @@ class PackedLayerStore:
             self._arenas.append(arenas)
             self._tensor_groups.append(groups)
             self._resident.append({})
+            self._ready.append({})
 
     def _check_idx(self, idx: int) -> None:
         if idx < 0 or idx >= self.num_layers:
@@ -149,8 +157,8 @@ class PackedLayerStore:
 
     def _take_slot(self, group: str) -> torch.Tensor:
         if self._free[group]:
-            slot, event = self._free[group].pop()
-            if event is not None:
+            slot, events = self._free[group].pop()
+            for event in events:
                 torch.cuda.current_stream(self.target_device).wait_event(event)
             return slot
         self._slots_allocated[group] += 1
@@ -184,11 +192,54 @@ class PackedLayerStore:
             if slot is None:
                 continue
             self._arenas[idx][g].bind(self._arenas[idx][g].host)
-            event = None
+            events = []
             if self.target_device.type == "cuda":
-                event = torch.cuda.Event()
-                event.record(torch.cuda.current_stream(self.target_device))
-            self._free[g].append((slot, event))
+                done = torch.cuda.Event()
+                done.record(torch.cuda.current_stream(self.target_device))
+                events.append(done)
+            unconsumed = self._ready[idx].pop(g, None)
+            if unconsumed is not None:
+                events.append(unconsumed)
+            self._free[g].append((slot, events))
+
+    # ---- copy-ahead on a second stream: the slot ring's events are the whole protocol -------------------------------
+    # A slot goes round as: free (carrying the events of its last use) -> copy target (the copying stream waits for
+    # those events) -> resident, perhaps with a "ready" event from the copy stream -> in use (the consumer waited for
+    # the ready event) -> free again.  No stream is ever synchronised with the host.
+
+    def copy_ahead(self, idx: int, groups: frozenset) -> None:
+        """Start bringing the missing groups of layer ``idx`` in on the store's copy stream (created on first use,
+        default priority).  Returns at once; ``make_ready`` later orders a consumer stream behind the copy."""
+        self._check_idx(idx)
+        missing = frozenset(g for g in groups if g in self._arenas[idx] and g not in self._resident[idx])
+        if not missing:
+            return
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=self.target_device)
+        with torch.cuda.stream(self._copy_stream):
+            self.move_to_gpu(idx, groups=missing, non_blocking=True)
+            landed = torch.cuda.Event()
+            landed.record(self._copy_stream)
+        for g in missing:
+            self._ready[idx][g] = landed
+
+    def make_ready(self, idx: int, groups: frozenset) -> None:
+        """After this call, work enqueued on the current stream may read ``groups`` of layer ``idx``: copies started by
+        ``copy_ahead`` are waited for (on the stream, not on the host), anything still missing is copied on the
+        current stream itself."""
+        self._check_idx(idx)
+        stream = torch.cuda.current_stream(self.target_device) if self.target_device.type == "cuda" else None
+        waited: set[int] = set()
+        for g in groups:
+            landed = self._ready[idx].pop(g, None)
+            if landed is not None and id(landed) not in waited:
+                stream.wait_event(landed)
+                waited.add(id(landed))
+        self.move_to_gpu(idx, groups=groups, non_blocking=True)
+
+    def copies_in_flight(self) -> set[int]:
+        """Layers with a copy-ahead that no consumer has been ordered behind yet."""
+        return {i for i, r in enumerate(self._ready) if r}
 
     def tensors_for_groups(self, idx: int, layer: nn.Module, groups: frozenset) -> list[torch.Tensor]:
         self._check_idx(idx)
@@ -228,67 +279,104 @@ class PackedLayerStore:
         for g in self._free:
             self._free[g].clear()
             self._slots_allocated[g] = 0
+        self._copy_stream = None
 
 
-class AsyncPrefetcher:
-    """Copies upcoming layers on a second stream (default priority); one event per layer so the compute
-    stream waits only for the layer it is about to run (reference ``layer_offload.py:422-462``)."""
-
-    def __init__(self, store: PackedLayerStore, layers) -> None:
-        self._store = store
-        self._layers = layers
-        self._stream = torch.cuda.Stream(device=store.target_device)
-        self._events: dict[int, tuple[Any, frozenset]] = {}
-
-    @property
-    def stream(self):
-        return self._stream
-
-    def prefetch(self, idx: int, groups: frozenset) -> None:
-        if self._store.is_on_gpu(idx, groups) or idx in self._events:
-            return
-        with torch.cuda.stream(self._stream):
-            self._store.move_to_gpu(idx, self._layers[idx], groups=groups, non_blocking=True)
-            event = torch.cuda.Event()
-            event.record(self._stream)
-        self._events[idx] = (event, groups)
-
-    def wait(self, idx: int) -> None:
-        pending = self._events.pop(idx, None)
-        if pending is not None:
-            torch.cuda.current_stream(self._store.target_device).wait_event(pending[0])
-
-    def pending(self) -> set[int]:
-        return set(self._events)
-
-    def clear_events(self) -> None:
-        self._events.clear()
-
-    def cleanup(self) -> None:
-        self._events.clear()
-        self._stream = None
-        self._layers = None
-        self._store = None
+def _layer_list(model: nn.Module, dotted: str) -> nn.ModuleList:
+    found = model.get_submodule(dotted) if dotted else model
+    if not isinstance(found, nn.ModuleList):
+        raise TypeError(f"'{dotted}' is a {type(found).__name__}; layer streaming needs an nn.ModuleList")
+    return found
 
 
-def _resolve_attr(module: nn.Module, dotted_path: str) -> nn.ModuleList:
-    obj: Any = module
-    for part in dotted_path.split("."):
-        obj = getattr(obj, part)
-    if not isinstance(obj, nn.ModuleList):
-        raise TypeError(f"Expected nn.ModuleList at '{dotted_path}', got {type(obj).__name__}")
-    return obj
+class LayerStreamer:
+    """Installs layer streaming on a model in place: every layer of the list gets a gate in front of its forward
+    (bring my groups in, start the copies for the layers after me) and one behind it (hand my slots back).
+
+    The model stays the callable; this object only owns the store, the schedule and the hook handles.
+    """
+
+    def __init__(self, model: nn.Module, layers: nn.ModuleList, target_device: torch.device, depth: int,
+                 keep_generation_resident: bool, resident_budget_bytes: Optional[int]) -> None:
+        self.model = model
+        self.layers = layers
+        self.device = target_device
+        self.depth = min(depth, max(len(layers) - 1, 0))
+        self.keep_generation = keep_generation_resident
+        self.budget = resident_budget_bytes
+        self.store = PackedLayerStore(layers, target_device)
+        managed = self.store.managed_tensor_ids()
+        self._outside = [t for t in itertools.chain(model.parameters(), model.buffers()) if id(t) not in managed]
+        for t in self._outside:
+            t.data = t.data.to(target_device)
+        self._tower: Optional[frozenset] = None       # groups of the call in progress / the last call
+        self._in_forward: dict[int, frozenset] = {}
+        self._handles = []
+        for idx, layer in enumerate(layers):
+            self._handles.append(layer.register_forward_pre_hook(self._gate_in(idx), with_kwargs=True))
+            self._handles.append(layer.register_forward_hook(self._gate_out(idx)))
+
+    # -- schedule ---------------------------------------------------------------------------------------------------
+    def _upcoming(self, idx: int):
+        """The layers whose copies should be under way while layer ``idx`` runs: the next ``depth`` ones, wrapping
+        round to the first layers, which the next pass over the list starts with."""
+        n = len(self.layers)
+        return [(idx + step) % n for step in range(1, self.depth + 1)]
+
+    def _retarget(self, groups: frozenset) -> None:
+        """The call reads other groups than the last one did: slots holding a group it does not read go back to the
+        ring (their events keep work in flight safe), except a generation tower that is being kept."""
+        stale = ALL_TENSOR_GROUPS - groups
+        if self.keep_generation and self._within_budget():
+            stale = stale - {GROUP_GENERATION}
+        if stale and self._tower is not None:
+            for idx in range(len(self.layers)):
+                self.store.evict_to_cpu(idx, groups=stale)
+        self._tower = groups
+
+    def _within_budget(self) -> bool:
+        return self.budget is None or self.store.device_bytes() <= self.budget
+
+    def _gate_in(self, idx: int):
+        def gate(layer, args, kwargs):
+            groups = required_tensor_groups(kwargs)
+            if groups != self._tower:
+                self._retarget(groups)
+            self.store.make_ready(idx, groups)
+            for nxt in self._upcoming(idx):
+                self.store.copy_ahead(nxt, groups)
+            self._in_forward[idx] = groups
+        return gate
+
+    def _gate_out(self, idx: int):
+        def gate(layer, args, output):
+            groups = self._in_forward.pop(idx, ALL_TENSOR_GROUPS)
+            if self.keep_generation and GROUP_GENERATION in groups and self._within_budget():
+                groups = groups - {GROUP_GENERATION}
+            self.store.evict_to_cpu(idx, groups=groups)
+        return gate
+
+    def remove(self) -> None:
+        """Take the gates off, wait for the device, put every tensor back on the host (layer tensors in their pinned
+        arenas) and drop the slot ring."""
+        for h in self._handles:
+            h.remove()
+        self._handles = []
+        self.store.cleanup()
+        for t in self._outside:
+            t.data = t.data.to("cpu")
 
 
 class LayerOffloadWrapper(nn.Module):
-    """Runs ``model`` with the layers of ``layers_attr`` streamed from pinned host memory.
+    """``model`` with the layers of ``layers_attr`` streamed from pinned host memory; same constructor arguments and
+    use as the reference's wrapper (``layer_offload.py:501-530``): call it like the model, read the model's attributes
+    through it, ``teardown()`` when done.
 
-    ``prefetch_count == 0``: a layer's groups are copied on the compute stream right before its forward;
-    ``>= 1``: that many layers ahead are copied on a second stream, wrapping around to the first layers
-    for the next pass.  Only the groups a call needs are brought in, chosen from the layer kwargs
-    ``exist_non_image_gen_tokens`` / ``exist_image_gen_tokens``.  Everything outside ``layers_attr`` is
-    moved to ``target_device`` once and stays there.  Inference only.
-    Constructor and behaviour after reference ``layer_offload.py:501-530,607-642,764-843,921-999``.
+    ``prefetch_count == 0``: a layer's groups are copied on the compute stream right before its forward; ``>= 1``:
+    that many layers ahead are copied on a second stream, wrapping around to the first layers for the next pass.
+    Only the groups a call needs are brought in, chosen from the layer kwargs ``exist_non_image_gen_tokens`` /
+    ``exist_image_gen_tokens``.  Everything outside ``layers_attr`` is moved to ``target_device`` once and stays
+    there.  Inference only.  The work is done by :class:`LayerStreamer` (``.streamer``).
     """
 
     def __init__(self, model: nn.Module, layers_attr: str, target_device: torch.device, prefetch_count: int = 0,
@@ -303,95 +391,30 @@ class LayerOffloadWrapper(nn.Module):
             raise ValueError("resident_budget_bytes must be > 0 when set")
         if model.training:
             raise RuntimeError("LayerOffloadWrapper only supports inference; call model.eval() first.")
-        self._model = model
-        self._layers = _resolve_attr(model, layers_attr)
-        self._target_device = target_device
-        self._prefetch_count = min(prefetch_count, max(len(self._layers) - 1, 0))
-        self._async_mode = self._prefetch_count >= 1
-        self._keep_generation_resident = keep_generation_resident
-        self._resident_budget_bytes = resident_budget_bytes
-        self._active_groups: Optional[frozenset] = None
-        self._hooks: list = []
-        self._store = PackedLayerStore(self._layers, target_device)
-        managed = self._store.managed_tensor_ids()
-        for t in itertools.chain(model.parameters(), model.buffers()):
-            if id(t) not in managed:
-                t.data = t.data.to(target_device)
-        self._prefetcher = AsyncPrefetcher(self._store, self._layers) if self._async_mode else None
-        self._register_hooks()
+        layers = _layer_list(model, layers_attr)
+        self.wrapped = model
+        # (a plain attribute, not a submodule: the streamer refers back to the model)
+        object.__setattr__(self, "streamer", LayerStreamer(model, layers, target_device, prefetch_count,
+                                                           keep_generation_resident, resident_budget_bytes))
 
     @property
     def store(self) -> PackedLayerStore:
-        return self._store
-
-    def _switch_groups(self, groups: frozenset) -> None:
-        """A change of tower drains the copy stream and evicts what the other tower left behind."""
-        if self._active_groups == groups:
-            return
-        if self._active_groups is not None:
-            torch.cuda.synchronize(self._target_device)
-            if self._prefetcher is not None:
-                self._prefetcher.clear_events()
-            for idx, layer in enumerate(self._layers):
-                self._store.evict_to_cpu(idx, layer)
-        self._active_groups = groups
-
-    def _groups_to_evict(self, idx: int, groups: frozenset) -> frozenset:
-        if not self._keep_generation_resident or GROUP_GENERATION not in groups:
-            return groups
-        if self._resident_budget_bytes is not None and self._store.device_bytes() > self._resident_budget_bytes:
-            return groups
-        return groups - {GROUP_GENERATION}
-
-    def _register_hooks(self) -> None:
-        num_layers = len(self._layers)
-        active: dict[int, frozenset] = {}
-
-        def pre_hook(module, args, kwargs, *, idx: int) -> None:
-            groups = required_tensor_groups(kwargs)
-            active[idx] = groups
-            self._switch_groups(groups)
-            if self._async_mode:
-                self._prefetcher.wait(idx)
-                if not self._store.is_on_gpu(idx, groups):
-                    self._store.move_to_gpu(idx, module, groups=groups, non_blocking=True)
-                for ahead in range(1, self._prefetch_count + 1):
-                    self._prefetcher.prefetch((idx + ahead) % num_layers, groups)
-            else:
-                self._store.move_to_gpu(idx, module, groups=groups, non_blocking=True)
-
-        def post_hook(module, _args, _output, *, idx: int) -> None:
-            groups = active.pop(idx, ALL_TENSOR_GROUPS)
-            self._store.evict_to_cpu(idx, module, groups=self._groups_to_evict(idx, groups))
-
-        for idx, layer in enumerate(self._layers):
-            self._hooks.append(layer.register_forward_pre_hook(functools.partial(pre_hook, idx=idx), with_kwargs=True))
-            self._hooks.append(layer.register_forward_hook(functools.partial(post_hook, idx=idx)))
+        return self.streamer.store
 
     def transfer_stats(self) -> tuple[int, dict[str, int]]:
-        return self._store.transfer_stats()
+        return self.streamer.store.transfer_stats()
 
     def teardown(self) -> None:
-        """Remove the hooks, drain the copies, leave every tensor on the host (layer tensors in their
-        pinned arenas) and release the device ring."""
-        for h in self._hooks:
-            h.remove()
-        self._hooks.clear()
-        torch.cuda.synchronize(self._target_device)
-        if self._prefetcher is not None:
-            self._prefetcher.cleanup()
-            self._prefetcher = None
-        self._store.cleanup()
-        managed = self._store.managed_tensor_ids()
-        for t in itertools.chain(self._model.parameters(), self._model.buffers()):
-            if id(t) not in managed:
-                t.data = t.data.to("cpu")
+        self.streamer.remove()
 
     def forward(self, *args: Any, **kwargs: Any) -> Any:
-        return self._model(*args, **kwargs)
+        return self.wrapped(*args, **kwargs)
 
     def __getattr__(self, name: str) -> Any:
-        try:
-            return super().__getattr__(name)
-        except AttributeError:
-            return getattr(self._model, name)
+        # nn.Module keeps submodules out of __dict__; anything this wrapper does not have is the model's
+        modules = self.__dict__.get("_modules", {})
+        if name in modules:
+            return modules[name]
+        if "wrapped" in modules:
+            return getattr(modules["wrapped"], name)
+        raise AttributeError(name)

@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import gguf_oracle as go
+from sensenova_u1_amd import ops
 from sensenova_u1_amd import (FusedProjections, GGUFLinear, GGUFParameter, gated_mlp, grouped_linear, load_gguf_checkpoint,
                               set_gguf2meta_model, synthetic)
 from tests.test_loader import H, I, TinyModel, _make_file
