@@ -74,7 +74,8 @@ enum {
     SNGGUF_E_LAUNCH = -5,    /* the HIP runtime refused the launch (hipGetLastError != 0)     */
     SNGGUF_E_NODEVICE = -6,  /* no usable gfx950 device / code object                         */
     SNGGUF_E_IO = -7,        /* a file could not be opened or mapped                          */
-    SNGGUF_E_FORMAT = -8     /* not a GGUF file, truncated, corrupt, or a tensor type of unknown size */
+    SNGGUF_E_FORMAT = -8,    /* not a GGUF file, truncated, corrupt, or a tensor type of unknown size */
+    SNGGUF_E_TOOLARGE = -9   /* sngguf_linear_static: M * N beyond sngguf_linear_static_max_outputs()         */
 };
 
 /* Library version (major*10000 + minor*100 + patch) and error text. */
@@ -148,6 +149,24 @@ int64_t sngguf_linear_workspace_bytes(int64_t N, int64_t K);
 int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
                      const void* bias, void* y, void* workspace, int64_t workspace_bytes, int numerics,
                      void* stream);
+
+/*
+ * sngguf_linear_ws without a workspace argument and without any allocation.  No counterpart in the reference:
+ * it exists for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc - and therefore cannot hand sngguf_linear_ws a workspace, yet want its K split
+ * for problems with few output tiles.  The workspace is a 64 MiB array inside the library's own device image
+ * (one copy per GPU, held until the process ends); the result is bit-identical to sngguf_linear_ws called with a
+ * 64 MiB workspace.
+ *
+ * Limit: M * N <= sngguf_linear_static_max_outputs() (= 8 Mi outputs: two fp32 slices of the output fit), else
+ * SNGGUF_E_TOOLARGE; such problems have enough tiles for sngguf_linear.
+ * The first call on a device looks up the array's address on that device (hipGetSymbolAddress) and caches it;
+ * make that call before a capture begins.  No call allocates or frees.  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race; calls on one stream are ordered.
+ */
+int64_t sngguf_linear_static_max_outputs(void);
+int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
+                         const void* bias, void* y, int numerics, void* stream);
 
 /*
  * SiLU-gated pair for the decode MLP: h[M][N] = silu(x.Wg^T) * (x.Wu^T), with both

@@ -20,6 +20,8 @@ int launch_dequantize_bf16(const void* q, int64_t rows, int64_t cols, void* out,
 int launch_gemv_bf16(const void* x, int64_t M, const void* wa, const void* wb, int64_t N, int64_t K, const void* bias,
                      const void* residual, void* y, bool gated, hipStream_t stream);
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
+int64_t static_scratch_bytes();
+int static_scratch(void** ptr);
 int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream_t stream);
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
                          const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
@@ -74,6 +76,7 @@ const char* sngguf_strerror(int code) {
     case SNGGUF_E_NODEVICE: return "no usable gfx950 device";
     case SNGGUF_E_IO: return "file could not be opened or mapped";
     case SNGGUF_E_FORMAT: return "not a GGUF file, or truncated / corrupt";
+    case SNGGUF_E_TOOLARGE: return "problem exceeds the static scratch area of the allocation-free entry point (use sngguf_linear_ws with a caller workspace)";
     default: return "unknown error";
     }
 }
@@ -212,8 +215,9 @@ bool grouped_dense_route_fits(int64_t M, int64_t N, int64_t K) {
 
 int64_t sngguf_linear_workspace_bytes(int64_t N, int64_t K) { return N > 0 && K > 0 && N < kMaxDim && K < kMaxDim ? 2 * N * K : 0; }
 
-int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
-                     void* workspace, int64_t workspace_bytes, int numerics, void* stream) {
+namespace {
+int linear_ws_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                   void* workspace, int64_t workspace_bytes, int numerics, void* stream) {
     const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
@@ -251,6 +255,26 @@ int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t
     const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
     if (rd != SNGGUF_OK) return rd;
     return sngguf::launch_gemm_dense(x, M, workspace, N, K, bias, y, s);
+}
+}  // namespace
+
+int sngguf_linear_ws(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                     void* workspace, int64_t workspace_bytes, int numerics, void* stream) {
+    return linear_ws_impl(x, M, q, qtype, N, K, bias, y, workspace, workspace_bytes, numerics, stream);
+}
+
+int64_t sngguf_linear_static_max_outputs(void) { return sngguf::static_scratch_bytes() / 8; }
+
+int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias, void* y,
+                         int numerics, void* stream) {
+    const int rc = check_matmul(x, M, q, qtype, N, K, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
+    // two fp32 slices of the output must fit the static area: the smallest K split there is
+    if (M * N > sngguf_linear_static_max_outputs()) return SNGGUF_E_TOOLARGE;
+    void* scratch = nullptr;
+    const int rs = sngguf::static_scratch(&scratch);
+    if (rs != SNGGUF_OK) return rs;
+    return linear_ws_impl(x, M, q, qtype, N, K, bias, y, scratch, sngguf::static_scratch_bytes(), numerics, stream);
 }
 
 int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype, int64_t N, int64_t K,

@@ -33,7 +33,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
-    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_linear_static_max_outputs", "sngguf_linear_static", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_rmsnorm_fits", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
@@ -78,6 +78,10 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_workspace_bytes.restype = i64
     lib.sngguf_linear_ws.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, i64, ci, vp]
     lib.sngguf_linear_ws.restype = ci
+    lib.sngguf_linear_static_max_outputs.argtypes = []
+    lib.sngguf_linear_static_max_outputs.restype = i64
+    lib.sngguf_linear_static.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, ci, vp]
+    lib.sngguf_linear_static.restype = ci
     lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu.restype = ci
     lib.sngguf_grouped_workspace_bytes.argtypes = [i64]
@@ -221,6 +225,23 @@ def linear_ws_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bia
         rc = load_library().sngguf_linear_ws(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
                                              _ptr(y2d), _ptr(workspace), ws_bytes, numerics, ctypes.c_void_p(_stream(dev)))
     _check(rc, "sngguf_linear_ws")
+
+
+def linear_static_max_outputs() -> int:
+    """Largest ``M * N`` that ``linear_static_into`` takes."""
+    return int(load_library().sngguf_linear_static_max_outputs())
+
+
+def linear_static_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],
+                       y2d: torch.Tensor, numerics: int) -> None:
+    """As ``linear_ws_into`` with the library's own static device area (64 MiB per GPU) as the workspace: the call
+    allocates nothing.  ``M * N`` beyond ``linear_static_max_outputs()`` is refused."""
+    dev = x2d.device
+    n, k = y2d.shape[1], x2d.shape[1]
+    with torch.cuda.device(dev):
+        rc = load_library().sngguf_linear_static(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
+                                                 _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+    _check(rc, "sngguf_linear_static")
 
 
 def linear_residual_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor],
