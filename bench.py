@@ -219,6 +219,51 @@ def main() -> None:
                            "down_us": round(dn * 1e3, 3)}
     result["decode_other_M"] = decode
 
+    # ---- configs[0]: a single Q8_0 linear 4096 -> 4096 at M = 1, over 32 distinct weights (570 MB, beyond the last-level cache)
+    if not args.no_extra:
+        singles = [synthetic.make_packed(Q8_0, HIDDEN, HIDDEN, seed=400 + i, device=dev) for i in range(32)]
+        xs1 = synthetic.make_activations(1, HIDDEN, seed=8, device=dev)
+        ys1 = torch.empty((1, HIDDEN), dtype=torch.bfloat16, device=dev)
+        wall_s, ev_s = run_region(lambda i: ops.linear_into(xs1, singles[i % 32], Q8_0, None, ys1, num), K, W)
+        sb = linear_bytes(1, HIDDEN, HIDDEN)
+        result["single_linear"] = {
+            "workload": "configs[0]: one Q8_0 linear 4096 -> 4096 at M=1 (sngguf_linear), 32 distinct weights in rotation",
+            "bytes_per_launch": sb, "avg_launch_us": round(ev_s / K * 1e3, 3),
+            "value": round(sb / (wall_s / K * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "pct_of_hbm_peak": round(100 * sb / (wall_s / K * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        del singles
+
+    # ---- the drop-in route of an unmodified Qwen3MLP.forward (modeling_qwen3.py:214-216): three GGUFLinear modules and
+    # torch's SiLU and product, i.e. down_proj(act_fn(gate_proj(x)) * up_proj(x)) through Module.forward ---------------
+    if not args.no_extra:
+        from sensenova_u1_amd import GGUFLinear, GGUFParameter
+
+        def as_module(packed, n, k):
+            lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+            lin.weight = GGUFParameter(packed, quant_type=Q8_0)
+            lin.numerics = num
+            return lin
+
+        mods = [(as_module(g, INTER, HIDDEN), as_module(u, INTER, HIDDEN), as_module(d, HIDDEN, INTER)) for g, u, d in layers]
+        drop = {}
+        for m in (1, 4, 16):
+            xm = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
+
+            def unfused_step(i):
+                gate_proj, up_proj, down_proj = mods[i % L]
+                return down_proj(torch.nn.functional.silu(gate_proj(xm)) * up_proj(xm))
+
+            kd = K if m == 1 else max(64, K // 4)
+            wall_d, _ = run_region(unfused_step, kd, min(W, 16))
+            gb = mlp_bytes(m) / (wall_d / kd * 1e-3) / 1e9
+            drop[f"M{m}"] = {"value": round(gb, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gb / HBM_PEAK_GBPS, 2),
+                             "ms_per_step": round(wall_d / kd, 6)}
+        drop["workload"] = ("the headline MLP as an unmodified Qwen3MLP.forward runs it after the module swap: three "
+                            "GGUFLinear.forward calls (gate, up, down: three decode launches), torch SiLU and product "
+                            "(two elementwise launches); same algorithmic bytes as the headline step")
+        result["mlp_unfused_dropin"] = drop
+        del mods
+
     # ---- the same MLP on the opt-in operand-order ("tiled") copy of the weights (made once at load time) ------------
     if not args.no_extra:
         tiled = [tuple(ops.q8_0_tile(t) for t in layer) for layer in layers]
@@ -364,7 +409,28 @@ def main() -> None:
         gh = (torch.rand(HIDDEN, generator=torch.Generator().manual_seed(15)) + 0.5).to(torch.bfloat16).to(dev)
         # the model's final RMSNorm (modeling_qwen3.py:1183; lm_head at :1264 reads its output) folded into the same launch
         _, ev_hn = run_region(lambda i: ops.rmsnorm_linear_into(xh, gh, 1e-6, heads[i % 2], Q8_0, None, logits, num), n_h, 32)
+        # greedy token: the arg-max folded into the projection (sngguf_lm_head_argmax) against logits + torch.argmax
+        lib = ops.load_library()
+        import ctypes
+        am_ws = torch.empty(int(lib.sngguf_lm_head_argmax_workspace_bytes(1, vocab)), dtype=torch.uint8, device=dev)
+        am_out = torch.empty(1, dtype=torch.int64, device=dev)
+        strm = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+        def head_argmax(i):
+            rc = lib.sngguf_lm_head_argmax(ctypes.c_void_p(xh.data_ptr()), 1, ctypes.c_void_p(heads[i % 2].data_ptr()), Q8_0, vocab, HIDDEN,
+                                           None, ctypes.c_void_p(am_ws.data_ptr()), ctypes.c_void_p(am_out.data_ptr()), num,
+                                           ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+            assert rc == 0, rc
+
+        def head_then_argmax(i):
+            ops.linear_into(xh, heads[i % 2], Q8_0, None, logits, num)
+            torch.argmax(logits, dim=-1, out=am_out)
+
+        _, ev_am = run_region(head_argmax, n_h, 32)
+        _, ev_la = run_region(head_then_argmax, n_h, 32)
+        del strm
         result["lm_head"] = {"workload": "Q8_0 lm_head 4096 -> 151936 at M=1, two weight copies alternating",
+                             "argmax_fused_us": round(ev_am / n_h * 1e3, 2), "logits_then_torch_argmax_us": round(ev_la / n_h * 1e3, 2),
                              "bytes_per_launch": hb, "avg_launch_us": round(ev_h / n_h * 1e3, 2),
                              "with_final_norm_fused_us": round(ev_hn / n_h * 1e3, 2),
                              "tiled_layout_us": round(ev_ht / n_h * 1e3, 2),
@@ -481,7 +547,7 @@ def main() -> None:
             "flop_per_step": flops,
             "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
             "roofline": {
-                "kernel": "sngguf::gemm_q8_kernel<upstream_fp16> (gate 4096->12288, M=4096)",
+                "kernel": "sngguf::gemm_tile_kernel<Q8_0, upstream_fp16> (gate 4096->12288, M=4096)",
                 "bound": "mfma",
                 "achieved": round(gate_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS,
@@ -681,7 +747,41 @@ def main() -> None:
                 "pct_of_bf16_mfma_peak": round(100 * flops / (wall2 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
             },
         }
-        del und, gen, xs, ys, wtmp
+        del und, gen, wtmp
+
+        # configs[4] as stated: all 36 layers x 2 towers resident (14.76 GB of Q8_0), the 7 grouped linears of every layer
+        # in ONE timed region (252 grouped launches), each linear fed the layer's fresh-standing N(0,1) input of its width
+        n_layers = 36
+        stack = [[(synthetic.make_packed(Q8_0, n, k, seed=20000 + 20 * li + j, device=dev),
+                   synthetic.make_packed(Q8_0, n, k, seed=20010 + 20 * li + j, device=dev)) for j, (_, n, k) in enumerate(shapes)]
+                 for li in range(n_layers)]
+        torch.cuda.synchronize()
+        stack_bytes = sum(a.numel() + b.numel() for layer in stack for a, b in layer)
+        dws = torch.empty(2 * INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
+
+        def stack_pass(i, ws_route):
+            for layer in stack:
+                for j, (_, n, k) in enumerate(shapes):
+                    wu, wg = layer[j]
+                    if ws_route:
+                        ops.grouped_linear_ws_into(xs[k], None, n_text, wu, Q8_0, wg, Q8_0, None, None, ys[n], None, dws, num)
+                    else:
+                        ops.grouped_linear_into(xs[k], None, n_text, wu, Q8_0, wg, Q8_0, None, None, ys[n], None, num)
+
+        stack_flops = n_layers * flops
+        wall_sf, _ = run_region(lambda i: stack_pass(i, False), 2, 1)
+        wall_sw, _ = run_region(lambda i: stack_pass(i, True), 2, 1)
+        result["grouped_stack"] = {
+            "workload": "configs[4]: 36 layers x 2 towers in Q8_0 resident in HBM, 512 text rows -> understanding weights + 4096 "
+                        "image rows -> generation weights through the modality-grouped launcher, 7 linears per layer, all "
+                        "layers in one timed region (linear projections only)",
+            "packed_bytes": stack_bytes, "flop_per_pass": stack_flops,
+            "value": round(stack_flops / (wall_sf / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sf / 2, 3),
+            "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sf / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            "workspace": {"value": round(stack_flops / (wall_sw / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sw / 2, 3),
+                          "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sw / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2)},
+        }
+        del stack, dws, xs, ys
 
     # ---- layer-offload streaming: decoder layers (understanding tower, 7 Q8_0 linears, 205 MB) kept in pinned
     # host arenas and copied in ahead of their forward on a second stream; the host link bounds this leg ----------

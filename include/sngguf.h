@@ -169,6 +169,23 @@ int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int
                          const void* bias, void* y, int numerics, void* stream);
 
 /*
+ * lm_head followed by torch.argmax: out_index[m] = argmax_n bf16(x[m] . W[n]^T + bias[n]), the greedy next token of
+ * the think loop (`torch.argmax(outputs.logits[:, -1, :], dim=-1)`, src/sensenova_u1/models/neo_unify/
+ * modeling_neo_chat.py:557,586, on the logits of `self.lm_head(...)`, modeling_qwen3.py:1264).  The decode kernel's
+ * epilogue keeps one (value, column) candidate per workgroup and activation row instead of storing N logits; a second
+ * small launch picks the winner.  Values compare as the bf16 logits the reference would have stored; among equal
+ * values the lowest column wins, a NaN counts as the largest value (torch.argmax's rules).
+ *
+ *  M <= 16, K % 256 == 0, any of the ten block types (not BF16); anything else is SNGGUF_E_BADSHAPE / _BADTYPE and
+ *  the caller runs sngguf_linear + its own arg-max.
+ *  workspace   device scratch of sngguf_lm_head_argmax_workspace_bytes(M, N) = 8 M ceil(N / 16) bytes, 16-byte aligned
+ *  out_index   int64[M] on the device
+ */
+int64_t sngguf_lm_head_argmax_workspace_bytes(int64_t M, int64_t N);
+int sngguf_lm_head_argmax(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K,
+                          const void* bias, void* workspace, int64_t* out_index, int numerics, void* stream);
+
+/*
  * SiLU-gated pair for the decode MLP: h[M][N] = silu(x.Wg^T) * (x.Wu^T), with both
  * projections rounded to bf16 first, silu evaluated in fp32 on the rounded gate and rounded
  * to bf16, and the product rounded to bf16 - the rounding chain of
@@ -194,6 +211,10 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
  * as sngguf_linear / sngguf_gate_up_silu.
  */
 int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K);
+/* The same norm as a launch of its own, y[M][K] = RMSNorm(x[M][K]; gamma, eps) (Qwen3RMSNorm.forward,
+ * src/sensenova_u1/models/neo_unify/modeling_qwen3.py:192-197), for the row counts the fused entry points do not
+ * take: bf16, 16-byte aligned, K % 8 == 0, y may be x. */
+int sngguf_rmsnorm(const void* x, int64_t M, int64_t K, const void* gamma, float eps, void* y, void* stream);
 int sngguf_rmsnorm_linear(const void* x, int64_t M, const void* gamma, float eps, const void* q, int qtype,
                           int64_t N, int64_t K, const void* bias, void* y, int numerics, void* stream);
 int sngguf_rmsnorm_gate_up_silu(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate,

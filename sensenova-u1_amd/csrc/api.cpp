@@ -12,13 +12,16 @@ int launch_gemv(const void* x, int64_t M, const void* qa, const void* qb, int qt
                 const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream);
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
-                        float eps);
+                        float eps, uint64_t* amax = nullptr);
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
-                        const void* gamma, float eps);
+                        const void* gamma, float eps, uint64_t* amax = nullptr);
+int64_t gemv_argmax_slots(int qtype, int64_t M, int64_t N);
+int launch_argmax_reduce(const uint64_t* keys, int64_t M, int64_t slots, int64_t* out_index, hipStream_t stream);
 int launch_dequantize_bf16(const void* q, int64_t rows, int64_t cols, void* out, int out_dtype, hipStream_t stream);
 int launch_gemv_bf16(const void* x, int64_t M, const void* wa, const void* wb, int64_t N, int64_t K, const void* bias,
                      const void* residual, void* y, bool gated, hipStream_t stream);
+int launch_rmsnorm(const void* x, int64_t M, int64_t K, const void* gamma, float eps, void* y, hipStream_t stream);
 int64_t q8_0_tiled_bytes(int64_t N, int64_t K);
 int64_t static_scratch_bytes();
 int static_scratch(void** ptr);
@@ -287,6 +290,37 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (qtype == SNGGUF_TYPE_BF16)
         return sngguf::launch_gemv_bf16(x, M, q_gate, q_up, N, K, nullptr, nullptr, h, true, static_cast<hipStream_t>(stream));
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+}
+
+int64_t sngguf_lm_head_argmax_workspace_bytes(int64_t M, int64_t N) {
+    return M > 0 && N > 0 && M <= 16 && N < kMaxDim ? 8 * M * ((N + 15) / 16) : 0;
+}
+
+int sngguf_lm_head_argmax(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
+                          void* workspace, int64_t* out_index, int numerics, void* stream) {
+    const int rc = check_matmul(x, M, q, qtype, N, K, x, numerics);      // (no y here: x stands in for its checks)
+    if (rc != SNGGUF_OK || M == 0) return rc;
+    if (N == 0 || M > 16 || K % 256 != 0) return SNGGUF_E_BADSHAPE;     // the matrix-core decode kernels only
+    if (!out_index) return SNGGUF_E_NULLPTR;
+    if (!aligned(out_index, 8)) return SNGGUF_E_ALIGN;
+    if (qtype == SNGGUF_TYPE_BF16) return SNGGUF_E_BADTYPE;
+    if (!workspace) return SNGGUF_E_NULLPTR;
+    if (!aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint64_t* keys = static_cast<uint64_t*>(workspace);
+    const int rl = qtype == SNGGUF_TYPE_Q8_0
+        ? sngguf::launch_gemv_q8_mfma(x, M, q, nullptr, N, K, bias, nullptr, nullptr, numerics, false, s, nullptr, 0.f, keys)
+        : sngguf::launch_gemv_kq_mfma(x, M, q, nullptr, qtype, N, K, bias, nullptr, nullptr, numerics, false, s, nullptr, 0.f, keys);
+    if (rl != SNGGUF_OK) return rl;
+    return sngguf::launch_argmax_reduce(keys, M, sngguf::gemv_argmax_slots(qtype, M, N), out_index, s);
+}
+
+int sngguf_rmsnorm(const void* x, int64_t M, int64_t K, const void* gamma, float eps, void* y, void* stream) {
+    if (M < 0 || K <= 0 || M >= kMaxDim || K >= kMaxDim || K % 8 != 0 || !(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
+    if (M == 0) return SNGGUF_OK;
+    if (!x || !gamma || !y) return SNGGUF_E_NULLPTR;
+    if (!aligned(x, 16) || !aligned(gamma, 16) || !aligned(y, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_rmsnorm(x, M, K, gamma, eps, y, static_cast<hipStream_t>(stream));
 }
 
 int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K) {

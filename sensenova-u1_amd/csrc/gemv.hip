@@ -247,11 +247,32 @@ static int launch_num(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* 
 
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
-                        const void* gamma = nullptr, float eps = 0.f);
+                        const void* gamma = nullptr, float eps = 0.f, uint64_t* amax = nullptr);
 
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
-                        const void* gamma = nullptr, float eps = 0.f);
+                        const void* gamma = nullptr, float eps = 0.f, uint64_t* amax = nullptr);
+
+// Second pass of the arg-max form of the decode kernels: keys[m][slots] -> out_index[m], one workgroup per activation
+// row.  (A key orders by value first and by lower column second, see argmax_key.)
+__global__ __launch_bounds__(256) void argmax_reduce_kernel(const uint64_t* __restrict__ keys, int64_t slots, int64_t* __restrict__ out_index) {
+    __shared__ uint64_t best[256];
+    const uint64_t* row = keys + (int64_t)blockIdx.x * slots;
+    uint64_t k = 0;
+    for (int64_t i = threadIdx.x; i < slots; i += 256) k = u64_max(k, row[i]);
+    best[threadIdx.x] = k;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) best[threadIdx.x] = u64_max(best[threadIdx.x], best[threadIdx.x + off]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out_index[blockIdx.x] = (int64_t)(0xFFFFFFFFu - (uint32_t)best[0]);
+}
+
+int launch_argmax_reduce(const uint64_t* keys, int64_t M, int64_t slots, int64_t* out_index, hipStream_t stream) {
+    argmax_reduce_kernel<<<dim3((unsigned)M), dim3(256), 0, stream>>>(keys, slots, out_index);
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
 
 // M in 1..16 (up to 64 when K % 256 == 0 and not gated), N >= 1, K a positive multiple of the block
 // size (checked by the caller).

@@ -375,7 +375,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                                 const bf16_t* __restrict__ gamma, float eps) {
+                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
     static_assert(!XN || MT == 1, "the fused norm is for at most 16 rows");
     typedef Slab<QT> S;
     constexpr int kRows = 16 * R;
@@ -542,6 +542,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
     for (int t = 0; t < MT; t++) {
         const int m = 16 * t + r;
         if (m >= M) continue;
+        uint64_t best = 0;   // arg-max form: best (value, column) of this workgroup's rows for activation row m
 #pragma unroll
         for (int rg = 0; rg < R; rg++) {
             f32x4_t sum = red[(rg * MT + t) * 64 + lane];
@@ -567,6 +568,12 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
+                if (amax) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < N) best = u64_max(best, argmax_key(o[v], n + v));
+                    continue;
+                }
             }
             bf16_t* yr = y + (int64_t)m * N + n;
             if (n + 3 < N && (N & 3) == 0) {
@@ -577,12 +584,15 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
                     if (n + v < N) yr[v] = f32_to_bf16(o[v]);
             }
         }
+        if constexpr (!GATED) {
+            if (amax) argmax_store(best, g, amax, m, blockIdx.x, gridDim.x);
+        }
     }
 }
 
 template <int QT, int NUM, int R>
 int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-             const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
+             const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream, uint64_t* amax) {
     const int64_t groups = (N + 16 * R - 1) / (16 * R);
     const int nsb = (int)(K >> 8);
     const int mt = (M + 15) / 16;
@@ -615,7 +625,7 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                                    \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH;                                                                 \
         gemv_kq_mfma_kernel<QT, NUM, R, G, WM, 1, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias,    \
-                                                                                           residual, y, gamma, eps);   \
+                                                                                           residual, y, gamma, eps, amax); \
     } while (0)
         if (gated) {
             if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
@@ -629,7 +639,7 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     }
     const size_t lds_bytes = slab > red ? slab : red;
 #define SNGGUF_LAUNCH(G, WM, MT_) \
-    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f)
+    gemv_kq_mfma_kernel<QT, NUM, R, G, WM, MT_><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f, amax)
     if (mt > 1) {
         // more than 16 activation rows: plain projections with one row group per wavefront only
         if constexpr (R == 1) {
@@ -651,23 +661,33 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
+// Row groups per wavefront (see launch_qt) as a function, so that the arg-max caller can size its slot array.
+inline int rows_per_workgroup(int64_t M, int64_t N) { return (N >= 32768 && M <= 16) ? 32 : 16; }
+
 template <int QT, int NUM>
 int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K, const bf16_t* bias,
-              const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream) {
+              const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps, hipStream_t stream, uint64_t* amax) {
     // Two row groups per wavefront only when one per wavefront would already give far more
     // wavefronts than the chip holds (a vocabulary-sized projection): otherwise more, smaller
     // workgroups spread more evenly over the 256 compute units.
-    if (N >= 32768 && M <= 16) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
-    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
+    if (rows_per_workgroup(M, N) == 32) return launch_r<QT, NUM, 2>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream, amax);
+    return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream, amax);
 }
 
 }  // namespace
+
+// Workgroups of a plain decode launch = (value, column) slots per activation row that its arg-max form writes.
+int64_t gemv_argmax_slots(int qtype, int64_t M, int64_t N) {
+    const int64_t rows = qtype == SNGGUF_TYPE_Q8_0 ? 16 : rows_per_workgroup(M, N);   // (Q8_0 has kernels of its own)
+    return (N + rows - 1) / rows;
+}
 
 // 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).  `gamma`
 // (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
-                        const void* gamma, float eps) {
+                        const void* gamma, float eps, uint64_t* amax) {
+    if (amax && (gated || M > 16)) return SNGGUF_E_BADSHAPE;
     const bf16_t* gp = static_cast<const bf16_t*>(gamma);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
@@ -678,9 +698,9 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
 #define SNGGUF_CASE(QT)                                                                                          \
     if (qtype == QT) {                                                                                           \
         if (numerics == SNGGUF_NUM_GGML_FP32)                                                                    \
-            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);          \
+            return launch_qt<QT, SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream, amax);          \
         if (numerics == SNGGUF_NUM_UPSTREAM_FP16)                                                                \
-            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);      \
+            return launch_qt<QT, SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream, amax);      \
         return SNGGUF_E_BADTYPE;                                                                                 \
     }
     SNGGUF_CASE(SNGGUF_TYPE_Q4_0)

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
                                                             const uint8_t* __restrict__ qa,
                                                             const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                             const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                            const bf16_t* __restrict__ gamma, float eps) {
+                                                            const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
     constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
     constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
     constexpr int kPieces = 16 * kRowPieces;      // per slab
@@ -197,6 +197,15 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
     } else {
 #pragma unroll
         for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
+        if (amax) {
+            // arg-max form: this row group's best (value, column) per activation row instead of the outputs
+            uint64_t key = 0;
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (n + v < N) key = u64_max(key, argmax_key(o[v], n + v));
+            argmax_store(key, g, amax, m, blockIdx.x, gridDim.x);
+            return;
+        }
     }
     bf16_t* yr = y + (int64_t)m * N + n;
     if (n + 3 < N && (N & 3) == 0) {
@@ -235,7 +244,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                                 const bf16_t* __restrict__ gamma, float eps) {
+                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
@@ -467,6 +476,15 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     } else {
 #pragma unroll
         for (int v = 0; v < 4; v++) o[v] = n + v < N ? add_residual(sum[v] + (bias ? bf16_to_f32(bias[n + v]) : 0.f), residual, (int64_t)m * N + n + v) : 0.f;
+        if (amax) {
+            // arg-max form: this row group's best (value, column) per activation row instead of the outputs
+            uint64_t key = 0;
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (n + v < N) key = u64_max(key, argmax_key(o[v], n + v));
+            argmax_store(key, g, amax, m, blockIdx.x, gridDim.x);
+            return;
+        }
     }
     bf16_t* yr = y + (int64_t)m * N + n;
     if (n + 3 < N && (N & 3) == 0) {
@@ -481,7 +499,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 template <int NUM>
 static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
                        const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
-                       hipStream_t stream) {
+                       hipStream_t stream, uint64_t* amax) {
     const int64_t groups = (N + 15) / 16;
     const int spans = (int)(K >> 11);
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
@@ -507,7 +525,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL>), \
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
-        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps); \
+        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax); \
     } while (0)
 #define SNGGUF_LAUNCH(G, WM) \
     do { \
@@ -519,7 +537,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, true, 4, false, true>),
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
-        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f);
+        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f, nullptr);
     } else if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
@@ -547,7 +565,7 @@ static int pick_k_split(int64_t groups, int steps, bool gated) {
 template <int NUM, int CB>
 static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
                      const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
-                     hipStream_t stream) {
+                     hipStream_t stream, uint64_t* amax) {
     const int64_t groups = (N + 15) / 16;
     const int steps = (int)(K / (32 * CB));
     const int w = pick_k_split(groups, steps, gated);
@@ -567,7 +585,7 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                                     \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH;                                                                  \
         gemv_q8_mfma_kernel<NUM, CB, G, WM, true><<<grid, block, lds_norm, stream>>>(x, M, qa, qb, N, K, bias, residual, \
-                                                                                     y, gamma, eps);                    \
+                                                                                     y, gamma, eps, amax);              \
     } while (0)
         if (gated) {
             if (waves <= 4) SNGGUF_LAUNCH_XN(true, 4);
@@ -581,7 +599,7 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     }
     const size_t lds_bytes = (size_t)waves * 16 * CB * 34;
     // WMAX only sets the register budget the compiler may assume for the workgroup size
-#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f)
+#define SNGGUF_LAUNCH(G, WM) gemv_q8_mfma_kernel<NUM, CB, G, WM><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f, amax)
     if (gated) {
         if (waves <= 4) SNGGUF_LAUNCH(true, 4);
         else SNGGUF_LAUNCH(true, 8);
@@ -596,7 +614,7 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 template <int NUM>
 static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64_t N, int64_t K,
                      const bf16_t* bias, const bf16_t* residual, bf16_t* y, bool gated, const bf16_t* gamma, float eps,
-                     hipStream_t stream) {
+                     hipStream_t stream, uint64_t* amax) {
     // The line-aligned variant needs whole 2048-element spans per wavefront; with few row groups
     // that leaves the chip short of wavefronts, and the block-aligned variant (which can cut K
     // every 256 elements) is the better fit.
@@ -605,15 +623,18 @@ static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     // activation fragments per weight byte in flight, so the bar is lower there; 4096 -> 4096 loses at every M)
     const int64_t span_waves = ((N + 15) / 16) * (K >> 11) * (gated ? 2 : 1);
     if (K % 2048 == 0 && span_waves >= (M >= 12 ? 1536 : 2048))
-        return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
-    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream);
+        return launch_span<NUM>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream, amax);
+    return launch_cb<NUM, 8>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream, amax);
 }
 
 // Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).  `gamma` (K bf16, 16-byte
-// aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
+// aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.  `amax` (plain projections
+// only): instead of y, every workgroup writes its best (value, column) key per activation row to
+// amax[m * ceil(N / 16) + workgroup].
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,
                         const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
-                        float eps) {
+                        float eps, uint64_t* amax) {
+    if (amax && gated) return SNGGUF_E_BADSHAPE;
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const uint8_t* a = static_cast<const uint8_t*>(qa);
     const uint8_t* b = static_cast<const uint8_t*>(qb);
@@ -621,8 +642,8 @@ int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb
     const bf16_t* rp = static_cast<const bf16_t*>(residual);
     bf16_t* yp = static_cast<bf16_t*>(y);
     const bf16_t* gp = static_cast<const bf16_t*>(gamma);
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream);
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_q8<SNGGUF_NUM_GGML_FP32>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream, amax);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_q8<SNGGUF_NUM_UPSTREAM_FP16>(xp, (int)M, a, b, N, K, bp, rp, yp, gated, gp, eps, stream, amax);
     return SNGGUF_E_BADTYPE;
 }
 

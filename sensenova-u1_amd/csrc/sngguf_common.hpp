@@ -383,6 +383,31 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// ---- arg-max over output columns (lm_head followed by torch.argmax) ------------------------------------------
+// A (value, column) pair packed so that an unsigned 64-bit maximum picks the largest bf16 value and, among equal
+// values, the lowest column - what torch.argmax returns (first maximal index); a NaN counts as the largest value,
+// as it does there.  High word: the bf16 bits mapped to an unsigned number that grows with the value; low word:
+// 2^32 - 1 - column.
+__device__ __forceinline__ uint64_t argmax_key(float v, int64_t n) {
+    const uint32_t b = f32_to_bf16(v);
+    uint32_t k = (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u);
+    if ((b & 0x7FFFu) > 0x7F80u) k = 0xFFFFu;   // NaN of either sign
+    return ((uint64_t)k << 32) | (uint64_t)(0xFFFFFFFFu - (uint32_t)n);
+}
+__device__ __forceinline__ uint64_t u64_max(uint64_t a, uint64_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
+    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, 64), hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, 64);
+    return ((uint64_t)hi << 32) | lo;
+}
+// The four lanes (r, g = 0..3) that hold one activation row's outputs of a 16-row group combine their keys; lane
+// g = 0 then writes the group's entry.  All four lanes of a row take the same branches, so the exchange is safe
+// inside code that rows >= M have left.
+__device__ __forceinline__ void argmax_store(uint64_t key, int g, uint64_t* __restrict__ amax, int m, int64_t slot, int64_t slots) {
+    key = u64_max(key, shfl_xor_u64(key, 16));
+    key = u64_max(key, shfl_xor_u64(key, 32));
+    if (g == 0) amax[(int64_t)m * slots + slot] = key;
+}
+
 // ---- RMSNorm in front of the contraction -------------------------------------------------------------
 // The decoder layers feed q / k / v and gate / up with RMSNorm(hidden) (modeling_qwen3.py:183-197, :919, :938):
 //   v = bf16(x * rsqrt(mean(x^2) + eps))   (fp32 arithmetic, one rounding)      out = bf16(gamma * v)

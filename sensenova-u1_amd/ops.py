@@ -33,9 +33,9 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
-    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_linear_static_max_outputs", "sngguf_linear_static", "sngguf_gate_up_silu", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_linear_static_max_outputs", "sngguf_linear_static", "sngguf_gate_up_silu", "sngguf_lm_head_argmax_workspace_bytes", "sngguf_lm_head_argmax", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
-    "sngguf_rmsnorm_fits", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
+    "sngguf_rmsnorm_fits", "sngguf_rmsnorm", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
@@ -84,6 +84,10 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_static.restype = ci
     lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu.restype = ci
+    lib.sngguf_lm_head_argmax_workspace_bytes.argtypes = [i64, i64]
+    lib.sngguf_lm_head_argmax_workspace_bytes.restype = i64
+    lib.sngguf_lm_head_argmax.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, ci, vp]
+    lib.sngguf_lm_head_argmax.restype = ci
     lib.sngguf_grouped_workspace_bytes.argtypes = [i64]
     lib.sngguf_grouped_workspace_bytes.restype = i64
     lib.sngguf_grouped_linear.argtypes = [vp, i64, vp, i64, vp, ci, vp, ci, i64, i64, vp, vp, vp, vp, ci, vp]
@@ -101,6 +105,8 @@ def load_library() -> ctypes.CDLL:
     cf = ctypes.c_float
     lib.sngguf_rmsnorm_fits.argtypes = [ci, i64, i64]
     lib.sngguf_rmsnorm_fits.restype = ci
+    lib.sngguf_rmsnorm.argtypes = [vp, i64, i64, vp, cf, vp, vp]
+    lib.sngguf_rmsnorm.restype = ci
     lib.sngguf_rmsnorm_linear.argtypes = [vp, i64, vp, cf, vp, ci, i64, i64, vp, vp, ci, vp]
     lib.sngguf_rmsnorm_linear.restype = ci
     lib.sngguf_rmsnorm_gate_up_silu.argtypes = [vp, i64, vp, cf, vp, vp, ci, i64, i64, vp, ci, vp]
@@ -265,9 +271,55 @@ def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, q
     _check(rc, "sngguf_gate_up_silu")
 
 
+def lm_head_argmax_fits(quant_type: int, m: int, k: int) -> bool:
+    """Whether ``lm_head_argmax`` has a fused kernel for ``m`` rows of width ``k`` of this weight type."""
+    return quant_type in GGML_QUANT_SIZES and quant_type != BF16 and 0 < m <= 16 and k % 256 == 0
+
+
+def lm_head_argmax(x: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor] = None,
+                   numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    """``torch.argmax(linear(x), dim=-1)`` without materialising the logits: int64 indices over the leading dims of
+    ``x``.  The greedy-token step of the reference's think loop (``modeling_neo_chat.py:557,586``).  Shapes the fused
+    kernels do not take (more than 16 rows, ``K % 256 != 0``, BF16 rows) run as ``linear`` followed by ``argmax``."""
+    packed, bias = _plain(packed), _plain(bias)
+    _require_device(x, packed, bias)
+    p, n, k = _packed_2d(packed, quant_type)
+    x2d = _as_bf16_rows(x, k, "lm_head_argmax")
+    m = x2d.shape[0]
+    if not lm_head_argmax_fits(quant_type, m, k) or n == 0:
+        if n == 0:
+            raise SnGgufError("lm_head_argmax: the weight has no rows")
+        return torch.ops.sn_gguf.linear(x, p, int(quant_type), bias, int(numerics)).argmax(dim=-1)
+    lib = load_library()
+    ws = torch.empty(int(lib.sngguf_lm_head_argmax_workspace_bytes(m, n)), dtype=torch.uint8, device=x.device)
+    out = torch.empty(x.shape[:-1], dtype=torch.int64, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.sngguf_lm_head_argmax(_ptr(x2d), m, _ptr(p), int(quant_type), n, k, _ptr(_bias_bf16(bias, n, "lm_head_argmax")),
+                                       _ptr(ws), _ptr(out), int(numerics), ctypes.c_void_p(_stream(x.device)))
+    _check(rc, "sngguf_lm_head_argmax")
+    return out
+
+
 def rmsnorm_fits(quant_type: int, m: int, k: int) -> bool:
     """Whether the fused-norm entry points take ``m`` rows of width ``k`` for this weight type."""
     return bool(load_library().sngguf_rmsnorm_fits(quant_type, m, k))
+
+
+def rms_norm(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
+    """``Qwen3RMSNorm.forward`` (``modeling_qwen3.py:192-197``) over the last dim of a bf16 tensor as one library launch."""
+    _require_device(x, gamma)
+    k = x.shape[-1]
+    if x.dtype != torch.bfloat16 or gamma.dtype != torch.bfloat16 or gamma.numel() != k or k % 8 != 0:
+        raise SnGgufError("rms_norm: bf16 rows with a bf16 weight of the same width (a multiple of 8) are needed")
+    x2d = x.reshape(-1, k)
+    x2d = x2d if x2d.is_contiguous() else x2d.contiguous()
+    y = torch.empty_like(x2d)
+    if x2d.shape[0]:
+        with torch.cuda.device(x.device):
+            rc = load_library().sngguf_rmsnorm(_ptr(x2d), x2d.shape[0], k, _ptr(gamma.contiguous()), float(eps), _ptr(y),
+                                               ctypes.c_void_p(_stream(x.device)))
+        _check(rc, "sngguf_rmsnorm")
+    return y.reshape(x.shape)
 
 
 def rmsnorm_linear_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, packed: torch.Tensor, quant_type: int,

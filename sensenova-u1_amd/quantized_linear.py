@@ -149,7 +149,11 @@ def set_decode_layout(model: nn.Module, layout: str = "tiled", build_now: bool =
 
 def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMSNorm as the decoder layers compute it (``Qwen3RMSNorm.forward``, ``modeling_qwen3.py:192-197``): statistic
-    and scaling in fp32, one rounding to the input dtype, then the product with the weight in that dtype."""
+    and scaling in fp32, one rounding to the input dtype, then the product with the weight in that dtype.  bf16 rows
+    on the device run as one library launch (``sngguf_rmsnorm``), anything else as the tensor operations."""
+    if (hidden_states.is_cuda and weight.is_cuda and hidden_states.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and hidden_states.shape[-1] % 8 == 0 and weight.numel() == hidden_states.shape[-1]):
+        return ops.rms_norm(hidden_states, weight, eps)        # the library's one-launch form
     h = hidden_states.float()
     h = h * torch.rsqrt(h.square().mean(dim=-1, keepdim=True) + eps)
     return weight * h.to(hidden_states.dtype)
@@ -305,6 +309,14 @@ class GGUFLinear(nn.Linear):
             ops.rmsnorm_linear_into(x2d, norm_weight.contiguous(), eps, self.weight, self._weight_type(), bias,
                                     out.view(-1, self.out_features), self.numerics)
         return out
+
+    def forward_argmax(self, inputs: torch.Tensor) -> torch.Tensor:
+        """``torch.argmax(self(inputs), dim=-1)`` - the greedy next-token step on an ``lm_head``
+        (``modeling_neo_chat.py:557,586``) - with the arg-max taken in the projection kernel's epilogue at decode, so the
+        vocabulary-sized logits row is never written."""
+        if inputs.dtype != torch.bfloat16 or (self.compute_dtype or inputs.dtype) != torch.bfloat16:
+            return self.forward(inputs).argmax(dim=-1)
+        return ops.lm_head_argmax(inputs, self.weight, self._weight_type(), self.bias, self.numerics)
 
     def forward_residual(self, inputs: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
         """``residual + self(inputs)`` (the decoder layer's ``hidden_states = residual + o_proj(...)`` /

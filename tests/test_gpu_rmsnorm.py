@@ -162,3 +162,43 @@ def test_rmsnorm_tiled_parity(dev, c_oracle, shape):
         big = synthetic.make_activations(16, k, seed=1).to(dev)
         with pytest.raises(ops.SnGgufError):
             ops.rmsnorm_linear_tiled_into(big, gamma.to(dev), EPS, tg, None, torch.empty((16, n), dtype=torch.bfloat16, device=dev), 1)
+
+
+@pytest.mark.parametrize("m,k", [(1, 4096), (4, 4096), (16, 4096), (3, 264), (40, 12288), (2, 16384), (2, 20480), (0, 64)])
+def test_standalone_rmsnorm_launch(dev, m, k):
+    """sngguf_rmsnorm against the oracle's Qwen3RMSNorm: the row statistic is summed in another order, so a normalized
+    value may sit one bf16 step off on a near tie; everything else is the same two roundings."""
+    print(f"case rmsnorm standalone m={m} k={k}", flush=True)
+    x = (synthetic.make_activations(max(m, 1), k, seed=m + k).float() * 2.5).to(torch.bfloat16)[:m]
+    gamma = _gamma(k, k + 1)
+    got = ops.rms_norm(x.to(dev), gamma.to(dev), EPS).cpu()
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    if m == 0:
+        return
+    want = go.qwen3_rms_norm(x, gamma, EPS)
+    assert go.rel_l2(got, want) <= 1e-3
+    frac = (got.view(torch.int16) != want.view(torch.int16)).float().mean().item()
+    assert frac < 0.01, frac
+    step = (got.float() - want.float()).abs() <= want.float().abs() * 2.0 ** -7 + 1e-30
+    assert bool(step.all())
+    # identity weight: the normalized rows themselves
+    one = torch.ones(k, dtype=torch.bfloat16)
+    got1 = ops.rms_norm(x.to(dev), one.to(dev), EPS).cpu()
+    assert (got1.view(torch.int16) != go.qwen3_rms_norm(x, one, EPS).view(torch.int16)).float().mean().item() < 0.01
+
+
+def test_module_helpers_use_the_library_norm_beyond_the_fused_row_count(dev):
+    from sensenova_u1_amd import GGUFLinear, GGUFParameter
+    from sensenova_u1_amd.quantized_linear import rms_norm
+    n, k = 512, 4096
+    packed = synthetic.make_packed(go.Q8_0, n, k, seed=7)
+    lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+    lin.weight = GGUFParameter(packed.to(dev), quant_type=go.Q8_0)
+    gamma = _gamma(k, 3)
+    for m in (4, 16, 100):
+        x = (synthetic.make_activations(m, k, seed=m).float() * 1.7).to(torch.bfloat16)
+        assert not ops.rmsnorm_fits(go.Q8_0, m, k)
+        got = lin.forward_normed(x.to(dev), gamma.to(dev), EPS).cpu()
+        want = go.gguf_linear_forward(go.qwen3_rms_norm(x, gamma, EPS), packed, go.Q8_0)
+        assert go.rel_l2(got, want) <= TOL
+        assert torch.equal(rms_norm(x.to(dev), gamma.to(dev), EPS), ops.rms_norm(x.to(dev), gamma.to(dev), EPS))
