@@ -244,20 +244,26 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                                                                  const uint8_t* __restrict__ qa,
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
+                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax,
+                                                                 int gpw) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
     constexpr int NQ = PAIRED ? 2 : 1;   // matrices per wavefront
+    // A workgroup holds gpw row groups (all wavefronts of a compute unit in one workgroup start together and share
+    // one staged copy of the activations); wavefronts [grp * wpg, (grp + 1) * wpg) work on row group grp of it.
     const int waves = blockDim.x >> 6;
-    const int W = (GATED && !PAIRED) ? waves >> 1 : waves;
-    const int kw = (GATED && !PAIRED) ? (wave >= W ? wave - W : wave) : wave;
-    const uint8_t* __restrict__ q = (GATED && !PAIRED && wave >= W) ? qb : qa;
+    const int wpg = waves / gpw;
+    const int grp = wave / wpg, lw = wave - grp * wpg, wbase = grp * wpg;
+    const int W = (GATED && !PAIRED) ? wpg >> 1 : wpg;
+    const int kw = (GATED && !PAIRED) ? (lw >= W ? lw - W : lw) : lw;
+    const uint8_t* __restrict__ q = (GATED && !PAIRED && lw >= W) ? qb : qa;
     const int r = lane & 15, g = lane >> 4;
     const int64_t row_bytes = (K >> 5) * 34;
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t n0 = ((int64_t)blockIdx.x * gpw + grp) * 16;
+    const bool live = n0 < N;            // the last workgroup's row groups may lie past the end: those wavefronts idle
     const int spans = (int)(K >> 11);
-    const int t0 = (int)((int64_t)kw * spans / W), t1 = (int)((int64_t)(kw + 1) * spans / W);
+    const int t0 = live ? (int)((int64_t)kw * spans / W) : 0, t1 = live ? (int)((int64_t)(kw + 1) * spans / W) : 0;
 
     // Two-line fetch: piece lane + 64 i is bytes [16 c, +16) of the 256-byte window of row
     // (lane / 16) + 4 i, c = lane % 16.  One-line fetch: row (lane / 8) + 8 i, piece lane % 8.
@@ -447,23 +453,26 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 
     // ---- add the wavefronts' partial sums (the rings are dead: reuse them) ---------------------------
     __syncthreads();
-    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [gate partial sums of the W K ranges | up partial sums][64]
+    // per row group: [gate partial sums of the W K ranges | up partial sums][64]; the paired mode keeps the up sums of
+    // all wavefronts behind the gate sums of all wavefronts
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);
     red[wave * 64 + lane] = acc[0];
-    if constexpr (PAIRED) red[(W + wave) * 64 + lane] = acc[NQ - 1];
+    if constexpr (PAIRED) red[(waves + wave) * 64 + lane] = acc[NQ - 1];
     __syncthreads();
-    if (wave != 0 || !has_x) return;
-    f32x4_t sum = red[lane];
+    if (lw != 0 || !has_x || !live) return;
+    f32x4_t sum = red[wbase * 64 + lane];
     for (int w = 1; w < W; w++) {
-        const f32x4_t v = red[w * 64 + lane];
+        const f32x4_t v = red[(wbase + w) * 64 + lane];
         sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
     }
     const int m = r;
     const int64_t n = n0 + 4 * g;
     float o[4];
     if constexpr (GATED) {
-        f32x4_t up = red[W * 64 + lane];
+        const int ubase = PAIRED ? waves + wbase : wbase + W;
+        f32x4_t up = red[ubase * 64 + lane];
         for (int w = 1; w < W; w++) {
-            const f32x4_t v = red[(W + w) * 64 + lane];
+            const f32x4_t v = red[(ubase + w) * 64 + lane];
             up[0] += v[0]; up[1] += v[1]; up[2] += v[2]; up[3] += v[3];
         }
 #pragma unroll
@@ -482,7 +491,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 #pragma unroll
             for (int v = 0; v < 4; v++)
                 if (n + v < N) key = u64_max(key, argmax_key(o[v], n + v));
-            argmax_store(key, g, amax, m, blockIdx.x, gridDim.x);
+            argmax_store(key, g, amax, m, (int64_t)blockIdx.x * gpw + grp, (N + 15) >> 4);
             return;
         }
     }
@@ -505,46 +514,51 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     int w = spans < 8 ? spans : 8;                 // one wavefront per span, at most 8 per row group
     if (gated && w > 4) w = 4;
     // (no cap for many row groups: a 151936-row projection runs 3 - 5 % faster with two wavefronts per group than with one)
-    // stage the activations in LDS when they are small enough to leave room for three workgroups
-    // per compute unit (or, for few row groups, one)
+    // stage the activations in LDS when they are small enough to leave room for a compute unit's worth of rings
     const size_t x_bytes = (size_t)M * (2 * K + 64);
-    const size_t x_budget = groups >= 512 ? 16 * 1024 : 96 * 1024;
+    const size_t x_budget = groups >= 512 ? 48 * 1024 : 96 * 1024;   // (5 rows at K = 4096: M = 4 gate/up 24.6 against 25.1 us fetched per wavefront)
     const bool xlds = x_bytes <= x_budget;
     // activations fetched from global memory for a gated pair: one wavefront takes both matrices of its K range
     const bool paired = gated && !xlds && M >= kPairedMinM;
-    const int waves = (gated && !paired) ? 2 * w : w;
-    const size_t ring_bytes = (size_t)(gated ? 2 * w : w) * 16 * kRingRow;
+    const int wpg = (gated && !paired) ? 2 * w : w;                       // wavefronts per row group
+    const size_t ring_per_wave = (size_t)(paired ? 2 : 1) * 16 * kRingRow;
     if (gamma && !xlds) return SNGGUF_E_BADSHAPE;   // the norm is applied to activations staged in LDS
-    const size_t lds_bytes = ring_bytes + (xlds ? x_bytes : 0) + (gamma ? (((size_t)4 * M * waves + 15) & ~(size_t)15) : 0);
-    const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
-    // the rings of 8 wavefronts plus staged activations can exceed the default dynamic-LDS limit:
-    // raise it once per kernel instance
-#define SNGGUF_LAUNCH_ONE(G, WM, XL) \
+    // Row groups per workgroup: all (about 12) wavefronts of a compute unit in ONE workgroup.  Workgroups that arrive
+    // on a compute unit one after the other keep the order of their first requests for the whole kernel - the last
+    // one finishes microseconds after the first - while the wavefronts of one workgroup start together and share
+    // one staged copy of the activations.
+    auto lds_for = [&](int g) {
+        const size_t wv = (size_t)g * wpg;
+        return wv * ring_per_wave + (xlds ? x_bytes : 0) + (gamma ? (((size_t)4 * M * wv + 15) & ~(size_t)15) : 0);
+    };
+    int gpw = xlds ? 12 / wpg : 1;   // (without a staged copy to share, small workgroups did better: M = 16 gate/up 29.2 against 30.5 us)
+    if (gpw < 1) gpw = 1;
+    while (gpw > 1 && (lds_for(gpw) > 160 * 1024 || groups < (int64_t)256 * gpw)) gpw--;
+    const int waves = gpw * wpg;
+    const size_t lds_bytes = lds_for(gpw);
+    if (lds_bytes > 160 * 1024) return SNGGUF_E_BADSHAPE;
+    const dim3 grid((unsigned)((groups + gpw - 1) / gpw)), block((unsigned)(64 * waves));
+    // the rings of a dozen wavefronts plus staged activations exceed the default dynamic-LDS limit: raise it once per
+    // kernel instance
+#define SNGGUF_LAUNCH_ONE(G, WM, XL, PR) \
     do { \
         static const hipError_t attr = hipFuncSetAttribute( \
-            reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL>), \
+            reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL, PR>), \
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
-        gemv_q8_span_kernel<NUM, G, WM, XL><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax); \
+        gemv_q8_span_kernel<NUM, G, WM, XL, PR><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax, gpw); \
     } while (0)
-#define SNGGUF_LAUNCH(G, WM) \
+#define SNGGUF_LAUNCH(G, XL, PR) \
     do { \
-        if (xlds) SNGGUF_LAUNCH_ONE(G, WM, true); \
-        else SNGGUF_LAUNCH_ONE(G, WM, false); \
+        if (waves <= 4) SNGGUF_LAUNCH_ONE(G, 4, XL, PR); \
+        else if (waves <= 8) SNGGUF_LAUNCH_ONE(G, 8, XL, PR); \
+        else SNGGUF_LAUNCH_ONE(G, 12, XL, PR); \
     } while (0)
-    if (paired) {
-        static const hipError_t attr = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, true, 4, false, true>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
-        gemv_q8_span_kernel<NUM, true, 4, false, true><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, nullptr, 0.f, nullptr);
-    } else if (gated) {
-        if (waves <= 4) SNGGUF_LAUNCH(true, 4);
-        else SNGGUF_LAUNCH(true, 8);
-    } else {
-        if (waves <= 4) SNGGUF_LAUNCH(false, 4);
-        else SNGGUF_LAUNCH(false, 8);
-    }
+    if (paired) SNGGUF_LAUNCH(true, false, true);
+    else if (gated && xlds) SNGGUF_LAUNCH(true, true, false);
+    else if (gated) SNGGUF_LAUNCH(true, false, false);
+    else if (xlds) SNGGUF_LAUNCH(false, true, false);
+    else SNGGUF_LAUNCH(false, false, false);
 #undef SNGGUF_LAUNCH
 #undef SNGGUF_LAUNCH_ONE
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
