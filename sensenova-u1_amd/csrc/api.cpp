@@ -467,6 +467,33 @@ int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator,
                              int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
                              const void* bias_gen, void* y, void* workspace, void* dense_workspace,
                              int64_t dense_workspace_bytes, int numerics, void* stream) {
+    // The contiguous [text rows | image rows] layout needs no row map, so the two groups are two plain problems on
+    // consecutive row ranges: each takes the route sngguf_linear_ws would pick for its own row count (a few hundred
+    // text rows: K split without a weight pass; thousands of image rows: weight pass + dense kernel), one after the
+    // other on the stream with the same workspace.  Measured on a 512 + 4096-row layer of seven Q8_0 projections:
+    // 1.9 ms against 2.3 ms for one dense launch over both groups, which decodes the understanding weights in full
+    // for two row tiles.
+    if (!indicator && dense_workspace && n_text >= 0 && n_text <= M && M > 0 && N > 0) {
+        int rc = check_matmul(x, M, q_und, qtype_und, N, K, y, numerics);
+        if (rc != SNGGUF_OK) return rc;
+        rc = check_matmul(x, M, q_gen, qtype_gen, N, K, y, numerics);
+        if (rc != SNGGUF_OK) return rc;
+        if (!aligned(dense_workspace, 16)) return SNGGUF_E_ALIGN;
+        // (a group boundary at an odd row of an odd-width matrix would leave the second group's rows 2-byte aligned)
+        const bool split_ok = (2 * n_text * K) % 16 == 0 && (2 * n_text * N) % 16 == 0;
+        if (split_ok) {
+            const char* xp = static_cast<const char*>(x);
+            char* yp = static_cast<char*>(y);
+            if (n_text > 0) {
+                rc = linear_ws_impl(xp, n_text, q_und, qtype_und, N, K, bias_und, yp, dense_workspace, dense_workspace_bytes, numerics, stream);
+                if (rc != SNGGUF_OK) return rc;
+            }
+            if (n_text < M)
+                rc = linear_ws_impl(xp + 2 * n_text * K, M - n_text, q_gen, qtype_gen, N, K, bias_gen, yp + 2 * n_text * N, dense_workspace,
+                                    dense_workspace_bytes, numerics, stream);
+            return rc;
+        }
+    }
     const bool two_pass = dense_workspace && dense_workspace_bytes >= 4 * N * K && K > 0 && N > 0 && grouped_dense_route_fits(M, N, K);
     // Few output tiles (narrow matrices such as k / v, or a few hundred rows) of one type the large-tile kernel decodes
     // itself: K split over workgroups, the fp32 partial sums in the dense workspace (as sngguf_linear_ws does)

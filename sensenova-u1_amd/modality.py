@@ -32,8 +32,10 @@ def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[t
     ``image_gen_indicators`` is a bool tensor over the leading dims.  When the layout is known
     to be ``[text rows | image rows]`` pass ``image_gen_indicators=None`` and ``n_text`` instead:
     no row map is built and both groups stream contiguous rows.  In that form, with more than 64
-    rows and unless ``proj.gemm_policy`` is ``"fused"``, each group goes through its module's
-    forward (bf16 weight pass + dense GEMM, see ``GGUFLinear``) and writes its slice of the result.
+    rows, ``proj.gemm_policy`` decides as it does for a single module: ``"auto"`` runs
+    ``sngguf_grouped_linear_ws`` on a pooled workspace (each group on the library kernels its row count calls
+    for), ``"fused"`` the fused grouped kernel, ``"two_pass"`` / ``"resident"`` a weight pass + the device
+    library's GEMM per group.
     """
     for mod in (proj, proj_mot_gen):
         if type(mod).__name__ != "GGUFLinear":
@@ -49,6 +51,16 @@ def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[t
             if not 0 <= split <= x2d.shape[0]:
                 raise ValueError(f"n_text={split} is outside 0..{x2d.shape[0]}")
             out = torch.empty((x2d.shape[0], proj.out_features), dtype=torch.bfloat16, device=hidden_states.device)
+            if proj.gemm_policy == "auto":
+                # the library's workspace route: each group takes the kernels its own row count calls for
+                x2d = proj._checked_rows(hidden_states)
+                proj_mot_gen._checked_rows(hidden_states)
+                ws = ops.pooled_workspace(x2d.device, ops.linear_workspace_bytes(proj.out_features, proj.in_features))
+                bu = proj.bias.detach().to(torch.bfloat16).contiguous() if proj.bias is not None else None
+                bg = proj_mot_gen.bias.detach().to(torch.bfloat16).contiguous() if proj_mot_gen.bias is not None else None
+                ops.grouped_linear_ws_into(x2d, None, split, proj.weight, int(proj.weight.quant_type), proj_mot_gen.weight,
+                                           int(proj_mot_gen.weight.quant_type), bu, bg, out, None, ws, proj.numerics)
+                return out.reshape(*hidden_states.shape[:-1], proj.out_features)
             for mod, lo, hi in ((proj, 0, split), (proj_mot_gen, split, x2d.shape[0])):
                 if hi - lo > 64:
                     mod.two_pass_into(x2d[lo:hi], out[lo:hi])

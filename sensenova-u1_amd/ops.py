@@ -215,6 +215,29 @@ def grouped_workspace_bytes(m: int) -> int:
     return int(load_library().sngguf_grouped_workspace_bytes(m))
 
 
+_workspaces: dict = {}
+
+
+def pooled_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """A device scratch tensor of at least ``nbytes`` bytes for the workspace entry points, kept per (device, stream)
+    and grown on demand, so that a forward pass over many modules allocates once.  Calls on one stream are ordered, and
+    nothing in a workspace outlives the call that filled it.  While a HIP graph is being captured a fresh tensor is
+    handed out instead (it then belongs to the graph's own memory pool)."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def release_workspaces() -> None:
+    """Drop the pooled workspaces (they are reallocated on the next call that needs one)."""
+    _workspaces.clear()
+
+
 def linear_workspace_bytes(n: int, k: int) -> int:
     """Bytes of workspace with which ``linear_ws_into`` can take the weight-pass route (2 * n * k)."""
     return int(load_library().sngguf_linear_workspace_bytes(n, k))

@@ -167,13 +167,13 @@ class GGUFLinear(nn.Linear):
     when ``in_features`` is a multiple of 256 - it is one fused dequant-GEMV launch that streams and
     decodes the weights once.  With more rows ``gemm_policy`` decides:
 
-    * ``"auto"``: ``"two_pass"``, except for up to 256 rows of a Q8_0 / Q4_K weight, where the library's
-      large-tile kernel with K split over workgroups (``sngguf_linear_ws``, fp32 partial sums in a transient
-      workspace of at most 2 * N * K bytes) is the faster one: 12288 -> 4096 at 128 rows 42 us against 74 us.
-    * ``"two_pass"``: one HIP dequantize launch writes the bf16 weight
-      (2 * N * K bytes of transient memory) and the device's dense GEMM consumes it.  Measured on
-      MI355X this is the faster route from there on: the weight pass costs about 30 us for a
-      12288 x 4096 matrix and the dense GEMM then runs at 1.5 PFLOP/s.
+    * ``"auto"`` (default): the library's own kernels through ``sngguf_linear_ws`` with a pooled workspace of
+      2 * N * K bytes (``ops.pooled_workspace``, one per device and stream, reused by every module): problems with few
+      output tiles run the large-tile kernel with K split over workgroups, the rest one weight pass into the
+      workspace (bf16, the same rounding chain) followed by the library's dense bf16 tile kernel.
+    * ``"two_pass"`` (opt-in): one HIP dequantize launch writes a transient bf16 weight and the device library's
+      dense GEMM (``torch.matmul``) consumes it: no kernel of this library does the contraction then.  At 4096 rows it
+      is about 10 % faster than ``"auto"`` on MI355X.
     * ``"fused"``: the fused dequant-GEMM kernels of the library (``sngguf_linear``), which need
       no transient memory.
     * ``"resident"``: as ``"two_pass"``, but the bf16 weight is kept (2 * N * K bytes per module) and
@@ -268,13 +268,10 @@ class GGUFLinear(nn.Linear):
                 raise ValueError(f"GGUFLinear.gemm_policy is {self.gemm_policy!r}; expected 'auto', 'two_pass', 'fused' or 'resident'")
             x2d = self._checked_rows(inputs)
             out = torch.empty((*inputs.shape[:-1], self.out_features), dtype=torch.bfloat16, device=inputs.device)
-            tiles = (self.out_features + 255) // 256     # output tiles of 256 x 256 for up to 256 rows
-            split_k = (self.gemm_policy == "auto" and rows <= 256 and tiles <= 128 and self.in_features >= 256
-                       and self.in_features % 64 == 0 and qtype in (ops.Q8_0, ops.Q4_K))
-            if split_k:
-                # room for as many K slices as the library will want: 256 / tiles of them, M * N floats each
-                nbytes = min(2 * self.out_features * self.in_features, 4 * max(2, 256 // tiles) * rows * self.out_features)
-                workspace = torch.empty(nbytes, dtype=torch.uint8, device=inputs.device)
+            if self.gemm_policy == "auto":
+                # the library's own kernels: K split over workgroups for few output tiles, else one weight pass into the
+                # pooled workspace + the dense tile kernel (sngguf_linear_ws picks)
+                workspace = ops.pooled_workspace(inputs.device, ops.linear_workspace_bytes(self.out_features, self.in_features))
                 bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
                 ops.linear_ws_into(x2d, self.weight, qtype, bias, out.view(-1, self.out_features), workspace, self.numerics)
             else:
