@@ -204,8 +204,8 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
  *     n = bf16( gamma * v )                       gamma: the norm's weight, K bf16 values, 16-byte aligned
  * and these two entry points contract n instead of x, applying the norm to the activations a workgroup has
  * staged in LDS - no launch and no buffer for the normalized rows.  Offered where that staging exists
- * (sngguf_rmsnorm_fits: any of the ten types, K % 256 == 0, M (2 K + 64) <= 16384, i.e. one row at K = 4096,
- * three at 2048); other sizes return SNGGUF_E_BADSHAPE and the caller runs the norm on its own.
+ * (sngguf_rmsnorm_fits: any of the ten types, K % 256 == 0, M (2 K + 64) <= 36864, i.e. four rows at K = 4096,
+ * eight at 2048); other sizes return SNGGUF_E_BADSHAPE and the caller runs the norm on its own.
  * The sum of squares is added up in a different order than torch's mean, so a normalized value can differ
  * from the reference's by one bf16 unit where the rounding is a near tie; everything after is the same chain
  * as sngguf_linear / sngguf_gate_up_silu.

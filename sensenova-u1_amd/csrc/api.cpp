@@ -324,8 +324,10 @@ int sngguf_rmsnorm(const void* x, int64_t M, int64_t K, const void* gamma, float
 }
 
 int sngguf_rmsnorm_fits(int qtype, int64_t M, int64_t K) {
-    // the fused norm works on activations staged in LDS: rows of whole 256-element runs, M (2 K + 64) <= 16 KB
-    return known_type(qtype) && qtype != SNGGUF_TYPE_BF16 && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 16384;
+    // the fused norm works on activations staged in LDS: rows of whole 256-element runs, M (2 K + 64) <= 36 KB
+    // (four rows at K = 4096, eight at 2048; with the decode kernels' slabs, and the rows staged twice by a gated pair,
+    // that stays within a compute unit's 160 KB for every type)
+    return known_type(qtype) && qtype != SNGGUF_TYPE_BF16 && M >= 1 && K > 0 && K < kMaxDim && K % 256 == 0 && M * (2 * K + 64) <= 36864;
 }
 
 namespace {

@@ -610,7 +610,7 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     if (gamma) {
         // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares; the
-        // caller keeps M (2 K + 64) within 16 KB
+        // caller keeps M (2 K + 64) within 36 KB
         if (mt > 1) return SNGGUF_E_BADSHAPE;
         const size_t xrow_b = (size_t)((nsb + w - 1) / w) * 512 + 16;
         const size_t staged = slab + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
@@ -683,7 +683,7 @@ int64_t gemv_argmax_slots(int qtype, int64_t M, int64_t N) {
 }
 
 // 1 <= M <= 64 (SiLU-gated pair: M <= 16), K % 256 == 0, 16-byte aligned x and q (checked by the caller).  `gamma`
-// (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
+// (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 36 KB then.
 int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb, int qtype, int64_t N, int64_t K,
                         const void* bias, const void* residual, void* y, int numerics, bool gated, hipStream_t stream,
                         const void* gamma, float eps, uint64_t* amax) {

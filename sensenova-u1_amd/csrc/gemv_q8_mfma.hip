@@ -587,7 +587,7 @@ static int launch_cb(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
     if (gamma) {
         // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares.
-        // The caller keeps M (2 K + 64) within 16 KB; a gated pair stages the rows twice (gate and up wavefronts),
+        // The caller keeps M (2 K + 64) within 36 KB; a gated pair stages the rows twice (gate and up wavefronts),
         // so with the slabs this can pass the default dynamic-LDS limit: raise it once per kernel instance
         const size_t xrow_b = (size_t)((steps + w - 1) / w) * CB * 64 + 16;
         const size_t lds_norm = (size_t)waves * 16 * CB * 34 + (size_t)waves * M * xrow_b + (((size_t)4 * M * waves + 15) & ~(size_t)15);
@@ -642,7 +642,7 @@ static int launch_q8(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* q
 }
 
 // Q8_0, 1 <= M <= 16, K % 256 == 0, 16-byte aligned rows (checked by the caller).  `gamma` (K bf16, 16-byte
-// aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.  `amax` (plain projections
+// aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 36 KB then.  `amax` (plain projections
 // only): instead of y, every workgroup writes its best (value, column) key per activation row to
 // amax[m * ceil(N / 16) + workgroup].
 int launch_gemv_q8_mfma(const void* x, int64_t M, const void* qa, const void* qb, int64_t N, int64_t K, const void* bias,

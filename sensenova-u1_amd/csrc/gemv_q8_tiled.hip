@@ -220,7 +220,7 @@ int launch_tiled(const bf16_t* x, int M, const uint8_t* ta, const uint8_t* tb, i
     const int64_t groups = (N + 15) / 16;
     const int runs = (int)(K >> 8);
     const size_t x_bytes = (size_t)M * (2 * K + 64);
-    const bool xlds = x_bytes <= 16 * 1024;
+    const bool xlds = x_bytes <= 16 * 1024 || (gamma != nullptr && x_bytes <= 36 * 1024);   // (the fused norm needs the staged copy)
     // wavefronts per matrix and row group: measured best at 8 (4 for the gated pair, which doubles them), never more
     // than there are runs.  With the activations fetched from global memory, fewer when the row groups alone fill the
     // chip several times over (a 151936-row projection at M = 4: 128 us with one wavefront per group, 159 us with eight);
@@ -273,7 +273,7 @@ int launch_q8_0_tile(const void* q, int64_t N, int64_t K, void* tiled, hipStream
 }
 
 // 1 <= M <= 16, K % 256 == 0, 16-byte aligned pointers (checked by the caller).
-// `gamma` (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 16 KB then.
+// `gamma` (K bf16, 16-byte aligned) switches the fused RMSNorm on; the caller keeps M (2 K + 64) <= 36 KB then.
 int launch_gemv_q8_tiled(const void* x, int64_t M, const void* ta, const void* tb, int64_t N, int64_t K, const void* bias,
                          const void* residual, void* y, int numerics, bool gated, hipStream_t stream, const void* gamma,
                          float eps) {

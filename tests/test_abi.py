@@ -87,15 +87,15 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_grouped_linear_ws(p, 4, None, 9, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_SHAPE
     assert lib.sngguf_grouped_linear_ws(p, 4, p, 0, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == E_NULL
     assert lib.sngguf_grouped_linear_ws(p, 0, None, 0, p, 8, p, 8, 4, 64, None, None, p, None, None, 0, 1, None) == 0
-    # RMSNorm fused in front of a decode projection: rows of whole 256-element runs, M (2 K + 64) <= 16 KB
-    assert lib.sngguf_rmsnorm_fits(8, 1, 4096) == 1 and lib.sngguf_rmsnorm_fits(8, 2, 4096) == 0
-    assert lib.sngguf_rmsnorm_fits(8, 3, 2048) == 1 and lib.sngguf_rmsnorm_fits(8, 1, 4128) == 0   # K % 256
+    # RMSNorm fused in front of a decode projection: rows of whole 256-element runs, M (2 K + 64) <= 36 KB
+    assert lib.sngguf_rmsnorm_fits(8, 1, 4096) == 1 and lib.sngguf_rmsnorm_fits(8, 4, 4096) == 1 and lib.sngguf_rmsnorm_fits(8, 5, 4096) == 0
+    assert lib.sngguf_rmsnorm_fits(8, 8, 2048) == 1 and lib.sngguf_rmsnorm_fits(8, 1, 4128) == 0   # K % 256
     assert lib.sngguf_rmsnorm_fits(12, 1, 4096) == 1 and lib.sngguf_rmsnorm_fits(8, 0, 4096) == 0
     assert lib.sngguf_rmsnorm_fits(16, 1, 4096) == 0 and lib.sngguf_rmsnorm_fits(2, 1, 4128) == 0   # unknown type; Q4_0 rows of 129 blocks
     eps = ctypes.c_float(1e-6)
     assert lib.sngguf_rmsnorm_linear(p, 1, p, eps, p, 16, 16, 256, None, p, 1, None) == E_TYPE       # unknown type
     assert lib.sngguf_rmsnorm_linear(p, 1, p, eps, p, 2, 16, 288, None, p, 1, None) == E_SHAPE       # Q4_0, K % 256
-    assert lib.sngguf_rmsnorm_linear(p, 2, p, eps, p, 8, 16, 4096, None, p, 1, None) == E_SHAPE      # rows do not fit
+    assert lib.sngguf_rmsnorm_linear(p, 5, p, eps, p, 8, 16, 4096, None, p, 1, None) == E_SHAPE      # rows do not fit
     assert lib.sngguf_rmsnorm_linear(p, 1, None, eps, p, 8, 16, 256, None, p, 1, None) == E_NULL     # gamma
     assert lib.sngguf_rmsnorm_linear(p, 1, odd, eps, p, 8, 16, 256, None, p, 1, None) == E_ALIGN
     assert lib.sngguf_rmsnorm_linear(p, 1, p, ctypes.c_float(-1.0), p, 8, 16, 256, None, p, 1, None) == E_SHAPE
@@ -103,7 +103,7 @@ def test_argument_validation_needs_no_device():
     assert lib.sngguf_rmsnorm_linear(p, 0, p, eps, p, 8, 16, 256, None, p, 1, None) == 0
     assert lib.sngguf_rmsnorm_gate_up_silu(p, 1, p, eps, p, None, 8, 16, 256, p, 1, None) == E_NULL
     assert lib.sngguf_rmsnorm_gate_up_silu(p, 1, p, eps, p, p, 8, 16, 256, p, 7, None) == E_TYPE
-    assert lib.sngguf_rmsnorm_linear_tiled(p, 2, p, eps, p, 16, 4096, None, p, 1, None) == E_SHAPE
+    assert lib.sngguf_rmsnorm_linear_tiled(p, 5, p, eps, p, 16, 4096, None, p, 1, None) == E_SHAPE
     assert lib.sngguf_rmsnorm_linear_tiled(p, 1, None, eps, p, 16, 256, None, p, 1, None) == E_NULL
     assert lib.sngguf_rmsnorm_linear_tiled(p, 0, p, eps, p, 16, 256, None, p, 1, None) == 0
     assert lib.sngguf_rmsnorm_gate_up_silu_tiled(p, 1, p, eps, p, None, 16, 256, p, 1, None) == E_NULL

@@ -88,8 +88,9 @@ def test_grouped_modules(tmp_path, dev):
 
 @pytest.mark.parametrize("quant", [8, 12, 2, 11])
 def test_gemm_policies_agree_with_the_oracle(tmp_path, dev, quant):
-    """More than 16 rows: "fused" (library GEMM kernels) and "auto" / "two_pass" (bf16 weight pass + dense
-    GEMM) both reproduce the oracle; with and without bias; 3-d inputs keep their leading dims."""
+    """More than 16 rows: "auto" (library workspace route), "fused" (library fused kernels) and "two_pass" / "resident"
+    (bf16 weight pass + the device library's dense GEMM) all reproduce the oracle; with and without bias; 3-d inputs keep
+    their leading dims."""
     print(f"case module gemm policies quant={quant}", flush=True)
     model, packed = _load(tmp_path, dev, quant)
     for name in ("layers.0.mlp.down_proj", "timestep_embedder"):
@@ -106,7 +107,9 @@ def test_gemm_policies_agree_with_the_oracle(tmp_path, dev, quant):
                 assert got.shape == (2, m, mod.out_features) and got.dtype == torch.bfloat16
                 assert go.rel_l2(got.cpu().reshape(2 * m, -1), want) <= TOL, (name, m, policy)
                 outs[policy] = got
-            assert torch.equal(outs["auto"], outs["two_pass"]) and torch.equal(outs["auto"], outs["resident"])
+            # "two_pass" and "resident" run the same dense GEMM on the same bf16 weight; "auto" and "fused" are the library's
+            # own kernels (another summation order), held to the oracle above
+            assert torch.equal(outs["two_pass"], outs["resident"])
         mod.gemm_policy = "sometimes"
         with pytest.raises(ValueError):
             mod(x.to(dev))

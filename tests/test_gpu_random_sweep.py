@@ -133,7 +133,7 @@ def test_random_rmsnorm_cases(dev, seed):
     for it in range(40):
         qt = rnd.choice(TYPES)
         k = 256 * rnd.randint(1, 24)
-        m = rnd.randint(1, min(16, 16384 // (2 * k + 64)))
+        m = rnd.randint(1, min(16, 36864 // (2 * k + 64)))
         n = rnd.choice([rnd.randint(1, 2500), rnd.randint(1, 2500), 6144, 33000 + rnd.randint(0, 40)])
         numerics = rnd.choice([0, 1])
         kind = rnd.choice(["linear", "gate_up", "tiled", "tiled_gate_up"])

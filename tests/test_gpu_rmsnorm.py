@@ -117,9 +117,9 @@ def test_normalized_rows_match_the_oracle_elementwise(dev):
 def test_rmsnorm_argument_errors(dev):
     packed = synthetic.make_packed(go.Q8_0, 64, 4096, seed=1).to(dev)
     gamma = _gamma(4096, 2).to(dev)
-    x = synthetic.make_activations(2, 4096, seed=3).to(dev)
-    y = torch.empty((2, 64), dtype=torch.bfloat16, device=dev)
-    assert not ops.rmsnorm_fits(go.Q8_0, 2, 4096)           # two rows of 4096 do not fit the staging area
+    x = synthetic.make_activations(5, 4096, seed=3).to(dev)
+    y = torch.empty((5, 64), dtype=torch.bfloat16, device=dev)
+    assert not ops.rmsnorm_fits(go.Q8_0, 5, 4096)           # five rows of 4096 do not fit the staging area
     assert ops.rmsnorm_fits(go.Q4_K, 1, 4096) and not ops.rmsnorm_fits(go.Q4_0, 1, 4096 + 32)
     with pytest.raises(ops.SnGgufError):
         ops.rmsnorm_linear_into(x, gamma, EPS, packed, go.Q8_0, None, y, 1)
@@ -158,7 +158,7 @@ def test_rmsnorm_tiled_parity(dev, c_oracle, shape):
     h_native = torch.empty_like(h)
     ops.rmsnorm_gate_up_silu_into(x.to(dev), gamma.to(dev), EPS, gate.to(dev), up.to(dev), go.Q8_0, h_native, 1)
     assert go.rel_l2(h.cpu(), h_native.cpu()) <= 5e-4
-    if 16 * (2 * k + 64) > 16384:      # sixteen rows of this width do not fit the staging area
+    if 16 * (2 * k + 64) > 36864:      # sixteen rows of this width do not fit the staging area
         big = synthetic.make_activations(16, k, seed=1).to(dev)
         with pytest.raises(ops.SnGgufError):
             ops.rmsnorm_linear_tiled_into(big, gamma.to(dev), EPS, tg, None, torch.empty((16, n), dtype=torch.bfloat16, device=dev), 1)
@@ -195,10 +195,39 @@ def test_module_helpers_use_the_library_norm_beyond_the_fused_row_count(dev):
     lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
     lin.weight = GGUFParameter(packed.to(dev), quant_type=go.Q8_0)
     gamma = _gamma(k, 3)
-    for m in (4, 16, 100):
+    for m in (5, 16, 100):
         x = (synthetic.make_activations(m, k, seed=m).float() * 1.7).to(torch.bfloat16)
         assert not ops.rmsnorm_fits(go.Q8_0, m, k)
         got = lin.forward_normed(x.to(dev), gamma.to(dev), EPS).cpu()
         want = go.gguf_linear_forward(go.qwen3_rms_norm(x, gamma, EPS), packed, go.Q8_0)
         assert go.rel_l2(got, want) <= TOL
         assert torch.equal(rms_norm(x.to(dev), gamma.to(dev), EPS), ops.rms_norm(x.to(dev), gamma.to(dev), EPS))
+
+
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K, go.Q6_K])
+@pytest.mark.parametrize("m", [2, 3, 4])
+def test_fused_norm_for_a_few_decode_rows_at_hidden_4096(dev, c_oracle, qt, m):
+    """Two to four decode rows at K = 4096 (the MLP configuration's M = 4): the norm rides inside the q|k|v-shaped
+    projection (block-aligned kernel), the vocabulary-sized one and the gate / up pair (line-aligned kernel for Q8_0)."""
+    print(f"case rmsnorm few rows qt={qt} m={m}", flush=True)
+    k = 4096
+    assert ops.rmsnorm_fits(qt, m, k) and not ops.rmsnorm_fits(qt, 5, k)
+    gamma = _gamma(k, 9)
+    x = (synthetic.make_activations(m, k, seed=90 + m).float() * 1.3).to(torch.bfloat16)
+    normed = go.qwen3_rms_norm(x, gamma, EPS)
+    for n in (6144, 530, 40000):
+        packed = synthetic.make_packed(qt, n, k, seed=n)
+        cols = torch.randint(0, n, (96,), generator=torch.Generator().manual_seed(n))
+        want = go.gguf_linear_forward(normed, packed[cols], qt)
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.rmsnorm_linear_into(x.to(dev), gamma.to(dev), EPS, packed.to(dev), qt, None, y, 1)
+        assert bool(torch.isfinite(y.float()).all())
+        assert go.rel_l2(y[:, cols.to(dev)].cpu(), want) <= TOL, n
+    n = 12288
+    gate, up = synthetic.make_packed(qt, n, k, seed=1, device=dev), synthetic.make_packed(qt, n, k, seed=2, device=dev)
+    cols = torch.randint(0, n, (96,), generator=torch.Generator().manual_seed(3))
+    g = go.gguf_linear_forward(normed, gate[cols.to(dev)].cpu(), qt)
+    u = go.gguf_linear_forward(normed, up[cols.to(dev)].cpu(), qt)
+    h = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.rmsnorm_gate_up_silu_into(x.to(dev), gamma.to(dev), EPS, gate, up, qt, h, 1)
+    assert go.rel_l2(h[:, cols.to(dev)].cpu(), c_oracle.silu_mul(g, u)) <= TOL
