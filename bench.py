@@ -31,7 +31,7 @@ HIDDEN, INTER, KV = 4096, 12288, 1024
 # HBM bytes per launch of the dominant kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
 # each scaled by what the same counter reads for the plain 256 MiB elementwise copy that
 # --calibrate-copy runs in the same process; None = not measured for this build.
-MEASURED_TRAFFIC = {"gemv_gate_up_m1": 107413709, "gemm_gate_m4096": 516332954}
+MEASURED_TRAFFIC = {"gemv_gate_up_m1": 107413256, "gemm_gate_m4096": 516227223, "gemm_dense_gate_m4096": 710260941}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -464,8 +464,8 @@ def main() -> None:
         _, ev_gate = run_region(gate_only, gs * 2, args.gemm_warmup)
         gate_ms = ev_gate / (gs * 2)
 
-        # the module's default for M > 16 (GGUFLinear.gemm_policy "auto"): one dequantize launch to a transient
-        # bf16 weight, then the device's dense GEMM (hipBLASLt through torch.matmul)
+        # GGUFLinear.gemm_policy "two_pass" (opt-in): one dequantize launch to a transient bf16 weight, then the
+        # device library's dense GEMM (hipBLASLt through torch.matmul); the default route is tower_ws below
         wtmp = torch.empty(INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
 
         def two_pass(x, packed, n, k, y):
@@ -486,6 +486,14 @@ def main() -> None:
         wall_ws, _ = run_region(tower_ws, gs, args.gemm_warmup)
         _, ev_gate_ws = run_region(lambda i: ops.linear_ws_into(xs[HIDDEN], tower[i % 2][4], Q8_0, None, ys[INTER], wtmp, num),
                                    gs * 2, args.gemm_warmup)
+        # the dense tile kernel alone on the gate shape: the weight pass's bf16 output kept, launched as a type-30 weight
+        gate_dense = [torch.empty((INTER, HIDDEN), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        for r in range(2):
+            ops.dequantize_into(tower[r][4], Q8_0, gate_dense[r], num)
+        _, ev_gate_dense = run_region(lambda i: ops.linear_into(xs[HIDDEN], gate_dense[i % 2].view(torch.uint8), 30, None,
+                                                                ys[INTER], num), gs * 2, args.gemm_warmup)
+        del gate_dense
+        dense_ms = ev_gate_dense / (gs * 2)
         wall2, _ = run_region(tower_two_pass, gs, args.gemm_warmup)
         _, ev_gate2 = run_region(lambda i: two_pass(xs[HIDDEN], tower[i % 2][4], INTER, HIDDEN, ys[INTER]), gs * 2, args.gemm_warmup)
         # gemm_policy "resident": the bf16 weights are produced once and kept (2 N K bytes per linear)
@@ -535,44 +543,57 @@ def main() -> None:
         wall_st, _ = run_region(tower_stacked, gs, args.gemm_warmup)
         wall_st_ws, _ = run_region(tower_stacked_ws, gs, args.gemm_warmup)
         del qkv, y_qkv
-        gate_tflops = 2.0 * m * INTER * HIDDEN / (gate_ms * 1e-3) / 1e12
+        gate_flop = 2.0 * m * INTER * HIDDEN
+        gate_tflops = gate_flop / (gate_ms * 1e-3) / 1e12
+        dense_tflops = gate_flop / (dense_ms * 1e-3) / 1e12
+        tflops_ws = flops / (wall_ws / gs * 1e-3) / 1e12
         result["gemm"] = {
             "workload": "configs[2]: Q8_0 generation-tower projections over M=4096 image tokens "
-                        "(q,o 4096^2; k,v 4096->1024; gate/up 4096->12288; down 12288->4096)",
-            "value": round(tflops, 2),
+                        "(q,o 4096^2; k,v 4096->1024; gate/up 4096->12288; down 12288->4096), seven separate linears",
+            "route": "sngguf_linear_ws (what GGUFLinear.forward does beyond 64 rows): weight pass into a pooled bf16 "
+                     "workspace + the library's dense tile kernel; k / v (64 tiles) stay on the fused tile kernel",
+            "value": round(tflops_ws, 2),
             "unit": "TFLOP/s",
             "steps": gs,
             "warmup": args.gemm_warmup,
-            "ms_per_step": round(wall / gs, 4),
+            "ms_per_step": round(wall_ws / gs, 4),
             "flop_per_step": flops,
-            "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+            "pct_of_bf16_mfma_peak": round(100 * tflops_ws / MFMA_BF16_PEAK_TFLOPS, 2),
+            "gate_us": round(ev_gate_ws / (gs * 2) * 1e3, 2),
+            "gate_tflops": round(gate_flop / (ev_gate_ws / (gs * 2) * 1e-3) / 1e12, 2),
             "roofline": {
-                "kernel": "sngguf::gemm_tile_kernel<Q8_0, upstream_fp16> (gate 4096->12288, M=4096)",
+                "kernel": "sngguf::gemm_tile_kernel<dense bf16> (gate 4096->12288, M=4096; the second launch of the route, "
+                          "timed alone on a kept bf16 weight)",
                 "bound": "mfma",
-                "achieved": round(gate_tflops, 2),
+                "achieved": round(dense_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
-                "frac": round(gate_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC["gemm_gate_m4096"],
-                "flop_per_launch": 2.0 * m * INTER * HIDDEN,
-                "avg_launch_us": round(gate_ms * 1e3, 2),
+                "frac": round(dense_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC["gemm_dense_gate_m4096"],
+                "flop_per_launch": gate_flop,
+                "avg_launch_us": round(dense_ms * 1e3, 2),
+            },
+            "fused": {
+                "what": "sngguf_linear: the Q8_0 decode inside the tile kernel (no workspace), the route of callers that "
+                        "pass none",
+                "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(wall / gs, 4),
+                "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+                "roofline": {
+                    "kernel": "sngguf::gemm_tile_kernel<Q8_0, upstream_fp16> (gate 4096->12288, M=4096)",
+                    "bound": "mfma", "achieved": round(gate_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(gate_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC["gemm_gate_m4096"],
+                    "flop_per_launch": gate_flop, "avg_launch_us": round(gate_ms * 1e3, 2),
+                },
             },
             "two_pass": {
                 "what": "same tower as sngguf dequantize (packed -> bf16, transient) + dense bf16 GEMM of the device "
-                        "library: what GGUFLinear does for M > 16 by default",
+                        "library (GGUFLinear.gemm_policy 'two_pass', opt-in)",
                 "value": round(flops / (wall2 / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
                 "ms_per_step": round(wall2 / gs, 4),
                 "pct_of_bf16_mfma_peak": round(100 * flops / (wall2 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
                 "gate_us": round(ev_gate2 / (gs * 2) * 1e3, 2),
                 "gate_tflops": round(2.0 * m * INTER * HIDDEN / (ev_gate2 / (gs * 2) * 1e-3) / 1e12, 2),
-            },
-            "workspace": {
-                "what": "sngguf_linear_ws: the same two passes inside the library (weight pass into a caller workspace + "
-                        "the library's own dense bf16 tile kernel); k / v (64 tiles) stay on the fused path",
-                "value": round(flops / (wall_ws / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(wall_ws / gs, 4),
-                "pct_of_bf16_mfma_peak": round(100 * flops / (wall_ws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
-                "gate_us": round(ev_gate_ws / (gs * 2) * 1e3, 2),
-                "gate_tflops": round(2.0 * m * INTER * HIDDEN / (ev_gate_ws / (gs * 2) * 1e-3) / 1e12, 2),
             },
             "stacked_qkv": {
                 "what": "the same tower with q, k and v as one stacked [6144, 4096] weight (one launch of 384 large tiles "
@@ -672,8 +693,9 @@ def main() -> None:
             wall, ev = run_region(ktower_step, gs, max(2, args.gemm_warmup // 2))
             flops = sum(2.0 * m * n * k for _, n, k, _ in kshapes)
             tflops = flops / (wall / gs * 1e-3) / 1e12
-            kq["tower_M4096"] = {"value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(wall / gs, 4),
-                                 "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2)}
+            kq["tower_M4096_fused"] = {"what": "sngguf_linear: Q4_K on the fused large-tile kernel, Q6_K on the 128-tile kernel",
+                                       "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(wall / gs, 4),
+                                       "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2)}
             kws = torch.empty(INTER * HIDDEN, dtype=torch.bfloat16, device=dev)
 
             def ktower_ws(i):
@@ -683,9 +705,9 @@ def main() -> None:
 
             wall_kws, _ = run_region(ktower_ws, gs, max(2, args.gemm_warmup // 2))
             tf_kws = flops / (wall_kws / gs * 1e-3) / 1e12
-            kq["tower_M4096_workspace"] = {"what": "the same tower through sngguf_linear_ws (weight pass + dense tile kernel)",
-                                           "value": round(tf_kws, 2), "unit": "TFLOP/s", "ms_per_step": round(wall_kws / gs, 4),
-                                           "pct_of_bf16_mfma_peak": round(100 * tf_kws / MFMA_BF16_PEAK_TFLOPS, 2)}
+            kq["tower_M4096"] = {"what": "sngguf_linear_ws (weight pass + dense tile kernel), the module's route beyond 64 rows",
+                                 "value": round(tf_kws, 2), "unit": "TFLOP/s", "ms_per_step": round(wall_kws / gs, 4),
+                                 "pct_of_bf16_mfma_peak": round(100 * tf_kws / MFMA_BF16_PEAK_TFLOPS, 2)}
             del kws
             del ktower, xs, ys
         kq["workload"] = ("configs[3]: Q4_K for q/k/v/o/gate/up, Q6_K for down; decode MLP at M=1,16 "
@@ -729,20 +751,23 @@ def main() -> None:
 
         wall_gws, _ = run_region(layer_ws, gs, max(2, args.gemm_warmup // 2))
         del dws
+        tflops_gws = flops / (wall_gws / gs * 1e-3) / 1e12
         result["grouped_layer"] = {
             "workload": "configs[4], one of the 36 layers: 512 text rows -> understanding weights, 4096 image rows -> "
                         "generation weights, 7 Q8_0 linears through the modality-grouped launcher (contiguous split)",
-            "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall / gs, 4),
-            "flop_per_layer": flops, "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
-            "workspace": {
-                "what": "sngguf_grouped_linear_ws: both weight sets decoded once into a caller workspace, one launch of the "
-                        "library's dense tile kernel over both row groups (k / v stay on the fused path)",
-                "value": round(flops / (wall_gws / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall_gws / gs, 4),
-                "pct_of_bf16_mfma_peak": round(100 * flops / (wall_gws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            "route": "sngguf_grouped_linear_ws (what modality.grouped_linear does with n_text): each group as its own "
+                     "workspace-route problem on its row range - K split for the 512 text rows, weight pass + dense tile "
+                     "kernel for the 4096 image rows",
+            "value": round(tflops_gws, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall_gws / gs, 4),
+            "flop_per_layer": flops, "pct_of_bf16_mfma_peak": round(100 * tflops_gws / MFMA_BF16_PEAK_TFLOPS, 2),
+            "fused": {
+                "what": "sngguf_grouped_linear: one launch of the fused tile kernel over both row groups, no workspace",
+                "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall / gs, 4),
+                "pct_of_bf16_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
             },
             "two_pass": {
-                "what": "per group: sngguf dequantize to a transient bf16 weight + dense bf16 GEMM into the group's rows "
-                        "(modality.grouped_linear with n_text, default policy)",
+                "what": "per group: sngguf dequantize to a transient bf16 weight + the device library's dense bf16 GEMM into "
+                        "the group's rows (gemm_policy 'two_pass', opt-in)",
                 "value": round(flops / (wall2 / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_layer": round(wall2 / gs, 4),
                 "pct_of_bf16_mfma_peak": round(100 * flops / (wall2 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
             },
@@ -776,10 +801,11 @@ def main() -> None:
                         "image rows -> generation weights through the modality-grouped launcher, 7 linears per layer, all "
                         "layers in one timed region (linear projections only)",
             "packed_bytes": stack_bytes, "flop_per_pass": stack_flops,
-            "value": round(stack_flops / (wall_sf / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sf / 2, 3),
-            "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sf / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
-            "workspace": {"value": round(stack_flops / (wall_sw / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sw / 2, 3),
-                          "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sw / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2)},
+            "route": "sngguf_grouped_linear_ws on one shared workspace (the host layer's default)",
+            "value": round(stack_flops / (wall_sw / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sw / 2, 3),
+            "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sw / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            "fused": {"value": round(stack_flops / (wall_sf / 2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_pass": round(wall_sf / 2, 3),
+                      "pct_of_bf16_mfma_peak": round(100 * stack_flops / (wall_sf / 2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2)},
         }
         del stack, dws, xs, ys
 

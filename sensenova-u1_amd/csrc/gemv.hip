@@ -255,22 +255,32 @@ int launch_gemv_kq_mfma(const void* x, int64_t M, const void* qa, const void* qb
 
 // Second pass of the arg-max form of the decode kernels: keys[m][slots] -> out_index[m], one workgroup per activation
 // row.  (A key orders by value first and by lower column second, see argmax_key.)
-__global__ __launch_bounds__(256) void argmax_reduce_kernel(const uint64_t* __restrict__ keys, int64_t slots, int64_t* __restrict__ out_index) {
-    __shared__ uint64_t best[256];
+__global__ __launch_bounds__(1024) void argmax_reduce_kernel(const uint64_t* __restrict__ keys, int64_t slots, int64_t* __restrict__ out_index) {
+    __shared__ uint64_t best[16];
     const uint64_t* row = keys + (int64_t)blockIdx.x * slots;
-    uint64_t k = 0;
-    for (int64_t i = threadIdx.x; i < slots; i += 256) k = u64_max(k, row[i]);
-    best[threadIdx.x] = k;
-    __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if ((int)threadIdx.x < off) best[threadIdx.x] = u64_max(best[threadIdx.x], best[threadIdx.x + off]);
-        __syncthreads();
+    // four independent loads per thread and trip: the keys were just written by the projection and sit in L2, so
+    // the pass costs a few load latencies, not one per key
+    uint64_t k0 = 0, k1 = 0, k2 = 0, k3 = 0;
+    for (int64_t i = threadIdx.x; i < slots; i += 4096) {
+        const uint64_t a = row[i];
+        const uint64_t b = i + 1024 < slots ? row[i + 1024] : 0;
+        const uint64_t c = i + 2048 < slots ? row[i + 2048] : 0;
+        const uint64_t d = i + 3072 < slots ? row[i + 3072] : 0;
+        k0 = u64_max(k0, a); k1 = u64_max(k1, b); k2 = u64_max(k2, c); k3 = u64_max(k3, d);
     }
-    if (threadIdx.x == 0) out_index[blockIdx.x] = (int64_t)(0xFFFFFFFFu - (uint32_t)best[0]);
+    uint64_t k = u64_max(u64_max(k0, k1), u64_max(k2, k3));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) k = u64_max(k, shfl_xor_u64(k, off));
+    if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++) k = u64_max(k, best[w]);
+        out_index[blockIdx.x] = (int64_t)(0xFFFFFFFFu - (uint32_t)k);
+    }
 }
 
 int launch_argmax_reduce(const uint64_t* keys, int64_t M, int64_t slots, int64_t* out_index, hipStream_t stream) {
-    argmax_reduce_kernel<<<dim3((unsigned)M), dim3(256), 0, stream>>>(keys, slots, out_index);
+    argmax_reduce_kernel<<<dim3((unsigned)M), dim3(1024), 0, stream>>>(keys, slots, out_index);
     return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
