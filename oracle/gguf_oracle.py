@@ -19,9 +19,11 @@ Two independent restatements live here:
 Pinning (see tests/test_oracle_*.py): one-hot positional blocks, scale-packing cases, the
 encode->decode round trip through the packers below (written from ggml's *quantize* side, not
 from the decoders), hand-written known-answer blocks in tests/golden, C-vs-torch bitwise
-agreement, fp16 arithmetic against numpy.  PARITY UNPINNED: which intermediates upstream
-rounds to fp16 (``dtype=None``) is taken from reading the upstream package, which is neither
-in the reference tree nor installed; no reference test or fixture covers it.
+agreement, and the fp16 chain of every type step by step against numpy float16 with an
+alternative rounding placement shown to differ (tests/test_oracle_fp16_chain.py).  PARITY
+UNPINNED: that the operation sequence restated here (``dtype=None``: every tensor op in fp16) is
+the one the upstream package executes is taken from reading that package, which is neither in
+the reference tree nor installed; no reference test or fixture covers it.
 """
 from __future__ import annotations
 

@@ -16,9 +16,12 @@
  * Pinning.  Numerics 0 is pinned by closed forms: one-hot positional blocks, scale-packing
  * cases, encode->decode round trips through independently written packers, hand-written
  * known-answer blocks and a bitwise cross-check against the vectorised restatement in
- * oracle.py.  Numerics 1 (which intermediate is rounded to fp16, and when) rests on reading
- * of the upstream package that cannot be imported here: PARITY UNPINNED for that choice; the
- * arithmetic of each rounding is pinned against numpy's float16.
+ * oracle.py.  Numerics 1 is pinned, per type, against the recorded operation sequence written out as
+ * numpy float16 operations, one rounding per tensor operation, with an alternative placement of a
+ * rounding shown to give different bits on the same blocks (tests/test_oracle_fp16_chain.py), so a
+ * moved or dropped rounding here fails.  That the recorded sequence is what the upstream package
+ * executes rests on a reading of that package, which cannot be imported here: PARITY UNPINNED for
+ * that one point (the order and kind of upstream's tensor operations), for every type.
  *
  * No dependency beyond libc; scalar loops; fp16/bf16 conversions written out by hand so that
  * they do not share code with numpy, torch or the device kernels.
