@@ -214,3 +214,71 @@ def test_random_split_k_cases(dev, seed):
                                            row_ws, ws, numerics)
             tag += f" form={form}"
         _ok(y.cpu(), want, tag)
+
+
+@pytest.mark.parametrize("seed", [51, 52])
+def test_random_bf16_static_argmax_cases(dev, seed):
+    """The later entry points over random shapes: BF16 (type 30) weights through every linear form (K of any length -
+    odd K takes the element-wise loads, K % 64 != 0 above 16 rows the chunked decode route), the allocation-free
+    sngguf_linear_static on every type, and the arg-max form of the projection against the arg-max of the library's
+    own logits (same kernels, so equal indices, ties included)."""
+    rnd = random.Random(seed)
+    for it in range(60):
+        kind = rnd.choice(["bf16_linear", "bf16_residual", "bf16_gate_up", "bf16_ws", "static", "argmax"])
+        numerics = rnd.choice([0, 1])
+        m = rnd.choice(ROWS)
+        if kind.startswith("bf16"):
+            qt = go.BF16
+            k = rnd.choice([rnd.randint(1, 3072), 8 * rnd.randint(1, 384), 64 * rnd.randint(1, 48)])
+            n = rnd.choice([rnd.randint(1, 2500), 4100, 5632])
+            if kind == "bf16_gate_up":
+                m = rnd.choice([r for r in ROWS if r <= 16])
+        elif kind == "static":
+            qt = rnd.choice(TYPES + [go.BF16])
+            bs = go.GGML_QUANT_SIZES[qt][0]
+            k = bs * rnd.randint(1, max(1, 3072 // bs)) if qt != go.BF16 else 64 * rnd.randint(1, 48)
+            n = rnd.choice([rnd.randint(1, 2500), 4100, 8200])
+        else:
+            qt = rnd.choice(TYPES)
+            m = rnd.choice([r for r in ROWS if r <= 16])
+            k = 256 * rnd.randint(1, 16)
+            n = rnd.choice([rnd.randint(1, 2500), 8200, 33000 + rnd.randint(0, 40)])
+            if qt == go.Q8_0 and rnd.random() < 0.5:
+                k = rnd.choice([2048, 4096])
+        if m * n > 6_000_000:
+            n = max(1, 6_000_000 // m)
+        use_bias = kind != "bf16_gate_up" and rnd.random() < 0.4
+        tag = f"seed={seed} it={it} kind={kind} qt={qt} m={m} n={n} k={k} numerics={numerics} bias={use_bias}"
+        print("case", tag, flush=True)
+        packed = synthetic.make_packed(qt, n, k, seed=it)
+        x = synthetic.make_activations(m, k, seed=1000 + it)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(it)) * 0.5).to(torch.bfloat16) if use_bias else None
+        xd, pd = x.to(dev), packed.to(dev)
+        bd = bias.to(dev) if bias is not None else None
+        if kind == "argmax":
+            got = ops.lm_head_argmax(xd, pd, qt, bd, numerics)
+            logits = ops.linear(xd, pd, qt, bd, numerics)
+            assert got.dtype == torch.int64 and got.shape == (m,), tag
+            assert torch.equal(got, torch.argmax(logits, dim=-1)), tag
+            _ok(logits.cpu(), go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics), tag)
+            continue
+        want = go.gguf_linear_forward(x, packed, qt, bias, numerics=numerics)
+        if kind == "bf16_linear":
+            got = ops.linear(xd, pd, qt, bd, numerics)
+        elif kind == "bf16_ws":
+            got = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            ws = torch.empty(n * k + 8, dtype=torch.bfloat16, device=dev)
+            ops.linear_ws_into(xd, pd, qt, bd, got, ws, numerics)
+        elif kind == "bf16_residual":
+            res = synthetic.make_activations(m, n, seed=5000 + it)
+            got = ops.linear_residual(xd, pd, qt, res.to(dev), bd, numerics)
+            want = (res.float() + want.float()).to(torch.bfloat16)
+        elif kind == "bf16_gate_up":
+            up = synthetic.make_packed(qt, n, k, seed=9000 + it)
+            want = torch.nn.functional.silu(want) * go.gguf_linear_forward(x, up, qt, None, numerics=numerics)
+            got = ops.gate_up_silu(xd, pd, up.to(dev), qt, numerics)
+        else:
+            assert m * n <= ops.linear_static_max_outputs(), tag
+            got = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            ops.linear_static_into(xd, pd, qt, bd, got, numerics)
+        _ok(got.cpu(), want, tag)
