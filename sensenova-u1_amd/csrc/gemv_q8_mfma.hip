@@ -245,7 +245,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K,
                                                                  const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
                                                                  const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax,
-                                                                 int gpw) {
+                                                                 int gpw, int skew) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
@@ -254,7 +254,20 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     // one staged copy of the activations); wavefronts [grp * wpg, (grp + 1) * wpg) work on row group grp of it.
     const int waves = blockDim.x >> 6;
     const int wpg = waves / gpw;
-    const int grp = wave / wpg, lw = wave - grp * wpg, wbase = grp * wpg;
+    // skew > 0 (twelve wavefronts per workgroup, two K halves of 8 steps per row group and matrix): the three
+    // wavefronts that share a SIMD are served oldest first, so the first-placed ones run ahead of the last-placed ones
+    // for the whole kernel.  Each K range is therefore shared by a first-placed wavefront (wave 0..3), which takes
+    // 8 + skew steps, and a last-placed one (wave 8..11), which takes 8 - skew; the middle four pair up 8 + 8.
+    // lwave is the wavefront's place in the [group][matrix][K half] order the reduction below uses.
+    int lwave = wave, skew_lo = 0;
+    if (skew > 0) {
+        const int slot = wave >> 2, i = wave & 3;
+        const int pair = slot == 1 ? 4 + (i >> 1) : i;
+        const int khalf = slot == 1 ? (i & 1) : (slot >> 1);
+        lwave = 2 * pair + khalf;
+        skew_lo = slot == 1 ? 0 : skew;
+    }
+    const int grp = lwave / wpg, lw = lwave - grp * wpg, wbase = grp * wpg;
     const int W = (GATED && !PAIRED) ? wpg >> 1 : wpg;
     const int kw = (GATED && !PAIRED) ? (lw >= W ? lw - W : lw) : lw;
     const uint8_t* __restrict__ q = (GATED && !PAIRED && lw >= W) ? qb : qa;
@@ -264,6 +277,13 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     const bool live = n0 < N;            // the last workgroup's row groups may lie past the end: those wavefronts idle
     const int spans = (int)(K >> 11);
     const int t0 = live ? (int)((int64_t)kw * spans / W) : 0, t1 = live ? (int)((int64_t)(kw + 1) * spans / W) : 0;
+    // this wavefront's steps [gs0, gs1) of the row's 8 * spans (whole spans unless skewed)
+    int gs0 = 8 * t0, gs1 = 8 * t1;
+    if (skew_lo > 0 && live) {
+        if (kw == 0) gs1 += skew_lo;
+        else gs0 += skew_lo;
+    }
+    const int tf = gs0 >> 3, s_first = gs0 & 7;   // a range that starts inside a span starts at one of its steps 1..6
 
     // Two-line fetch: piece lane + 64 i is bytes [16 c, +16) of the 256-byte window of row
     // (lane / 16) + 4 i, c = lane % 16.  One-line fetch: row (lane / 8) + 8 i, piece lane % 8.
@@ -330,9 +350,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 
     if constexpr (XLDS) {
         // weights of the first step are requested before the activations are staged
-        if (t0 < t1) {
-            fetch2(t0, 0, pa);
-            fetch2(t0, 1, pb);
+        if (gs0 < gs1) {
+            fetch2(tf, s_first, pa);
+            fetch2(tf, s_first + 1, pb);
         }
         const int pieces_per_row = (int)(K >> 3);  // 16-byte pieces
         if (gamma == nullptr) {
@@ -367,20 +387,23 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
             }
         }
         __syncthreads();
-    } else if (t0 < t1) {
-        fetch_x(t0, 0, xa);
-        fetch2(t0, 0, pa);
-        fetch2(t0, 1, pb);
+    } else if (gs0 < gs1) {
+        fetch_x(tf, 0, xa);      // (ranges of whole spans only: see the launcher)
+        fetch2(tf, 0, pa);
+        fetch2(tf, 1, pb);
     }
-    for (int t = t0; t < t1; t++) {
+    for (int t = tf; 8 * t < gs1; t++) {
 #pragma unroll
         for (int s = 0; s < 8; s++) {
+            const int gs = 8 * t + s;
+            if (gs < gs0 || gs >= gs1) continue;
+            const bool more = gs + 1 < gs1;   // the step after this one is still this wavefront's
             u32x4_t (&xc)[8] = (s & 1) ? xb : xa;
             u32x4_t (&xn)[8] = (s & 1) ? xa : xb;
-            // -- lines fetched during the previous step go into the ring
-            if (s == 0) {
-                store2(0, pa);
-                store2(1, pb);
+            // -- lines fetched during the previous step go into the ring (a range's first step: both line pairs)
+            if (s == 0 || (s < 7 && gs == gs0)) {
+                store2(s, pa);
+                store2(s + 1, pb);
             } else if (s < 7) {
                 store2(s + 1, pa);
             } else {
@@ -391,7 +414,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
             }
             // -- requests for the next step: activations first, so that waiting for them does not
             //    also wait for the weight lines
-            if (s < 7) {
+            if (!more) {
+            } else if (s < 7) {
                 fetch_x(t, s + 1, xn);
                 if (s < 6) {
                     fetch2(t, s + 2, pa);
@@ -402,7 +426,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                         for (int i = 0; i < 2; i++)
                             pa[h][i] = *reinterpret_cast<const u32x4_t*>((h ? base2 : base) + (int64_t)t * kSpanBytes + goff1[i]);
                 }
-            } else if (t + 1 < t1) {
+            } else {
                 fetch_x(t + 1, 0, xn);
                 fetch2(t + 1, 0, pa);
                 fetch2(t + 1, 1, pb);
@@ -456,8 +480,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     // per row group: [gate partial sums of the W K ranges | up partial sums][64]; the paired mode keeps the up sums of
     // all wavefronts behind the gate sums of all wavefronts
     f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);
-    red[wave * 64 + lane] = acc[0];
-    if constexpr (PAIRED) red[(waves + wave) * 64 + lane] = acc[NQ - 1];
+    red[lwave * 64 + lane] = acc[0];
+    if constexpr (PAIRED) red[(waves + lwave) * 64 + lane] = acc[NQ - 1];
     __syncthreads();
     if (lw != 0 || !has_x || !live) return;
     f32x4_t sum = red[wbase * 64 + lane];
@@ -538,6 +562,11 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
     const size_t lds_bytes = lds_for(gpw);
     if (lds_bytes > 160 * 1024) return SNGGUF_E_BADSHAPE;
     const dim3 grid((unsigned)((groups + gpw - 1) / gpw)), block((unsigned)(64 * waves));
+    // one extra step for the first-placed wavefront of each K range, one less for the last-placed (12288 x 4096 gate/up at
+    // M = 1, extra steps 0 / 1 / 2 / 3: 24.5 / 23.9 / 24.3 / 24.4 us; per-wavefront loop ends by placement 16.8 / 17.7 / 19.6 us
+    // unskewed, 18.4 / 18.4 / 19.6 us with one step moved)
+    constexpr int kSkewSteps = 1;
+    const int skew = (xlds && waves == 12 && spans == 2 && w == 2) ? kSkewSteps : 0;
     // the rings of a dozen wavefronts plus staged activations exceed the default dynamic-LDS limit: raise it once per
     // kernel instance
 #define SNGGUF_LAUNCH_ONE(G, WM, XL, PR) \
@@ -546,7 +575,7 @@ static int launch_span(const bf16_t* x, int M, const uint8_t* qa, const uint8_t*
             reinterpret_cast<const void*>(&gemv_q8_span_kernel<NUM, G, WM, XL, PR>), \
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH; \
-        gemv_q8_span_kernel<NUM, G, WM, XL, PR><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax, gpw); \
+        gemv_q8_span_kernel<NUM, G, WM, XL, PR><<<grid, block, lds_bytes, stream>>>(x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax, gpw, skew); \
     } while (0)
 #define SNGGUF_LAUNCH(G, XL, PR) \
     do { \
