@@ -258,7 +258,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     // wavefronts that share a SIMD are served oldest first, so the first-placed ones run ahead of the last-placed ones
     // for the whole kernel.  Each K range is therefore shared by a first-placed wavefront (wave 0..3), which takes
     // 8 + skew steps, and a last-placed one (wave 8..11), which takes 8 - skew; the middle four pair up 8 + 8.
-    // lwave is the wavefront's place in the [group][matrix][K half] order the reduction below uses.
+    // The first-placed wavefront takes its extra steps - the first `skew` steps of the other one's span - BEFORE its
+    // own span, so that the lines the two share are requested by both at the start of the kernel and come from
+    // memory once.  lwave is the wavefront's place in the [group][matrix][K half] order the reduction below uses.
     int lwave = wave, skew_lo = 0;
     if (skew > 0) {
         const int slot = wave >> 2, i = wave & 3;
@@ -277,10 +279,12 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     const bool live = n0 < N;            // the last workgroup's row groups may lie past the end: those wavefronts idle
     const int spans = (int)(K >> 11);
     const int t0 = live ? (int)((int64_t)kw * spans / W) : 0, t1 = live ? (int)((int64_t)(kw + 1) * spans / W) : 0;
-    // this wavefront's steps [gs0, gs1) of the row's 8 * spans (whole spans unless skewed)
-    int gs0 = 8 * t0, gs1 = 8 * t1;
+    // this wavefront's steps: an optional pre-segment, steps [0, npre) of span tpre, then steps [gs0, gs1) of the row's
+    // 8 * spans (whole spans unless skewed)
+    int gs0 = 8 * t0, gs1 = 8 * t1, npre = 0;
+    const int tpre = t1;
     if (skew_lo > 0 && live) {
-        if (kw == 0) gs1 += skew_lo;
+        if (kw == 0) npre = skew_lo;
         else gs0 += skew_lo;
     }
     const int tf = gs0 >> 3, s_first = gs0 & 7;   // a range that starts inside a span starts at one of its steps 1..6
@@ -350,7 +354,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 
     if constexpr (XLDS) {
         // weights of the first step are requested before the activations are staged
-        if (gs0 < gs1) {
+        if (npre > 0) {
+            fetch2(tpre, 0, pa);
+            fetch2(tpre, 1, pb);
+        } else if (gs0 < gs1) {
             fetch2(tf, s_first, pa);
             fetch2(tf, s_first + 1, pb);
         }
@@ -392,16 +399,22 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         fetch2(tf, 0, pa);
         fetch2(tf, 1, pb);
     }
-    for (int t = tf; 8 * t < gs1; t++) {
+    const int nit = (npre > 0 ? 1 : 0) + (gs0 < gs1 ? ((gs1 - 1) >> 3) - tf + 1 : 0);
+    for (int it = 0; it < nit; it++) {
+        const bool in_pre = npre > 0 && it == 0;
+        const int t = in_pre ? tpre : tf + it - (npre > 0 ? 1 : 0);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             const int gs = 8 * t + s;
-            if (gs < gs0 || gs >= gs1) continue;
-            const bool more = gs + 1 < gs1;   // the step after this one is still this wavefront's
+            if (in_pre ? s >= npre : (gs < gs0 || gs >= gs1)) continue;
+            // the step after this one: in the same span, in the next segment (which starts at a span's step 0), or none
+            const bool more_here = in_pre ? s + 1 < npre : (s < 7 && gs + 1 < gs1);
+            const bool more = more_here || (in_pre ? gs0 < gs1 : gs + 1 < gs1);
+            const int tn = in_pre ? tf : t + 1;
             u32x4_t (&xc)[8] = (s & 1) ? xb : xa;
             u32x4_t (&xn)[8] = (s & 1) ? xa : xb;
-            // -- lines fetched during the previous step go into the ring (a range's first step: both line pairs)
-            if (s == 0 || (s < 7 && gs == gs0)) {
+            // -- lines fetched during the previous step go into the ring (a segment's first step: both line pairs)
+            if (s == 0 || (s < 7 && !in_pre && gs == gs0)) {
                 store2(s, pa);
                 store2(s + 1, pb);
             } else if (s < 7) {
@@ -415,7 +428,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
             // -- requests for the next step: activations first, so that waiting for them does not
             //    also wait for the weight lines
             if (!more) {
-            } else if (s < 7) {
+            } else if (more_here) {
                 fetch_x(t, s + 1, xn);
                 if (s < 6) {
                     fetch2(t, s + 2, pa);
@@ -427,9 +440,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
                             pa[h][i] = *reinterpret_cast<const u32x4_t*>((h ? base2 : base) + (int64_t)t * kSpanBytes + goff1[i]);
                 }
             } else {
-                fetch_x(t + 1, 0, xn);
-                fetch2(t + 1, 0, pa);
-                fetch2(t + 1, 1, pb);
+                fetch_x(tn, 0, xn);
+                fetch2(tn, 0, pa);
+                fetch2(tn, 1, pb);
             }
             // -- decode and contract the 8 blocks of this step
 #pragma unroll
