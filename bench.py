@@ -267,7 +267,34 @@ def main() -> None:
                             "GGUFLinear.forward calls (gate, up, down: three decode launches), torch SiLU and product "
                             "(two elementwise launches); same algorithmic bytes as the headline step")
         result["mlp_unfused_dropin"] = drop
-        del mods
+
+        # the same modules inside a Qwen3MLP-shaped nn.Module whose forward the one-call loader has pointed at the fused
+        # gated MLP (modality.fuse_gated_mlps): Module.__call__ -> gated_mlp -> sngguf_gate_up_silu + sngguf_linear
+        from sensenova_u1_amd import fuse_gated_mlps
+
+        class GatedMLP(torch.nn.Module):
+            def __init__(self, g, u, d):
+                super().__init__()
+                self.gate_proj, self.up_proj, self.down_proj, self.act_fn = g, u, d, torch.nn.SiLU()
+
+            def forward(self, x):
+                return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+        mlps = [GatedMLP(*t) for t in mods]
+        n_fused = sum(fuse_gated_mlps(mm) for mm in mlps)
+        fusedleg = {}
+        for m in (1, 4, 16):
+            xm = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
+            kd = K if m == 1 else max(64, K // 4)
+            wall_f, _ = run_region(lambda i: mlps[i % L](xm), kd, min(W, 16))
+            gb = mlp_bytes(m) / (wall_f / kd * 1e-3) / 1e9
+            fusedleg[f"M{m}"] = {"value": round(gb, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gb / HBM_PEAK_GBPS, 2),
+                                 "ms_per_step": round(wall_f / kd, 6)}
+        fusedleg["workload"] = (f"the headline MLP through Module.forward of {n_fused} Qwen3MLP-shaped modules as "
+                                "load_gguf_model leaves them (forward pointed at the fused gated MLP; output tensors "
+                                "allocated per call by torch's caching allocator)")
+        result["mlp_loader_fused_module"] = fusedleg
+        del mods, mlps
 
     # ---- the same MLP on the opt-in operand-order ("tiled") copy of the weights (made once at load time) ------------
     if not args.no_extra:

@@ -170,7 +170,7 @@ def count_gguf_linear(model: nn.Module) -> int:
 
 
 def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.dtype,
-                    device: str | torch.device | None, model_factory=None) -> nn.Module:
+                    device: str | torch.device | None, model_factory=None, fuse_mlp: bool = True) -> nn.Module:
     """The whole GGUF branch of the reference's model loader in one call
     (``_load_from_gguf``, ``src/sensenova_u1/utils/checkpoint_loading.py:288-323``): build the model without
     storage, parse the file, swap the quantized linears in and place the tensors on ``device``, report how many
@@ -180,6 +180,10 @@ def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.
     ``config_or_meta_model`` is either a model that already lives on the meta device, or a config: then
     ``model_factory(config)`` is called under ``torch.device("meta")``, and without a factory the reference's own
     construction is used (``transformers.AutoModel.from_config`` under ``accelerate.init_empty_weights``).
+
+    ``fuse_mlp`` (an addition to the reference's behaviour, on by default): the SiLU-gated MLPs whose three
+    projections became ``GGUFLinear`` get ``modality.fuse_gated_mlps``'s forward, i.e. gate, up and the SiLU product in
+    one launch at decode row counts; the results keep every rounding of the three module calls.
     """
     print(f"[gguf] loading quantized checkpoint from {gguf_checkpoint}")
     if isinstance(config_or_meta_model, nn.Module):
@@ -209,6 +213,10 @@ def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.
     print(f"[gguf] {n_gguf_linear} GGUFLinear modules active (HIP dequant-GEMV / dequant-GEMM at forward time)")
     if n_gguf_linear == 0:
         print("[gguf] WARNING: no GGUFLinear modules found — no Linear of the model has a quantized weight in the file")
+    if fuse_mlp and n_gguf_linear:
+        from .modality import fuse_gated_mlps
+
+        print(f"[gguf] {fuse_gated_mlps(model)} gated MLP modules run gate / up / SiLU as one launch at decode")
 
     del state_dict
     gc.collect()

@@ -180,3 +180,63 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     else:
         h = torch.nn.functional.silu(gate_proj(x)) * up_proj(x)
     return down_proj(h)
+
+
+def _is_silu(fn) -> bool:
+    """Whether ``fn`` computes SiLU (``ACT2FN["silu"]`` is an ``nn.SiLU`` or a class of its own, depending on the
+    transformers version): decided on three values, bit for bit."""
+    if not callable(fn):
+        return False
+    probe = torch.tensor([-1.5, 0.0, 2.25], dtype=torch.float32)
+    try:
+        return bool(torch.equal(fn(probe), torch.nn.functional.silu(probe)))
+    except Exception:
+        return False
+
+
+def _fused_mlp_forward(self, x):
+    return gated_mlp(x, self.gate_proj, self.up_proj, self.down_proj)
+
+
+def fuse_gated_mlps(model: nn.Module) -> int:
+    """Point the forward of every SiLU-gated MLP of ``model`` at ``gated_mlp``; returns how many were found.
+
+    A module qualifies when it looks like ``Qwen3MLP`` (``modeling_qwen3.py:203-216``; the generation tower's
+    ``mlp_mot_gen`` is the same class): children ``gate_proj``, ``up_proj``, ``down_proj`` that are all ``GGUFLinear``,
+    an ``act_fn`` that computes SiLU, and a forward of one argument.  Its forward then is
+    ``down_proj(silu(gate_proj(x)) * up_proj(x))`` with the gate / up pair and the SiLU product in one launch at decode
+    row counts, every rounding of the three-launch form kept, and the unchanged three module calls beyond 16 rows.  The
+    original forward is kept and ``unfuse_gated_mlps`` puts it back."""
+    import inspect
+    import types
+
+    n = 0
+    for m in model.modules():
+        if "_sn_unfused_forward" in m.__dict__:
+            n += 1
+            continue
+        projs = [getattr(m, name, None) for name in ("gate_proj", "up_proj", "down_proj")]
+        if not all(isinstance(p, GGUFLinear) for p in projs) or not _is_silu(getattr(m, "act_fn", None)):
+            continue
+        try:
+            params = [p for p in inspect.signature(m.forward).parameters.values()
+                      if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)]
+        except (TypeError, ValueError):
+            continue
+        if len(params) != 1:
+            continue
+        m.__dict__["_sn_unfused_forward"] = m.forward
+        m.forward = types.MethodType(_fused_mlp_forward, m)
+        n += 1
+    return n
+
+
+def unfuse_gated_mlps(model: nn.Module) -> int:
+    """Undo ``fuse_gated_mlps``; returns how many modules got their own forward back."""
+    n = 0
+    for m in model.modules():
+        if "_sn_unfused_forward" in m.__dict__:
+            del m.__dict__["_sn_unfused_forward"]
+            m.__dict__.pop("forward", None)   # the class's forward shows through again
+            n += 1
+    return n

@@ -391,3 +391,53 @@ def test_module_paths_refuse_host_tensors_and_wrong_widths(dev):
     with pytest.raises(ops.SnGgufError):
         lin.forward_residual(synthetic.make_activations(2, k).to(dev), synthetic.make_activations(2, n))   # residual on the host
     torch.cuda.synchronize()
+
+
+def test_loader_fused_mlp_forward_matches_the_three_module_calls(tmp_path, dev):
+    """A Qwen3MLP-shaped module loaded through load_gguf_model runs gate / up / SiLU as one launch at decode row counts:
+    its output holds the tolerance against the oracle and against its own unfused forward, at 1, 4 and 16 rows; beyond
+    16 rows the fused forward IS the three module calls (bit-equal); a captured graph of the fused forward replays."""
+    from sensenova_u1_amd import load_gguf_model, unfuse_gated_mlps
+    from sensenova_u1_amd.gguf_file import write_gguf
+    from tests.test_loader import _GatedMLP
+    print("case loader-fused mlp", flush=True)
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.mlp = _GatedMLP()
+
+    torch.manual_seed(3)
+    ref = Wrap()
+    packed = {n: go.quantize_q8_0(t.detach().numpy()) for n, t in ref.state_dict().items()}
+    path = str(tmp_path / "w.gguf")
+    write_gguf(path, [(n, p, 8) for n, p in packed.items()])
+    with torch.device("meta"):
+        meta = Wrap()
+    model = load_gguf_model(meta, path, dtype=torch.bfloat16, device=dev)
+    outs = {}
+    for m in (1, 4, 16, 40):
+        x = (torch.randn(m, H, generator=torch.Generator().manual_seed(m)) * 0.7).to(torch.bfloat16)
+        outs[m] = model.mlp(x.to(dev))
+        g = go.gguf_linear_forward(x, torch.from_numpy(packed["mlp.gate_proj.weight"]), go.Q8_0)
+        u = go.gguf_linear_forward(x, torch.from_numpy(packed["mlp.up_proj.weight"]), go.Q8_0)
+        want = go.gguf_linear_forward(torch.nn.functional.silu(g) * u, torch.from_numpy(packed["mlp.down_proj.weight"]), go.Q8_0)
+        assert go.rel_l2(outs[m].cpu(), want) <= 1e-3, m
+    xg = (torch.randn(2, H, generator=torch.Generator().manual_seed(9)) * 0.7).to(torch.bfloat16).to(dev)
+    eager = model.mlp(xg)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        yg = model.mlp(xg)
+    for _ in range(3):
+        yg.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yg, eager)
+    assert unfuse_gated_mlps(model) == 1
+    for m in (1, 4, 16, 40):
+        x = (torch.randn(m, H, generator=torch.Generator().manual_seed(m)) * 0.7).to(torch.bfloat16)
+        plain = model.mlp(x.to(dev))
+        if m > 16:
+            assert torch.equal(plain, outs[m])
+        else:
+            assert go.rel_l2(outs[m].cpu(), plain.cpu()) <= 1e-3, m

@@ -320,3 +320,62 @@ def test_module_with_host_weight_raises_before_any_launch(rows):
         lin(torch.zeros(rows, 256, dtype=torch.bfloat16))
     with pytest.raises(ops.SnGgufError):
         lin._checked_rows(torch.zeros(rows, 256, dtype=torch.bfloat16), torch.ones(256, dtype=torch.bfloat16))
+
+
+class _GatedMLP(nn.Module):
+    """The shape of the reference's Qwen3MLP (modeling_qwen3.py:203-216)."""
+
+    def __init__(self, act=None):
+        super().__init__()
+        self.gate_proj = nn.Linear(H, I, bias=False)
+        self.up_proj = nn.Linear(H, I, bias=False)
+        self.down_proj = nn.Linear(I, H, bias=False)
+        self.act_fn = act if act is not None else nn.SiLU()
+
+    def forward(self, x):
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+
+class _TwoArgMLP(_GatedMLP):
+    def forward(self, x, scale):
+        return super().forward(x) * scale
+
+
+class _MLPModel(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a = _GatedMLP()
+        self.b = _GatedMLP(act=nn.GELU())
+        self.c = _TwoArgMLP()
+        self.d = _GatedMLP(act=torch.nn.functional.silu)
+
+
+def test_gated_mlps_are_fused_by_the_one_call_loader(tmp_path, capsys):
+    """load_gguf_model points the forward of Qwen3MLP-shaped modules (three GGUFLinear projections, a SiLU act_fn, a
+    forward of one argument) at the fused gated MLP; other activations and other signatures keep their own forward;
+    fuse_mlp=False and unfuse_gated_mlps leave / restore the class's forward."""
+    from sensenova_u1_amd import fuse_gated_mlps, load_gguf_model, modality, unfuse_gated_mlps
+    torch.manual_seed(1)
+    ref = _MLPModel()
+    tensors = [(n, go.quantize_q8_0(t.detach().numpy()), int(GGMLQuantizationType.Q8_0)) for n, t in ref.state_dict().items()]
+    path = str(tmp_path / "mlp.gguf")
+    write_gguf(path, tensors)
+
+    def fused(m):
+        return getattr(m.forward, "__func__", None) is modality._fused_mlp_forward
+
+    with torch.device("meta"):
+        meta = _MLPModel()
+    model = load_gguf_model(meta, path, dtype=torch.bfloat16, device="cpu")
+    out = capsys.readouterr().out
+    assert "[gguf] 12 GGUFLinear modules active" in out
+    assert "[gguf] 2 gated MLP modules run gate / up / SiLU as one launch at decode" in out
+    assert fused(model.a) and fused(model.d) and not fused(model.b) and not fused(model.c)
+    assert fuse_gated_mlps(model) == 2                     # idempotent
+    assert unfuse_gated_mlps(model) == 2
+    assert not fused(model.a) and model.a.forward.__func__ is _GatedMLP.forward
+    with torch.device("meta"):
+        meta2 = _MLPModel()
+    model2 = load_gguf_model(meta2, path, dtype=torch.bfloat16, device="cpu", fuse_mlp=False)
+    assert "gated MLP modules" not in capsys.readouterr().out
+    assert not fused(model2.a) and not fused(model2.d)
