@@ -419,9 +419,52 @@ def main() -> None:
             wall_l, _ = run_region(fn, k3, min(W, 16))
             legs[name] = {"launches": launches, "us_per_layer": round(wall_l / k3 * 1e3, 2),
                           "value": round(lbytes / (wall_l / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"}
+        # the same seven linears and two adds as nn.Modules with the reference's call pattern (q_proj(x), k_proj(x), v_proj(x),
+        # residual + o_proj(.), residual + mlp(.) with Qwen3MLP's forward): as set_gguf2meta_model leaves them, and as
+        # load_gguf_model leaves them (q / k / v on one stacked weight tensor, the MLP's forward pointed at the fused one)
+        from sensenova_u1_amd import GGUFLinear, GGUFParameter, fuse_gated_mlps, stack_shared_input_projections
+
+        def qlin(packed, n, k):
+            lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+            lin.weight = GGUFParameter(packed, quant_type=Q8_0)
+            lin.numerics = num
+            return lin
+
+        class MLP(torch.nn.Module):
+            def __init__(self, g, u, d):
+                super().__init__()
+                self.gate_proj, self.up_proj, self.down_proj = qlin(g, INTER, HIDDEN), qlin(u, INTER, HIDDEN), qlin(d, HIDDEN, INTER)
+                self.act_fn = torch.nn.SiLU()
+
+            def forward(self, x):
+                return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+        class Layer(torch.nn.Module):
+            def __init__(self, a, mlp):
+                super().__init__()
+                self.q_proj, self.k_proj, self.v_proj = qlin(a[0], HIDDEN, HIDDEN), qlin(a[1], KV, HIDDEN), qlin(a[2], KV, HIDDEN)
+                self.o_proj, self.mlp = qlin(a[3], HIDDEN, HIDDEN), MLP(*mlp)
+
+            def forward(self, x):
+                q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+                h = x + self.o_proj(q)
+                return h + self.mlp(h), k, v
+
+        for leg, prepare in (("modules_swapped_only", None), ("modules_as_loaded", True)):
+            mods_l = [Layer(attn[i], layers[i]) for i in range(nl)]   # (the second pass re-lays q / k / v into one tensor)
+            if prepare:
+                for ml in mods_l:
+                    stack_shared_input_projections(ml)
+                    fuse_gated_mlps(ml)
+            wall_l, _ = run_region(lambda i: mods_l[i % nl](x1), k3, min(W, 16))
+            legs[leg] = {"launches": "7 linears + SiLU, product, 2 adds through Module.forward" if not prepare else
+                         "q|k|v in one launch (SharedInputStack), o, fused gate/up/SiLU, down, 2 adds through Module.forward",
+                         "us_per_layer": round(wall_l / k3 * 1e3, 2), "value": round(lbytes / (wall_l / k3 * 1e-3) / 1e9, 1), "unit": "GB/s"}
+            del mods_l
         result["decode_layer"] = {
             "workload": "the 7 Q8_0 linears of one decoder layer at M=1 (q,o 4096^2; k,v 4096->1024; gate/up fused with SiLU; "
-                        "down) and its two residual adds; no attention; the with_norms legs add the layer's two RMSNorms",
+                        "down) and its two residual adds; no attention; the with_norms legs add the layer's two RMSNorms; the "
+                        "modules_* legs run the reference's call pattern through nn.Module forwards",
             "bytes_per_layer": lbytes, **legs,
         }
         del attn, qkv, t_mlp, t_qkv, t_o

@@ -170,7 +170,8 @@ def count_gguf_linear(model: nn.Module) -> int:
 
 
 def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.dtype,
-                    device: str | torch.device | None, model_factory=None, fuse_mlp: bool = True) -> nn.Module:
+                    device: str | torch.device | None, model_factory=None, fuse_mlp: bool = True,
+                    stack_qkv: bool = True) -> nn.Module:
     """The whole GGUF branch of the reference's model loader in one call
     (``_load_from_gguf``, ``src/sensenova_u1/utils/checkpoint_loading.py:288-323``): build the model without
     storage, parse the file, swap the quantized linears in and place the tensors on ``device``, report how many
@@ -184,6 +185,8 @@ def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.
     ``fuse_mlp`` (an addition to the reference's behaviour, on by default): the SiLU-gated MLPs whose three
     projections became ``GGUFLinear`` get ``modality.fuse_gated_mlps``'s forward, i.e. gate, up and the SiLU product in
     one launch at decode row counts; the results keep every rounding of the three module calls.
+    ``stack_qkv`` (likewise, when the model lands on a HIP device): ``q_proj`` / ``k_proj`` / ``v_proj`` of every
+    attention module share one weight tensor (``modality.SharedInputStack``) and one decode launch.
     """
     print(f"[gguf] loading quantized checkpoint from {gguf_checkpoint}")
     if isinstance(config_or_meta_model, nn.Module):
@@ -217,6 +220,10 @@ def load_gguf_model(config_or_meta_model, gguf_checkpoint: str, *, dtype: torch.
         from .modality import fuse_gated_mlps
 
         print(f"[gguf] {fuse_gated_mlps(model)} gated MLP modules run gate / up / SiLU as one launch at decode")
+    if stack_qkv and n_gguf_linear and target_device is not None and torch.device(target_device).type == "cuda":
+        from .modality import stack_shared_input_projections
+
+        print(f"[gguf] {stack_shared_input_projections(model)} q / k / v groups share one weight tensor and one decode launch")
 
     del state_dict
     gc.collect()

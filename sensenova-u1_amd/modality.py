@@ -240,3 +240,110 @@ def unfuse_gated_mlps(model: nn.Module) -> int:
             m.__dict__.pop("forward", None)   # the class's forward shows through again
             n += 1
     return n
+
+
+class SharedInputStack:
+    """Projections that the model calls one after the other on the same tensor (``q_proj``, ``k_proj``, ``v_proj``:
+    ``modeling_qwen3.py:444,450,456`` and the ``_mot_gen`` triple at ``:602,608,614``), with their packed rows stored one
+    after another in ONE device tensor and every module's ``weight.data`` a view of its rows.
+
+    The modules stay separate ``GGUFLinear`` objects and the model code stays as it is.  At decode row counts the first
+    member's forward runs one launch over all rows - packed GGUF rows are independent, so the stacked rows are a valid
+    weight of ``sum(out_features)`` rows - and keeps the result; the following members, called with the same tensor
+    (same storage, shape, strides and version counter), return their columns of it.  Anything else - another input,
+    more than 16 rows, a weight that no longer lies where the stack put it (``.to()``, an offloader's rebinding) -
+    falls back to the member's own launch, so the stack never changes what a call returns, only how many launches
+    a decode step needs (three -> one: the 4096 -> 1024 k / v launches cost more in launch overhead than in bytes).
+    Outputs of one step are column ranges of one buffer: disjoint, but not separately allocated."""
+
+    def __init__(self, members) -> None:
+        members = list(members)
+        first = members[0]
+        for mod in members:
+            if not isinstance(mod, GGUFLinear):
+                raise TypeError(f"SharedInputStack needs GGUFLinear modules, got {type(mod).__name__}")
+            if mod.in_features != first.in_features or int(mod.weight.quant_type) != int(first.weight.quant_type):
+                raise ValueError("stacked projections must share in_features and quant type")
+            if mod.bias is not None or mod.numerics != first.numerics or mod.compute_dtype != first.compute_dtype:
+                raise ValueError("stacked projections must have no bias and agree on numerics and compute dtype")
+            if not mod.weight.is_cuda or mod.weight.device != first.weight.device:
+                raise ValueError("stacked projections must live on one HIP device")
+        self.members = members
+        self.index = {id(mod): i for i, mod in enumerate(members)}
+        self.splits = [mod.out_features for mod in members]
+        self.offsets = [sum(self.splits[:i]) for i in range(len(members))]
+        self.row_bytes = first.weight.as_tensor().reshape(first.out_features, -1).shape[1]
+        if any((off * self.row_bytes) % 16 for off in self.offsets):
+            raise ValueError("a member's rows would not start 16-byte aligned inside the stack")
+        self.stacked = torch.cat([mod.weight.as_tensor().reshape(mod.out_features, -1) for mod in members], dim=0)
+        for mod, off in zip(members, self.offsets):
+            mod.weight.data = self.stacked[off:off + mod.out_features]
+            mod.weights_changed()
+            mod.__dict__["_shared_stack"] = self
+        self._pending = None
+
+    def intact(self) -> bool:
+        base = self.stacked.data_ptr()
+        first = self.members[0]
+        for mod, off in zip(self.members, self.offsets):
+            w = mod.weight
+            if (w.data_ptr() != base + off * self.row_bytes or w.device != self.stacked.device or mod.decode_layout != "native"
+                    or mod.numerics != first.numerics or int(w.quant_type) != int(first.weight.quant_type) or mod.bias is not None):
+                return False
+        return True
+
+    def member_forward(self, mod: GGUFLinear, x: torch.Tensor) -> Optional[torch.Tensor]:
+        """The member's output if the stack can supply it, else None (the member then runs its own launch)."""
+        i = self.index[id(mod)]
+        rows = x.numel() // mod.in_features if x.numel() else 0
+        if not (0 < rows <= 16 and x.is_cuda and x.dtype == torch.bfloat16):
+            if i == 0:
+                self._pending = None
+            return None
+        key = (x.data_ptr(), x._version, tuple(x.shape), tuple(x.stride()))
+        if i == 0:
+            self._pending = None
+            if len(self.members) == 1 or not self.intact():
+                return None
+            first = self.members[0]
+            y = ops.linear(x, self.stacked, int(first.weight.quant_type), None, first.numerics)
+            self._pending = (key, y)
+            return y[..., :self.splits[0]]
+        pending = self._pending
+        if pending is None or pending[0] != key:
+            return None
+        if i == len(self.members) - 1:
+            self._pending = None
+        return pending[1][..., self.offsets[i]:self.offsets[i] + self.splits[i]]
+
+    def dissolve(self) -> None:
+        """Give every member its own storage back (a copy of its rows) and detach it from the stack."""
+        for mod, off in zip(self.members, self.offsets):
+            if mod.__dict__.get("_shared_stack") is self:
+                del mod.__dict__["_shared_stack"]
+                mod.weight.data = mod.weight.data.clone()
+                mod.weights_changed()
+        self._pending = None
+
+
+def stack_shared_input_projections(model: nn.Module, names=("q_proj", "k_proj", "v_proj")) -> int:
+    """Build a ``SharedInputStack`` for every module of ``model`` that owns the projections ``names`` (and for their
+    ``_mot_gen`` twins) as ``GGUFLinear`` modules on a HIP device with one quant type, no bias and the native decode
+    layout; returns how many stacks were built.  Groups that do not qualify are left alone."""
+    n = 0
+    for parent in model.modules():
+        for suffix in ("", MOT_GEN_SUFFIX):
+            members = [getattr(parent, name + suffix, None) for name in names]
+            if not all(isinstance(m, GGUFLinear) for m in members):
+                continue
+            if any("_shared_stack" in m.__dict__ for m in members):
+                n += all(m.__dict__.get("_shared_stack") is members[0].__dict__.get("_shared_stack") for m in members)
+                continue
+            try:
+                if any(m.decode_layout != "native" for m in members):
+                    continue
+                SharedInputStack(members)
+            except (TypeError, ValueError):
+                continue
+            n += 1
+    return n

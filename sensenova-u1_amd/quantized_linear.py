@@ -258,6 +258,11 @@ class GGUFLinear(nn.Linear):
             raise RuntimeError(f"GGUFLinear: input dtype {inputs.dtype} does not match compute dtype {compute_dtype}")
         if compute_dtype == torch.bfloat16:
             rows = inputs.numel() // self.in_features if inputs.numel() else 0
+            stack = self.__dict__.get("_shared_stack")   # modality.SharedInputStack: q / k / v in one decode launch
+            if stack is not None:
+                out = stack.member_forward(self, inputs)
+                if out is not None:
+                    return out
             if self.decode_layout != "native":
                 out = self._decode_tiled(inputs, None)
                 if out is not None:

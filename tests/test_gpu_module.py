@@ -441,3 +441,77 @@ def test_loader_fused_mlp_forward_matches_the_three_module_calls(tmp_path, dev):
             assert torch.equal(plain, outs[m])
         else:
             assert go.rel_l2(outs[m].cpu(), plain.cpu()) <= 1e-3, m
+
+
+def test_loader_stacks_qkv_into_one_decode_launch(tmp_path, dev):
+    """q_proj / k_proj / v_proj of an attention-shaped module loaded through load_gguf_model share one weight tensor; at
+    decode row counts the q call runs one launch over all rows and k / v return their columns of it.  Every output
+    holds the tolerance against the oracle; other inputs, an input changed in place between the calls, more than 16
+    rows and a weight moved away from the stack all take the member's own launch."""
+    from sensenova_u1_amd import load_gguf_model
+    from sensenova_u1_amd.gguf_file import write_gguf
+    print("case loader-stacked qkv", flush=True)
+    NQ, NKV, HK = 512, 128, 256
+
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(HK, NQ, bias=False)
+            self.k_proj = torch.nn.Linear(HK, NKV, bias=False)
+            self.v_proj = torch.nn.Linear(HK, NKV, bias=False)
+            self.o_proj = torch.nn.Linear(NQ, HK, bias=False)
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.self_attn = Attn()
+
+    torch.manual_seed(4)
+    ref = Wrap()
+    packed = {n: go.quantize_q8_0(t.detach().numpy()) for n, t in ref.state_dict().items()}
+    path = str(tmp_path / "a.gguf")
+    write_gguf(path, [(n, p, 8) for n, p in packed.items()])
+    with torch.device("meta"):
+        meta = Wrap()
+    model = load_gguf_model(meta, path, dtype=torch.bfloat16, device=dev)
+    att = model.self_attn
+    stack = att.q_proj.__dict__["_shared_stack"]
+    assert stack is att.k_proj.__dict__["_shared_stack"] is att.v_proj.__dict__["_shared_stack"] and "_shared_stack" not in att.o_proj.__dict__
+    assert stack.intact() and att.k_proj.weight.data_ptr() == att.q_proj.weight.data_ptr() + NQ * (HK // 32) * 34
+
+    def want(name, x):
+        return go.gguf_linear_forward(x.cpu(), torch.from_numpy(packed[f"self_attn.{name}.weight"]), go.Q8_0)
+
+    for m in (1, 5, 16):
+        x = (torch.randn(1, m, HK, generator=torch.Generator().manual_seed(m)) * 0.8).to(torch.bfloat16).to(dev)
+        q = att.q_proj(x)
+        assert stack._pending is not None
+        k, v = att.k_proj(x), att.v_proj(x)
+        assert stack._pending is None                                  # consumed by the last member
+        assert q.shape == (1, m, NQ) and k.shape == (1, m, NKV) and v.shape == (1, m, NKV)
+        assert k.data_ptr() == q.data_ptr() + 2 * NQ and v.data_ptr() == k.data_ptr() + 2 * NKV   # columns of one buffer
+        q.view(1, m, -1, 64)                                           # the reference's reshape of the outputs works
+        for name, got in (("q_proj", q), ("k_proj", k), ("v_proj", v)):
+            assert go.rel_l2(got.cpu().reshape(m, -1), want(name, x.reshape(m, HK))) <= 1e-3, (name, m)
+    # another tensor for k: its own launch on that tensor
+    x1 = (torch.randn(2, HK, generator=torch.Generator().manual_seed(50)) * 0.8).to(torch.bfloat16).to(dev)
+    x2 = (torch.randn(2, HK, generator=torch.Generator().manual_seed(51)) * 0.8).to(torch.bfloat16).to(dev)
+    q = att.q_proj(x1)
+    k = att.k_proj(x2)
+    assert go.rel_l2(k.cpu(), want("k_proj", x2)) <= 1e-3 and k.data_ptr() != q.data_ptr() + 2 * NQ
+    # the same tensor changed in place between the calls: the version counter moved, k reads the new values
+    q = att.q_proj(x1)
+    x1.mul_(0.5)
+    k = att.k_proj(x1)
+    assert go.rel_l2(k.cpu(), want("k_proj", x1)) <= 1e-3
+    # more rows than the decode kernels take: three launches, separate tensors
+    xl = (torch.randn(40, HK, generator=torch.Generator().manual_seed(52)) * 0.8).to(torch.bfloat16).to(dev)
+    q, k = att.q_proj(xl), att.k_proj(xl)
+    assert q.is_contiguous() and k.is_contiguous() and go.rel_l2(k.cpu(), want("k_proj", xl)) <= 1e-3
+    # a weight that left the stack (an offloader's rebinding): no stacked launch, same results
+    att.k_proj.weight.data = att.k_proj.weight.data.clone()
+    assert not stack.intact()
+    q, k = att.q_proj(x2), att.k_proj(x2)
+    assert stack._pending is None and go.rel_l2(q.cpu(), want("q_proj", x2)) <= 1e-3 and go.rel_l2(k.cpu(), want("k_proj", x2)) <= 1e-3
+    stack.dissolve()
+    assert "_shared_stack" not in att.q_proj.__dict__ and go.rel_l2(att.v_proj(x2).cpu(), want("v_proj", x2)) <= 1e-3
