@@ -307,7 +307,9 @@ class SharedInputStack:
                 return None
             first = self.members[0]
             y = ops.linear(x, self.stacked, int(first.weight.quant_type), None, first.numerics)
-            self._pending = (key, y)
+            # x itself is kept with the result: while it is alive no other tensor can take its address, so an equal key
+            # can only come from a tensor that shares its storage, shape, strides and version - the same values
+            self._pending = (key, y, x)
             return y[..., :self.splits[0]]
         pending = self._pending
         if pending is None or pending[0] != key:
