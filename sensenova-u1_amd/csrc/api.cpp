@@ -207,6 +207,25 @@ namespace {
 // The dense kernel wants whole K steps and 32-bit activation offsets.  One weight pass + the dense kernel beat the
 // fused kernels from 65 rows on (measured on the four projection shapes of the 8B model, 65 ... 4096 rows); the
 // grouped form decodes two weight sets, which pays from a few hundred rows and enough tiles to occupy the chip.
+// How many workgroups share the K range of one 256 x 256 tile.  More slices shorten every workgroup's K loop but each
+// adds an fp32 copy of the output that is written and read again; fitted on the k / v, q, gate and down shapes at 128,
+// 512 and 4096 rows: time ~ rounds of 256 workgroups x K steps per slice x 1.9 us + slices x 8 M N bytes at 5 TB/s.
+int64_t pick_k_slices(int64_t M, int64_t N, int64_t tiles, int64_t ksteps, int64_t room, bool fused_decode) {
+    int64_t smax = 256 / tiles;
+    if (smax > room) smax = room;
+    if (smax > ksteps / 2) smax = ksteps / 2;   // at least two K steps per workgroup
+    if (smax > 64) smax = 64;
+    if (smax < 2) return 1;
+    const double t_step = fused_decode ? 1.9 : 1.65, t_slice = 8.0 * (double)M * (double)N / 5e6;   // us
+    int64_t best = 2;
+    double best_t = 1e30;
+    for (int64_t sl = 2; sl <= smax; sl++) {
+        const double t = (double)((ksteps + sl - 1) / sl) * t_step + (double)sl * t_slice;
+        if (t < best_t) { best_t = t; best = sl; }
+    }
+    return best;
+}
+
 bool dense_route_fits(int64_t M, int64_t N, int64_t K) {
     (void)N;
     return M >= 65 && K % 64 == 0 && M * K < ((int64_t)1 << 31);
@@ -238,11 +257,8 @@ int linear_ws_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N
     const bool tile_type = qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K;
     const int64_t dense_bytes = tile_type ? 0 : 2 * N * K;
     if (tiles <= 128 && workspace_bytes > dense_bytes) {
-        int64_t slices = 256 / tiles;
         const int64_t room = (workspace_bytes - dense_bytes) / (4 * M * N);
-        if (slices > room) slices = room;
-        if (slices > ksteps / 2) slices = ksteps / 2;   // at least two K steps per workgroup
-        if (slices > 64) slices = 64;
+        const int64_t slices = pick_k_slices(M, N, tiles, ksteps, room, tile_type);
         if (slices >= 2) {
             float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + dense_bytes);
             if (tile_type)
@@ -503,11 +519,8 @@ int sngguf_grouped_linear_ws(const void* x, int64_t M, const uint8_t* indicator,
     if (!two_pass && dense_workspace && tile_types && M >= 65 && N > 0 && K > 0 && K % 64 == 0 && M < kMaxDim && N < kMaxDim
         && K < kMaxDim && M * K < ((int64_t)1 << 31)) {
         const int64_t tiles = ((M + 255) / 256 + 1) * ((N + 255) / 256);   // a split into two groups adds one partial row tile
-        int64_t slices = tiles <= 128 ? 256 / tiles : 0;
         const int64_t room = dense_workspace_bytes / (4 * M * N);
-        if (slices > room) slices = room;
-        if (slices > K / 128) slices = K / 128;   // at least two K steps per workgroup
-        if (slices > 64) slices = 64;
+        const int64_t slices = tiles <= 128 ? pick_k_slices(M, N, tiles, K / 64, room, true) : 0;
         if (slices >= 2) {
             int rc = check_matmul(x, M, q_und, qtype_und, N, K, y, numerics);
             if (rc != SNGGUF_OK) return rc;
