@@ -247,14 +247,14 @@ class SharedInputStack:
     ``modeling_qwen3.py:444,450,456`` and the ``_mot_gen`` triple at ``:602,608,614``), with their packed rows stored one
     after another in ONE device tensor and every module's ``weight.data`` a view of its rows.
 
-    The modules stay separate ``GGUFLinear`` objects and the model code stays as it is.  At decode row counts the first
-    member's forward runs one launch over all rows - packed GGUF rows are independent, so the stacked rows are a valid
+    The modules stay separate ``GGUFLinear`` objects and the model code stays as it is.  For a single activation row (a
+    decode step) the first member's forward runs one launch over all rows - packed GGUF rows are independent, so the stacked rows are a valid
     weight of ``sum(out_features)`` rows - and keeps the result; the following members, called with the same tensor
     (same storage, shape, strides and version counter), return their columns of it.  Anything else - another input,
-    more than 16 rows, a weight that no longer lies where the stack put it (``.to()``, an offloader's rebinding) -
+    more than one row, a weight that no longer lies where the stack put it (``.to()``, an offloader's rebinding) -
     falls back to the member's own launch, so the stack never changes what a call returns, only how many launches
     a decode step needs (three -> one: the 4096 -> 1024 k / v launches cost more in launch overhead than in bytes).
-    Outputs of one step are column ranges of one buffer: disjoint, but not separately allocated."""
+    Outputs of one step are ranges of one buffer: contiguous and disjoint, but not separately allocated."""
 
     def __init__(self, members) -> None:
         members = list(members)
@@ -296,7 +296,9 @@ class SharedInputStack:
         """The member's output if the stack can supply it, else None (the member then runs its own launch)."""
         i = self.index[id(mod)]
         rows = x.numel() // mod.in_features if x.numel() else 0
-        if not (0 < rows <= 16 and x.is_cuda and x.dtype == torch.bfloat16):
+        # one row only: the members' outputs are then contiguous tensors like those of their own launches (with several
+        # rows they would be strided column ranges, which `.view(...)` calls that merge dimensions refuse)
+        if not (rows == 1 and x.is_cuda and x.dtype == torch.bfloat16):
             if i == 0:
                 self._pending = None
             return None
