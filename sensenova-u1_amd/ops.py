@@ -14,6 +14,7 @@ Ops (all launch on the current torch stream of the input's device, never synchro
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 from typing import Optional
@@ -161,12 +162,28 @@ def _require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_NO_GUARD = contextlib.nullcontext()
+
+
 def _stream(dev: torch.device) -> int:
+    """The current torch stream of ``dev`` as a raw handle."""
+    if _raw_stream is not None:
+        return _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(dev).cuda_stream
 
 
+def _on(dev: torch.device):
+    """Context in which ``dev`` is the current device (a launch on one of its streams needs that); free of charge when
+    it already is, which is every call of a one-GPU process."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(dev)
+
+
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device address for a ``void*`` argument (ctypes converts the integer)."""
+    return None if t is None else t.data_ptr()
 
 
 def _packed_2d(packed: torch.Tensor, quant_type: int):
@@ -174,6 +191,11 @@ def _packed_2d(packed: torch.Tensor, quant_type: int):
     if quant_type not in GGML_QUANT_SIZES:
         raise SnGgufError(f"quant type {quant_type} is not implemented (have Q4_0=2, Q4_1=3, Q5_0=6, Q5_1=7, Q8_0=8, Q2_K=10, Q3_K=11, Q4_K=12, Q5_K=13, Q6_K=14, BF16=30)")
     bs, ts = GGML_QUANT_SIZES[quant_type]
+    if type(packed) is torch.Tensor and packed.dtype == torch.uint8 and packed.dim() == 2 and packed.is_contiguous() \
+            and not packed.requires_grad:
+        if packed.shape[1] % ts != 0:
+            raise SnGgufError(f"packed row of {packed.shape[1]} bytes is not a whole number of {ts}-byte blocks")
+        return packed, packed.shape[0], packed.shape[1] // ts * bs
     p = packed.detach()
     if p.dtype != torch.uint8:
         p = p.view(torch.uint8)
@@ -193,9 +215,9 @@ def dequantize_into(packed: torch.Tensor, quant_type: int, out: torch.Tensor, nu
     p, n, k = _packed_2d(packed, quant_type)
     if out.numel() != n * k or not out.is_contiguous() or out.dtype not in _OUT_CODE:
         raise SnGgufError("dequantize: out must be a contiguous fp32/fp16/bf16 tensor of N*K elements")
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_dequantize(_ptr(p), quant_type, n, k, _ptr(out), _OUT_CODE[out.dtype], numerics,
-                                              ctypes.c_void_p(_stream(dev)))
+                                              _stream(dev))
     _check(rc, "sngguf_dequantize")
 
 
@@ -204,9 +226,9 @@ def linear_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: 
     """y2d[M, N] = x2d[M, K] @ W^T (+ bias); x2d / y2d contiguous bf16, no checks beyond the library's."""
     dev = x2d.device
     n, k = y2d.shape[1], x2d.shape[1]
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_linear(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
-                                          _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+                                          _ptr(y2d), numerics, _stream(dev))
     _check(rc, "sngguf_linear")
 
 
@@ -250,9 +272,9 @@ def linear_ws_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int, bia
     dev = x2d.device
     n, k = y2d.shape[1], x2d.shape[1]
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_linear_ws(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
-                                             _ptr(y2d), _ptr(workspace), ws_bytes, numerics, ctypes.c_void_p(_stream(dev)))
+                                             _ptr(y2d), _ptr(workspace), ws_bytes, numerics, _stream(dev))
     _check(rc, "sngguf_linear_ws")
 
 
@@ -267,9 +289,9 @@ def linear_static_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: int,
     allocates nothing.  ``M * N`` beyond ``linear_static_max_outputs()`` is refused."""
     dev = x2d.device
     n, k = y2d.shape[1], x2d.shape[1]
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_linear_static(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
-                                                 _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+                                                 _ptr(y2d), numerics, _stream(dev))
     _check(rc, "sngguf_linear_static")
 
 
@@ -278,19 +300,19 @@ def linear_residual_into(x2d: torch.Tensor, packed: torch.Tensor, quant_type: in
     """y2d[M, N] = residual2d + (x2d @ W^T + bias), rounded to bf16 after the projection and after the add."""
     dev = x2d.device
     n, k = y2d.shape[1], x2d.shape[1]
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_linear_residual(_ptr(x2d), x2d.shape[0], _ptr(packed), quant_type, n, k, _ptr(bias),
-                                                   _ptr(residual2d), _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+                                                   _ptr(residual2d), _ptr(y2d), numerics, _stream(dev))
     _check(rc, "sngguf_linear_residual")
 
 
 def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int, h2d: torch.Tensor,
                       numerics: int) -> None:
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_gate_up_silu(_ptr(x2d), x2d.shape[0], _ptr(gate), _ptr(up), quant_type,
                                                 h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
-                                                ctypes.c_void_p(_stream(dev)))
+                                                _stream(dev))
     _check(rc, "sngguf_gate_up_silu")
 
 
@@ -350,10 +372,10 @@ def rmsnorm_linear_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float, pack
     """y2d[M, N] = RMSNorm(x2d; gamma, eps) @ W^T (+ bias), the norm of Qwen3RMSNorm
     (modeling_qwen3.py:192-197) applied inside the projection kernel; shapes as ``rmsnorm_fits`` allows."""
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_rmsnorm_linear(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(packed), quant_type,
                                                   y2d.shape[1], x2d.shape[1], _ptr(bias), _ptr(y2d), numerics,
-                                                  ctypes.c_void_p(_stream(dev)))
+                                                  _stream(dev))
     _check(rc, "sngguf_rmsnorm_linear")
 
 
@@ -361,10 +383,10 @@ def rmsnorm_gate_up_silu_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float
                               quant_type: int, h2d: torch.Tensor, numerics: int) -> None:
     """h2d = silu(n @ Wg^T) * (n @ Wu^T) with n = RMSNorm(x2d; gamma, eps), in one launch."""
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_rmsnorm_gate_up_silu(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(gate), _ptr(up),
                                                         quant_type, h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
-                                                        ctypes.c_void_p(_stream(dev)))
+                                                        _stream(dev))
     _check(rc, "sngguf_rmsnorm_gate_up_silu")
 
 
@@ -372,10 +394,10 @@ def rmsnorm_linear_tiled_into(x2d: torch.Tensor, gamma: torch.Tensor, eps: float
                               bias: Optional[torch.Tensor], y2d: torch.Tensor, numerics: int) -> None:
     """``rmsnorm_linear_into`` with W given as its tiled copy."""
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_rmsnorm_linear_tiled(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(tiled),
                                                         y2d.shape[1], x2d.shape[1], _ptr(bias), _ptr(y2d), numerics,
-                                                        ctypes.c_void_p(_stream(dev)))
+                                                        _stream(dev))
     _check(rc, "sngguf_rmsnorm_linear_tiled")
 
 
@@ -383,21 +405,21 @@ def rmsnorm_gate_up_silu_tiled_into(x2d: torch.Tensor, gamma: torch.Tensor, eps:
                                     tiled_up: torch.Tensor, h2d: torch.Tensor, numerics: int) -> None:
     """``rmsnorm_gate_up_silu_into`` on two tiled matrices."""
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_rmsnorm_gate_up_silu_tiled(_ptr(x2d), x2d.shape[0], _ptr(gamma), float(eps), _ptr(tiled_gate),
                                                               _ptr(tiled_up), h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
-                                                              ctypes.c_void_p(_stream(dev)))
+                                                              _stream(dev))
     _check(rc, "sngguf_rmsnorm_gate_up_silu_tiled")
 
 
 def grouped_linear_into(x2d, indicator, n_text, packed_und, qt_und, packed_gen, qt_gen, bias_und, bias_gen, y2d,
                         workspace, numerics) -> None:
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_grouped_linear(
             _ptr(x2d), x2d.shape[0], _ptr(indicator), n_text, _ptr(packed_und), qt_und, _ptr(packed_gen), qt_gen,
             y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), numerics,
-            ctypes.c_void_p(_stream(dev)))
+            _stream(dev))
     _check(rc, "sngguf_grouped_linear")
 
 
@@ -407,11 +429,11 @@ def grouped_linear_ws_into(x2d, indicator, n_text, packed_und, qt_und, packed_ge
     bytes large problems decode both weight sets once and run one dense tile-GEMM launch over both row groups."""
     dev = x2d.device
     dw_bytes = dense_workspace.numel() * dense_workspace.element_size() if dense_workspace is not None else 0
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_grouped_linear_ws(
             _ptr(x2d), x2d.shape[0], _ptr(indicator), n_text, _ptr(packed_und), qt_und, _ptr(packed_gen), qt_gen,
             y2d.shape[1], x2d.shape[1], _ptr(bias_und), _ptr(bias_gen), _ptr(y2d), _ptr(workspace), _ptr(dense_workspace),
-            dw_bytes, numerics, ctypes.c_void_p(_stream(dev)))
+            dw_bytes, numerics, _stream(dev))
     _check(rc, "sngguf_grouped_linear_ws")
 
 
@@ -433,18 +455,18 @@ def linear_tiled_into(x2d: torch.Tensor, tiled: torch.Tensor, bias: Optional[tor
                       y2d: torch.Tensor, numerics: int) -> None:
     """y2d[M, N] = x2d[M, K] @ W^T (+ bias) (+ residual) with W given as its tiled copy; M <= 16."""
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_linear_tiled(_ptr(x2d), x2d.shape[0], _ptr(tiled), y2d.shape[1], x2d.shape[1], _ptr(bias),
-                                                _ptr(residual), _ptr(y2d), numerics, ctypes.c_void_p(_stream(dev)))
+                                                _ptr(residual), _ptr(y2d), numerics, _stream(dev))
     _check(rc, "sngguf_linear_tiled")
 
 
 def gate_up_silu_tiled_into(x2d: torch.Tensor, tiled_gate: torch.Tensor, tiled_up: torch.Tensor, h2d: torch.Tensor,
                             numerics: int) -> None:
     dev = x2d.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = load_library().sngguf_gate_up_silu_tiled(_ptr(x2d), x2d.shape[0], _ptr(tiled_gate), _ptr(tiled_up), h2d.shape[1],
-                                                      x2d.shape[1], _ptr(h2d), numerics, ctypes.c_void_p(_stream(dev)))
+                                                      x2d.shape[1], _ptr(h2d), numerics, _stream(dev))
     _check(rc, "sngguf_gate_up_silu_tiled")
 
 
@@ -455,6 +477,16 @@ def _as_bf16_rows(x: torch.Tensor, k: int, what: str) -> torch.Tensor:
         raise SnGgufError(f"{what}: last dim of the input is {x.shape[-1]}, the weight has in_features={k}")
     x2d = x.reshape(-1, k)
     return x2d if x2d.is_contiguous() else x2d.contiguous()
+
+
+def _bf16_rows_flat(x: torch.Tensor, k: int, what: str):
+    """``x`` as contiguous bf16 rows of width ``k`` without making a view: (tensor whose memory is [M, K], M)."""
+    if x.dtype != torch.bfloat16:
+        raise SnGgufError(f"{what}: activations must be torch.bfloat16, got {x.dtype}")
+    if x.shape[-1] != k:
+        raise SnGgufError(f"{what}: last dim of the input is {x.shape[-1]}, the weight has in_features={k}")
+    xc = x if x.is_contiguous() else x.contiguous()
+    return xc, (xc.numel() // k if k else 0)
 
 
 def _bias_bf16(bias: Optional[torch.Tensor], n: int, what: str) -> Optional[torch.Tensor]:
@@ -489,12 +521,16 @@ def _dequantize_hip(packed, quant_type, out_dtype, numerics):
 
 
 def _linear_hip(x, packed, quant_type, bias, numerics):
-    _require_device(x, packed, bias)
+    dev = _require_device(x, packed, bias)
     p, n, k = _packed_2d(packed, quant_type)
-    x2d = _as_bf16_rows(x, k, "linear")
-    y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
-    if y.numel():
-        linear_into(x2d, p, quant_type, _bias_bf16(bias, n, "linear"), y.view(-1, n), numerics)
+    xc, m = _bf16_rows_flat(x, k, "linear")
+    y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=dev)
+    if m and n:
+        b = _bias_bf16(bias, n, "linear")   # (held until the launch is enqueued)
+        with _on(dev):
+            rc = load_library().sngguf_linear(xc.data_ptr(), m, p.data_ptr(), quant_type, n, k, _ptr(b), y.data_ptr(),
+                                              numerics, _stream(dev))
+        _check(rc, "sngguf_linear")
     return y
 
 
@@ -518,10 +554,14 @@ def _gate_up_silu_hip(x, gate, up, quant_type, numerics):
     pu, n2, k2 = _packed_2d(up, quant_type)
     if (n, k) != (n2, k2):
         raise SnGgufError("gate_up_silu: gate and up weights differ in shape")
-    x2d = _as_bf16_rows(x, k, "gate_up_silu")
+    xc, m = _bf16_rows_flat(x, k, "gate_up_silu")
     h = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
-    if h.numel():
-        gate_up_silu_into(x2d, pg, pu, quant_type, h.view(-1, n), numerics)
+    if m and n:
+        dev = x.device
+        with _on(dev):
+            rc = load_library().sngguf_gate_up_silu(xc.data_ptr(), m, pg.data_ptr(), pu.data_ptr(), quant_type, n, k,
+                                                    h.data_ptr(), numerics, _stream(dev))
+        _check(rc, "sngguf_gate_up_silu")
     return h
 
 
@@ -597,7 +637,18 @@ def _plain(t):
     """Strip Parameter subclasses so the dispatcher sees an ordinary tensor."""
     if t is None:
         return None
-    return t.as_tensor() if hasattr(t, "as_tensor") else t.detach()
+    if type(t) is torch.Tensor:
+        return t if not t.requires_grad else t.detach()
+    with torch._C.DisableTorchFunctionSubclass():   # (attribute reads of a tagged Parameter cost microseconds each otherwise)
+        return torch.Tensor._make_subclass(torch.Tensor, t, False)
+
+
+def _eager(x: torch.Tensor) -> bool:
+    """Whether a call can go straight to the HIP implementation: a real device tensor, nothing tracing or intercepting.
+    (The registered ops stay the route of torch.compile / export / dispatch modes; in plain eager inference the dispatcher
+    hop costs about as much host time as the launch itself.)"""
+    return (type(x) is torch.Tensor and x.is_cuda and not torch.compiler.is_compiling()
+            and torch._C._len_torch_dispatch_stack() == 0)
 
 
 def dequantize(packed: torch.Tensor, quant_type: int, out_dtype: torch.dtype = torch.float32,
@@ -607,17 +658,23 @@ def dequantize(packed: torch.Tensor, quant_type: int, out_dtype: torch.dtype = t
 
 def linear(x: torch.Tensor, packed: torch.Tensor, quant_type: int, bias: Optional[torch.Tensor] = None,
            numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    if _eager(x):
+        return _linear_hip(x, _plain(packed), int(quant_type), _plain(bias), int(numerics))
     return torch.ops.sn_gguf.linear(x, _plain(packed), int(quant_type), _plain(bias), int(numerics))
 
 
 def linear_residual(x: torch.Tensor, packed: torch.Tensor, quant_type: int, residual: torch.Tensor,
                     bias: Optional[torch.Tensor] = None, numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
     """``residual + linear(x)`` in one launch (bf16 rounding after the projection and after the add)."""
+    if _eager(x):
+        return _linear_residual_hip(x, _plain(packed), int(quant_type), _plain(bias), residual, int(numerics))
     return torch.ops.sn_gguf.linear_residual(x, _plain(packed), int(quant_type), _plain(bias), residual, int(numerics))
 
 
 def gate_up_silu(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int,
                  numerics: int = NUM_UPSTREAM_FP16) -> torch.Tensor:
+    if _eager(x):
+        return _gate_up_silu_hip(x, _plain(gate), _plain(up), int(quant_type), int(numerics))
     return torch.ops.sn_gguf.gate_up_silu(x, _plain(gate), _plain(up), int(quant_type), int(numerics))
 
 

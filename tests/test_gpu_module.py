@@ -522,3 +522,37 @@ def test_loader_stacks_qkv_into_one_decode_launch(tmp_path, dev):
     assert stack._pending is None and go.rel_l2(q.cpu(), want("q_proj", x2)) <= 1e-3 and go.rel_l2(k.cpu(), want("k_proj", x2)) <= 1e-3
     stack.dissolve()
     assert "_shared_stack" not in att.q_proj.__dict__ and go.rel_l2(att.v_proj(x2).cpu(), want("v_proj", x2)) <= 1e-3
+
+
+def test_registered_ops_and_direct_eager_route_agree(dev):
+    """ops.linear / gate_up_silu / linear_residual go straight to the HIP implementation in plain eager calls and through
+    the registered sn_gguf ops otherwise (torch.compile, export, dispatch modes): both routes give the same bits."""
+    print("case eager route vs registered ops", flush=True)
+    n, k = 320, 512
+    w = synthetic.make_packed(go.Q8_0, n, k, seed=1).to(dev)
+    u = synthetic.make_packed(go.Q8_0, n, k, seed=2).to(dev)
+    x = synthetic.make_activations(3, k, seed=3).to(dev).reshape(1, 3, k)
+    res = synthetic.make_activations(3, n, seed=4).to(dev).reshape(1, 3, n)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(5)) * 0.5).to(torch.bfloat16).to(dev)
+    assert ops._eager(x)
+    assert torch.equal(ops.linear(x, w, go.Q8_0, bias), torch.ops.sn_gguf.linear(x, w, go.Q8_0, bias, 1))
+    assert torch.equal(ops.gate_up_silu(x, w, u, go.Q8_0), torch.ops.sn_gguf.gate_up_silu(x, w, u, go.Q8_0, 1))
+    assert torch.equal(ops.linear_residual(x, w, go.Q8_0, res, bias), torch.ops.sn_gguf.linear_residual(x, w, go.Q8_0, bias, res, 1))
+    # a non-contiguous input and a tagged parameter as the weight take the same route
+    xt = synthetic.make_activations(k, 3, seed=6).to(dev).t()
+    wp = GGUFParameter(w, quant_type=go.Q8_0)
+    assert not xt.is_contiguous()
+    assert torch.equal(ops.linear(xt, wp, go.Q8_0), torch.ops.sn_gguf.linear(xt.contiguous(), w, go.Q8_0, None, 1))
+    # under a dispatch mode the registered op is used (the mode sees it)
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    seen = []
+
+    class Spy(TorchDispatchMode):
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            seen.append(str(func))
+            return func(*args, **(kwargs or {}))
+
+    with Spy():
+        y = ops.linear(x, w, go.Q8_0, bias)
+    assert any("sn_gguf.linear" in f for f in seen) and torch.equal(y, ops.linear(x, w, go.Q8_0, bias))
