@@ -265,13 +265,53 @@ __device__ __forceinline__ void decode_q3_k(half4_t ident, const uint8_t* row, i
 }
 
 
+// (d * scale, dmin * min) of sub-blocks 4 HALF .. 4 HALF + 3 of the lane's row (Q4_K and Q5_K).  The four lanes
+// (r, g = 0..3) that decode one row all need the same four pairs: lane (r, g) extracts and scales the pair of
+// sub-block 4 HALF + g only, and the four exchange their results through the cross-lane network (ds_bpermute, which
+// touches no LDS memory).  Same arithmetic on the same operands as computing every pair in every lane, so the
+// values are bit-identical; it takes a quarter of the decode's vector instructions away.  Must be called by all
+// 64 lanes.
+template <int NUM, int HALF>
+__device__ __forceinline__ void q4k_pairs(const u32x4_t& head, int g, typename Num<NUM>::T (&D)[4], typename Num<NUM>::T (&DM)[4]) {
+    typedef Num<NUM> A;
+    uint32_t sc, mn;
+    if constexpr (HALF == 0) {
+        sc = (head[1] >> (8 * g)) & 63u;
+        mn = (head[2] >> (8 * g)) & 63u;
+    } else {
+        const uint32_t b = (head[3] >> (8 * g)) & 0xFFu;
+        sc = (b & 0x0Fu) | (((head[1] >> (8 * g + 6)) & 3u) << 4);
+        mn = (b >> 4) | (((head[2] >> (8 * g + 6)) & 3u) << 4);
+    }
+    const typename A::T mine_d = A::scale((uint16_t)(head[0] & 0xFFFF)) * A::integer((int)sc);
+    const typename A::T mine_m = A::scale((uint16_t)(head[0] >> 16)) * A::integer((int)mn);
+    const int self = 4 * (int)(threadIdx.x & 15);  // byte address of lane (r, 0) for ds_bpermute
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const half2_t both = {mine_d, mine_m};
+        const int bits = __builtin_bit_cast(int, both);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const half2_t got = __builtin_bit_cast(half2_t, __builtin_amdgcn_ds_bpermute(self + 64 * jj, bits));
+            D[jj] = got[0];
+            DM[jj] = got[1];
+        }
+    } else {
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            D[jj] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(self + 64 * jj, __builtin_bit_cast(int, mine_d)));
+            DM[jj] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(self + 64 * jj, __builtin_bit_cast(int, mine_m)));
+        }
+    }
+}
+
 // The four A operands of half a super-block (sub-blocks 4 HALF .. 4 HALF + 3) of one row, fed to
 // `emit(jj, a)` with jj = 0..3.  `row` points at the row's super-block in the slab; g = lane / 16.
 template <int NUM, int HALF, typename Emit>
 __device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
     typedef Num<NUM> A;
     const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
-    const typename A::T d = A::scale((uint16_t)(head[0] & 0xFFFF)), dmin = A::scale((uint16_t)(head[0] >> 16));
+    typename A::T Ds[4], DMs[4];
+    q4k_pairs<NUM, HALF>(head, g, Ds, DMs);
 #pragma unroll
     for (int cc = 0; cc < 2; cc++) {
         const int c = 2 * HALF + cc;
@@ -279,9 +319,7 @@ __device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, i
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
             const int j = 2 * c + hi;
-            uint32_t sc, mn;
-            q4k_scale_min(head[1], head[2], head[3], j, sc, mn);
-            const typename A::T D = d * A::integer((int)sc), DM = dmin * A::integer((int)mn);
+            const typename A::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
             const uint32_t v0 = (hi ? qs[0] >> 4 : qs[0]) & 0x0F0F0F0Fu, v1 = (hi ? qs[1] >> 4 : qs[1]) & 0x0F0F0F0Fu;
             uint32_t a0, a1, a2, a3;
             kq_dword_bf16<NUM, true>(ident, v0, 0.f, D, DM, a0, a1);
@@ -296,7 +334,8 @@ template <int NUM, int HALF, typename Emit>
 __device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
     typedef Num<NUM> A;
     const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
-    const typename A::T d = A::scale((uint16_t)(head[0] & 0xFFFF)), dmin = A::scale((uint16_t)(head[0] >> 16));
+    typename A::T Ds[4], DMs[4];
+    q4k_pairs<NUM, HALF>(head, g, Ds, DMs);
     const u32x2_t qh = *reinterpret_cast<const u32x2_t*>(row + 16 + 8 * g);
 #pragma unroll
     for (int cc = 0; cc < 2; cc++) {
@@ -305,9 +344,7 @@ __device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, i
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
             const int j = 2 * c + hi;
-            uint32_t sc, mn;
-            q4k_scale_min(head[1], head[2], head[3], j, sc, mn);
-            const typename A::T D = d * A::integer((int)sc), DM = dmin * A::integer((int)mn);
+            const typename A::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
             uint32_t a[4];
 #pragma unroll
             for (int w = 0; w < 2; w++) {
@@ -367,9 +404,11 @@ __device__ __forceinline__ void decode_half(half4_t ident, const uint8_t* row, i
     }
 }
 
-// XN (MT = 1 only): RMSNorm(x) with weight `gamma` is what gets contracted (see rmsnorm_piece).  Each wavefront
-// stages the K range it works on (all M rows) in LDS behind the slabs, the workgroup adds up the sums of squares,
-// every wavefront normalizes its own share in place, and the B fragments come from there.
+// XN (MT = 1 only): the B fragments come from LDS.  Each wavefront stages the K range it works on (all M rows)
+// behind the slabs.  With `gamma` set, RMSNorm(x) with weight `gamma` is what gets contracted (see rmsnorm_piece):
+// the workgroup adds up the sums of squares and every wavefront normalizes its own share in place.  Without it
+// the rows are staged as they are, which takes the eight activation requests per step off the vector memory
+// path (worth it for Q6_K, whose unaligned slab pieces already load that path most).
 template <int QT, int NUM, int R, bool GATED, int WMAX, int MT, bool XN = false>
 __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* __restrict__ x, int M,
                                                                  const uint8_t* __restrict__ qa,
@@ -500,7 +539,20 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
         float* ssum = reinterpret_cast<float*>(lds + waves * kSlab + waves * (M * xrow_b));  // [M][waves]
         const int pieces = (s1 - s0) * 32;               // 16-byte pieces per row in this wavefront's K range
         const int64_t k0 = (int64_t)s0 * 256;
-        for (int m = 0; m < M; m++) {
+        if (!gamma) {
+            // plain staging, four requests in flight per lane; a wavefront reads back only what it wrote itself
+            for (int m = 0; m < M; m++)
+                for (int c0 = lane; c0 < pieces; c0 += 256) {
+                    u32x4_t v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        if (c0 + 64 * u < pieces) v[u] = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + k0 + 8 * (c0 + 64 * u));
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        if (c0 + 64 * u < pieces) *reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * (c0 + 64 * u)) = v[u];
+                }
+        }
+        for (int m = 0; gamma && m < M; m++) {
             float ss = 0.f;
             for (int c = lane; c < pieces; c += 64) {
                 const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * K + k0 + 8 * c);
@@ -510,8 +562,8 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
             ss = wave_sum(ss);
             if (lane == 0) ssum[m * waves + wave] = ss;
         }
-        __syncthreads();
-        for (int m = 0; m < M; m++) {
+        if (gamma) __syncthreads();   // (uniform over the workgroup)
+        for (int m = 0; gamma && m < M; m++) {
             float tot = 0.f;
             for (int w = 0; w < W; w++) tot += ssum[m * waves + w];   // wavefronts [0, W) cover K once
             const float rstd = rsqrtf(tot / (float)K + eps);
@@ -608,7 +660,11 @@ int launch_r(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int64
     const size_t slab = (size_t)waves * 16 * R * Slab<QT>::stride;
     const size_t red = (size_t)waves * R * mt * 64 * sizeof(f32x4_t);
     const dim3 grid((unsigned)groups), block((unsigned)(64 * waves));
-    if (gamma) {
+    // Q6_K streams its activations from LDS too when one or two rows of them fit there and the matrix is large
+    // (12288 x 4096 at M = 1: 13.6 against 15.3 us; the other formats and small matrices lose by it)
+    const bool stage = QT == SNGGUF_TYPE_Q6_K && !gamma && M <= 2 && N * K >= ((int64_t)32 << 20) &&
+                       (size_t)M * (2 * (size_t)K + 64) <= 36 * 1024;
+    if (gamma || stage) {
         // slabs, then every wavefront's share of the activations ([M][xrow_b]), then [M][waves] sums of squares; the
         // caller keeps M (2 K + 64) within 36 KB
         if (mt > 1) return SNGGUF_E_BADSHAPE;

@@ -100,3 +100,46 @@ def test_q8_0_down_projection_with_residual_at_decode(dev):
         y = ops.linear_residual(x, packed, go.Q8_0, res)
         assert torch.equal(y, res + ops.linear(x, packed, go.Q8_0))
         _sample_check(ops.linear(x, packed, go.Q8_0), x, packed, go.Q8_0, gen, f"down m={m}")
+
+
+@pytest.mark.parametrize("num", [ops.NUM_GGML_FP32, ops.NUM_UPSTREAM_FP16])
+def test_q6_k_large_projection_with_activations_staged_in_lds(dev, c_oracle, num):
+    """Q6_K at 12288 x 4096: with one or two activation rows the decode kernel streams them from LDS, with three it
+    reads them from global memory.  Plain projection with bias and residual, and the gated pair; the rows that both
+    routes compute must agree bit for bit (same fragments, same order of accumulation)."""
+    n, k = 12288, 4096
+    qt = go.Q6_K
+    gen = torch.Generator().manual_seed(14 + num)
+    gate = synthetic.make_packed(qt, n, k, seed=45, device=dev)
+    up = synthetic.make_packed(qt, n, k, seed=46, device=dev)
+    bias = synthetic.make_activations(1, n, seed=47, device=dev).reshape(n)
+    x3 = synthetic.make_activations(3, k, seed=90, device=dev)
+    y3 = torch.empty((3, n), dtype=torch.bfloat16, device=dev)
+    ops.linear_into(x3, gate, qt, bias, y3, num)
+    h3 = torch.empty((3, n), dtype=torch.bfloat16, device=dev)
+    ops.gate_up_silu_into(x3, gate, up, qt, h3, num)
+    for m in (1, 2):
+        print(f"case full q6_k staged num={num} m={m}", flush=True)
+        x = x3[:m].contiguous()
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.linear_into(x, gate, qt, bias, y, num)
+        assert torch.equal(y, y3[:m])
+        if num == ops.NUM_UPSTREAM_FP16:
+            _sample_check(y, x, gate, qt, gen, f"staged linear m={m}", bias=bias)
+        h = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.gate_up_silu_into(x, gate, up, qt, h, num)
+        assert torch.equal(h, h3[:m])
+        if num == ops.NUM_UPSTREAM_FP16:
+            cols = torch.randint(0, n, (64,), generator=gen)
+            cols[0], cols[1] = 0, n - 1
+            g = go.gguf_linear_forward(x.cpu(), gate[cols.to(dev)].cpu(), qt)
+            u = go.gguf_linear_forward(x.cpu(), up[cols.to(dev)].cpu(), qt)
+            assert go.rel_l2(h[:, cols.to(dev)].cpu(), c_oracle.silu_mul(g, u)) <= TOL
+    # the 12288 -> 4096 projection with a residual, one row (two rows of K = 12288 do not fit and take the other route)
+    down = synthetic.make_packed(qt, 4096, 12288, seed=48, device=dev)
+    xd = synthetic.make_activations(2, 12288, seed=91, device=dev)
+    res = synthetic.make_activations(2, 4096, seed=92, device=dev)
+    y2 = ops.linear_residual(xd, down, qt, res)
+    y1 = ops.linear_residual(xd[:1].contiguous(), down, qt, res[:1].contiguous())
+    assert torch.equal(y1, y2[:1])
+    _sample_check(ops.linear(xd[:1].contiguous(), down, qt), xd[:1].contiguous(), down, qt, gen, "staged down m=1")
