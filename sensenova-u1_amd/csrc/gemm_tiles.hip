@@ -1,5 +1,6 @@
-// Dequant-GEMM, large-tile variant for Q8_0 (K % 64 == 0) and Q4_K - and, as the second pass of the
-// workspace route, for weights already decoded to bf16: 256 x 256 output tile per
+// Dequant-GEMM, large-tile variant for Q8_0 (K % 64 == 0) and Q4_K - and for weights already decoded to
+// bf16 (second pass of the workspace route) in the launches that the four-wavefront dense kernel of
+// gemm_dense4.hip does not take (an odd number of K steps per workgroup): 256 x 256 output tile per
 // workgroup, K step 64, eight wavefronts of 64 (rows) x 128 (columns) - 2 x 4 MFMA tiles of 32 x 32,
 // 128 accumulator registers each, two wavefronts per SIMD - and two LDS stages.
 //
@@ -638,6 +639,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 
 }  // namespace
 
+int launch_gemm_dense4(const GemmArgs& a, hipStream_t stream);
+
 // Q8_0 with K % 64 == 0 (rows are then 4-byte aligned), Q4_K, or type 30 = weights that are already bf16 rows
 // (K % 64 == 0; the numerics mode plays no role); both row groups of that type.
 int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t stream) {
@@ -646,7 +649,13 @@ int launch_gemm_tiles(const GemmArgs& a, int qtype, int numerics, hipStream_t st
     SNGGUF_CASE(SNGGUF_TYPE_Q8_0, SNGGUF_NUM_UPSTREAM_FP16);
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_GGML_FP32);
     SNGGUF_CASE(SNGGUF_TYPE_Q4_K, SNGGUF_NUM_UPSTREAM_FP16);
-    if (qtype == kTypeBF16) return launch_tiles<kTypeBF16, SNGGUF_NUM_GGML_FP32>(a, stream);
+    if (qtype == kTypeBF16) {
+        // the four-wavefront form takes every launch whose workgroups get an even number of K steps (its loop has
+        // one body for a pair of steps); the dense form of the tile kernel above keeps the rest
+        const int64_t S = a.ksplit > 1 ? a.ksplit : 1;
+        if ((a.K / TK) % (2 * S) == 0) return launch_gemm_dense4(a, stream);
+        return launch_tiles<kTypeBF16, SNGGUF_NUM_GGML_FP32>(a, stream);
+    }
 #undef SNGGUF_CASE
     return SNGGUF_E_BADTYPE;
 }
