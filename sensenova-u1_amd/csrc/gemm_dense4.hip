@@ -31,14 +31,14 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const void* p) {
     return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
 }
 
-// EP: which epilogue this instance carries (one per instance, so that the 256 accumulators of a lane are read out of
-// their accumulation registers group by group on one path instead of all at once in front of a three-way branch):
-// 0 = bf16 tile staged through LDS (N % 8 == 0), 1 = fp32 partial sums of a K slice, 2 = direct stores (any N).
 // byte offset of an LDS address within the workgroup's LDS allocation (what M0 and the ds instructions take)
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
+// EP: which epilogue this instance carries (one per instance, so that the 256 accumulators of a lane are read out of
+// their accumulation registers group by group on one path instead of all at once in front of a three-way branch):
+// 0 = bf16 tile staged through LDS (N % 8 == 0), 1 = fp32 partial sums of a K slice, 2 = direct stores (any N).
 template <int EP>
 __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
