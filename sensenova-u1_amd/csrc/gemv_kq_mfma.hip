@@ -566,7 +566,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_kq_mfma_kernel(const bf16_t* _
         for (int m = 0; gamma && m < M; m++) {
             float tot = 0.f;
             for (int w = 0; w < W; w++) tot += ssum[m * waves + w];   // wavefronts [0, W) cover K once
-            const float rstd = rsqrtf(tot / (float)K + eps);
+            const float rstd = rms_rstd(tot, K, eps);
             for (int c = lane; c < pieces; c += 64) {
                 u32x4_t* cell = reinterpret_cast<u32x4_t*>(xw + m * xrow_b + 16 * c);
                 const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + k0 + 8 * c);

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
             for (int m = 0; m < M; m++) {
                 float tot = 0.f;
                 for (int w = 0; w < waves; w++) tot += ssum[m * waves + w];
-                const float rstd = rsqrtf(tot / (float)K + eps);
+                const float rstd = rms_rstd(tot, K, eps);
                 for (int c = tid; c < pieces_per_row; c += (int)blockDim.x) {
                     u32x4_t* cell = reinterpret_cast<u32x4_t*>(lds + m * xs_stride + 16 * c);
                     const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gamma + 8 * c);

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(const bf16_t* __
     float tot = 0.f;
 #pragma unroll
     for (int w = 0; w < kThreads / 64; w++) tot += part[w];
-    const float rstd = rsqrtf(tot / (float)K + eps);
+    const float rstd = rms_rstd(tot, K, eps);
     if (pieces <= (int64_t)kThreads * kPiecesPerThread) {
 #pragma unroll
         for (int i = 0; i < kPiecesPerThread; i++) {

@@ -414,6 +414,15 @@ __device__ __forceinline__ void argmax_store(uint64_t key, int g, uint64_t* __re
 // With `gamma` given, a kernel below applies it to the activations it has staged in LDS, so the norm needs no
 // launch and no buffer of its own.  Only offered where the activations are staged once per workgroup (or once
 // per wavefront share) - a few rows; applied per fragment it would cost as much vector work as the weight decode.
+// 1 / sqrt(mean of squares + eps) with a correctly rounded square root and a correctly rounded division - the two
+// roundings of torch.rsqrt on the CPU - instead of the hardware's reciprocal-square-root approximation, which is
+// within one unit in the last place of that.  A last-place difference in rstd is invisible except for a row whose
+// activations share a mantissa for which x * rstd falls exactly between two bf16 values: dozens of normalized
+// activations then round the other way.  (The order in which the squares are added up is the other source of such
+// a difference, and that one cannot be matched to a CPU reduction.)
+__device__ __forceinline__ float rms_rstd(float sum_of_squares, int64_t K, float eps) {
+    return 1.0f / sqrtf(sum_of_squares / (float)K + eps);
+}
 __device__ __forceinline__ float sumsq_piece(u32x4_t xv) {
     float ss = 0.f;
 #pragma unroll
