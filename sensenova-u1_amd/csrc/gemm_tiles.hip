@@ -238,6 +238,14 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
 
     uint32_t rw[12];  // this lane's pieces, read back from the raw slab (Q8_0 uses 9 dwords)
 
+// One global -> LDS copy request written as the instruction itself: uniform 64-bit base in scalar registers + this
+// lane's 32-bit byte offset, LDS destination base in M0 (one wait state between the scalar write of M0 and the request
+// that reads it).  The builtin gets a 64-bit address per lane and a 64-bit vector add in front of it; the dense form
+// is 7 % faster with this one.  The compiler does not count these requests: every use below is followed by an explicit
+// s_waitcnt vmcnt(0) before the data is read.
+#define SNGGUF_ASM_COPY(INSN, ldsptr_, voff_, sbase_)                                                         \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t" INSN " %1, %2"                                           \
+                 :: "s"((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)(ldsptr_)), "v"(voff_), "s"(sbase_) : "memory", "m0")
 // global -> raw slab, directly: lane l writes its piece into the 16-byte slot l after a uniform base
 // (a 12-byte piece leaves the slot's last dword unwritten); three slots make one row of the slab.
 // Pieces [I0, I1) of step kb.
@@ -253,9 +261,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
         } else {                                                                                             \
             const uint8_t* p_ = scalar_ptr(wbase + (int64_t)((kb) + ks0) * 68);                              \
             _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                           \
-                __builtin_amdgcn_global_load_lds(                                                            \
-                    (const __attribute__((address_space(1))) void*)(p_ + goff[i_]),                          \
-                    (__attribute__((address_space(3))) void*)(raw + 256 * i_), 12, 0, 0);                    \
+                SNGGUF_ASM_COPY("global_load_lds_dwordx3", raw + 256 * i_, goff[i_], p_);                    \
         }                                                                                                    \
     } while (0)
 #define SNGGUF_PICK_W()                                                                                      \
@@ -270,17 +276,13 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
     do {                                                                                                     \
         const uint8_t* xb_ = scalar_ptr(a.x + (int64_t)((kb) + ks0) * TK);                                   \
         _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
-            __builtin_amdgcn_global_load_lds(                                                                \
-                (const __attribute__((address_space(1))) void*)(xb_ + xoff[i_]),                             \
-                (__attribute__((address_space(3))) void*)(xs[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
+            SNGGUF_ASM_COPY("global_load_lds_dwordx4", xs[stage] + (xrow0 + 64 * i_) * 64, xoff[i_], xb_);   \
     } while (0)
 #define SNGGUF_LOAD_WD(kb, stage, I0, I1)                                                                    \
     do {                                                                                                     \
         const uint8_t* wb_ = scalar_ptr(wbase + (int64_t)((kb) + ks0) * (2 * TK));                           \
         _Pragma("unroll") for (int i_ = (I0); i_ < (I1); i_++)                                               \
-            __builtin_amdgcn_global_load_lds(                                                                \
-                (const __attribute__((address_space(1))) void*)(wb_ + woff[i_]),                             \
-                (__attribute__((address_space(3))) void*)(ws[stage] + (xrow0 + 64 * i_) * 64), 16, 0, 0);    \
+            SNGGUF_ASM_COPY("global_load_lds_dwordx4", ws[stage] + (xrow0 + 64 * i_) * 64, woff[i_], wb_);   \
     } while (0)
 // Scales of the 32 elements this thread decodes out of rw (the pieces of step kbn): Q8_0 the block
 // scale copied into both halves of sc_a (first block of a pair: low half of dword 0, second: high
