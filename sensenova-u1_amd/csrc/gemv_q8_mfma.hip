@@ -334,7 +334,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         for (int h = 0; h < NQ; h++) {
             const uint8_t* p = (h ? base2 : base) + (int64_t)t * kSpanBytes + 256 * grp;
 #pragma unroll
-            for (int i = 0; i < 4; i++) dst[h][i] = *reinterpret_cast<const u32x4_t*>(p + goff2[i]);
+            // whole 128-byte lines, each read once by one wavefront: requested with the non-temporal hint, so that the
+            // stream does not displace what the caches hold (2 - 4 % on the gated pair; the block-aligned and K-quant
+            // kernels, which touch a line in two consecutive steps, lose 4 - 6 % with the same hint and do not use it)
+            for (int i = 0; i < 4; i++) dst[h][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p + goff2[i]));
         }
     };
     auto store2 = [&](int grp, const u32x4_t (&src)[NQ][4]) {
