@@ -287,7 +287,9 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
                 for (int e = 0; e < 4; e++)
                     o[e] = pack_bf16(bf16lo_to_f32(rs[e]) + bf16lo_to_f32(o[e]), bf16hi_to_f32(rs[e]) + bf16hi_to_f32(o[e]));
             }
-            *reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n) = o;
+            // written once, read by a later launch at the earliest: stored with the non-temporal hint, so that a round's
+            // 32 MB of output does not displace the operand tiles the next round's workgroups share in L2 (gate shape -3 %)
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n));
         }
         return;
     }

@@ -550,7 +550,7 @@ __global__ __launch_bounds__(512) void gemm_tile_kernel(GemmArgs a) {
                 for (int e = 0; e < 4; e++)
                     o[e] = pack_bf16(bf16lo_to_f32(rs[e]) + bf16lo_to_f32(o[e]), bf16hi_to_f32(rs[e]) + bf16hi_to_f32(o[e]));
             }
-            *reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n) = o;
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(a.y + gr * a.N + n));   // (see gemm_dense4.hip)
         }
         return;
     }

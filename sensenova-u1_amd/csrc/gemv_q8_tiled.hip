@@ -87,8 +87,9 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_tiled_kernel(const bf16_t* 
             const uint8_t* qh = qp + h * pair_delta;
             const uint8_t* sh = sp + h * pair_delta;
 #pragma unroll
-            for (int p = 0; p < 4; p++) wq[buf][h][p] = *reinterpret_cast<const u32x4_t*>(qh + (uint32_t)(run * 4096 + p * 1024));
-            ws[buf][h] = *reinterpret_cast<const u32x4_t*>(sh + (uint32_t)(run * 256));
+            // whole lines, each read once: non-temporal hint (gate/up at M = 1 22.5 -> 21.5 us, down 13.6 -> 13.0 us)
+            for (int p = 0; p < 4; p++) wq[buf][h][p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(qh + (uint32_t)(run * 4096 + p * 1024)));
+            ws[buf][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sh + (uint32_t)(run * 256)));
         }
         if constexpr (!XLDS) {
 #pragma unroll
