@@ -60,7 +60,9 @@ __global__ __launch_bounds__(256) void gemv_bf16_kernel(const bf16_t* __restrict
         for (int64_t e0 = (int64_t)lane * 8; e0 < K; e0 += 64 * 8) {
             u32x4_t w[NW];
 #pragma unroll
-            for (int t = 0; t < NW; t++) w[t] = *reinterpret_cast<const u32x4_t*>(rows[t] + e0);
+            // weight rows are read once, in whole lines: non-temporal hint (12288 x 4096 gated pair at M = 1 39.0 -> 36.5 us,
+            // 4096 x 12288 at M = 4 49.6 -> 40.3 us)
+            for (int t = 0; t < NW; t++) w[t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rows[t] + e0));
 #pragma unroll
             for (int m = 0; m < 16; m++) {
                 if (m < M) {
