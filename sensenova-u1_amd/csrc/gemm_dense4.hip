@@ -1,10 +1,12 @@
 // Dense bf16 GEMM for weights that are already bf16 rows (the second pass of the workspace routes, and plain BF16
 // tensors), four-wavefront form: 256 x 256 output tile per workgroup, K step 64, four wavefronts of 128 (rows) x 128
-// (columns) - 4 x 4 MFMA tiles of 32 x 32, 256 accumulator registers each, one wavefront per SIMD - and two LDS
-// stages of 64 KB.
+// (columns) - 8 x 8 MFMA tiles of 16 x 16 (x 32 of K), 256 accumulator registers each, one wavefront per SIMD - and
+// two LDS stages of 64 KB.  (The 32 x 32 x 16 instruction, with the same tile, the same copies and bit-equal sums,
+// runs the gate shape 7 % slower: it moves half the operand registers per flop but twice the accumulator registers,
+// and the device sustains a lower clock under it.)
 //
-// Against the eight-wavefront form of gemm_tiles.hip (wavefronts of 64 x 128) every wavefront reads 4 + 4 fragments
-// per 16 matrix instructions instead of 2 + 4 per 8: a third fewer LDS bytes per flop.  There the fragment reads and
+// Against the eight-wavefront form of gemm_tiles.hip (wavefronts of 64 x 128) every wavefront reads a third fewer
+// LDS bytes per flop (128 + 128 rows of fragments per 128 x 128 outputs instead of 64 + 128 per 64 x 128).  There the fragment reads and
 // the direct copies together keep the LDS port busy for as long as the matrix instructions take, so neither ever
 // runs at its own rate; here the port has a quarter of its time to spare.  Tile numbering, operand copies (global ->
 // LDS directly, swizzle applied on the global side), barrier placement and epilogues are those of the
@@ -108,18 +110,17 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
     const int xrow0 = 8 * wave;
     const uint8_t* __restrict__ wbase = q + nb0 * row_bytes;
 
-    // fragment reads: row (lane % 32) of a 32-row tile, logical chunk 2 ks + lane / 32
-    int foff[4];
+    // fragment reads: row (lane % 16) of a 16-row tile, logical chunk 4 ks + lane / 16 (ks: the two 32-element halves
+    // of a K step)
+    int foff[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) foff[ks] = (lane & 31) * 64 + 8 * ((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7));
+    for (int ks = 0; ks < 2; ks++) foff[ks] = (lane & 15) * 64 + 8 * ((4 * ks + (lane >> 4)) ^ ((lane >> 1) & 7));
 
-    f32x16_t acc[4][4];  // [weight-row tile i][activation-row tile j]
+    f32x4_t acc[8][8];  // [weight-row tile i][activation-row tile j]
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < 8; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+        for (int j = 0; j < 8; j++) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
 // Base pointers of the copies of K step kb (clamped to the last step: the loop below requests one and two steps
 // ahead without asking whether they exist; a repeated last step lands in a stage nobody reads any more).
@@ -136,56 +137,53 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
 #define SNGGUF_COPY1(base_, off_, tile_, i_)                                                                 \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"                             \
                  :: "s"(lds_offset((tile_) + (xrow0 + 32 * (i_)) * 64)), "v"((off_)[i_]), "s"(base_) : "memory", "m0")
-// fragment f (0..3 weight tiles, 4..7 activation tiles) of slice ks_ of a stage
+// fragment f (0..7 weight tiles, 8..15 activation tiles) of half ks_ of a stage
 #define SNGGUF_FRAG1(stage, ks_, buf, f)                                                                     \
     do {                                                                                                     \
-        if ((f) < 4) af_[buf][(f) & 3] = *reinterpret_cast<const bf16x8_t*>(ws[stage] + wn * 128 * 64 + ((f) & 3) * 32 * 64 + foff[ks_]); \
-        else bf_[buf][(f) & 3] = *reinterpret_cast<const bf16x8_t*>(xs[stage] + wm * 128 * 64 + ((f) & 3) * 32 * 64 + foff[ks_]);         \
+        if ((f) < 8) af_[buf][(f) & 7] = *reinterpret_cast<const bf16x8_t*>(ws[stage] + wn * 128 * 64 + ((f) & 7) * 16 * 64 + foff[ks_]); \
+        else bf_[buf][(f) & 7] = *reinterpret_cast<const bf16x8_t*>(xs[stage] + wm * 128 * 64 + ((f) & 7) * 16 * 64 + foff[ks_]);         \
     } while (0)
-// One K step on stage CUR, written out instruction group by instruction group with a scheduling fence after each:
-// a lone wavefront per SIMD issues in order, so what sits between two matrix instructions decides whether the
-// matrix pipe runs dry.  Every matrix instruction is followed by at most one fragment read (those of the next slice,
-// under the first eight of a slice's sixteen) and, in the two slices that carry copies, every second one by one
-// copy request - a burst of requests that filled the memory pipeline's queue would hold up the matrix instructions
-// behind it.  The workgroup's one barrier per step sits in front of the last slice: by then every wavefront holds
-// that slice's fragments in registers, so stage CUR is free, and the copies into the other stage - requested behind
-// the previous barrier and in this step's first slice - have had most of a step to arrive.  Half of the copies of
-// step kb + 2 go into stage CUR behind the barrier, the other half in the first slice of the next step.
-#define SNGGUF_K_STEP4(kb, CUR)                                                                              \
-    do {                                                                                                     \
-        SNGGUF_STEP_BASE((kb) + 1, xb1_, wb1_);                                                              \
-        SNGGUF_STEP_BASE((kb) + 2, xb2_, wb2_);                                                              \
-        _Pragma("unroll") for (int ks = 0; ks < 4; ks++) {                                                   \
-            if (ks == 3) {                                                                                   \
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                  \
-                __syncthreads();                                                                             \
-            }                                                                                                \
-            _Pragma("unroll") for (int m = 0; m < 16; m++) {                                                 \
-                acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[ks & 1][m >> 2], bf_[ks & 1][m & 3], \
-                                                                             acc[m >> 2][m & 3], 0, 0, 0);   \
-                if (m < 8) {                                                                                 \
-                    if (ks < 3) SNGGUF_FRAG1(CUR, (ks + 1) & 3, (ks + 1) & 1, m);                            \
-                    else SNGGUF_FRAG1((CUR) ^ 1, 0, 0, m);                                                   \
-                }                                                                                            \
-                if (m & 1) {                                                                                 \
-                    const int c = m >> 1;                                                                    \
-                    if (ks == 0) {                                                                           \
-                        if (c < 4) SNGGUF_COPY1(wb1_, woff, ws[(CUR) ^ 1], 4 + (c & 3));                     \
-                        else SNGGUF_COPY1(xb1_, xoff, xs[(CUR) ^ 1], 4 + (c & 3));                           \
-                    }                                                                                        \
-                    if (ks == 3) {                                                                           \
-                        if (c < 4) SNGGUF_COPY1(wb2_, woff, ws[CUR], c & 3);                                 \
-                        else SNGGUF_COPY1(xb2_, xoff, xs[CUR], c & 3);                                       \
-                    }                                                                                        \
-                }                                                                                            \
-                __builtin_amdgcn_sched_barrier(0);                                                           \
-            }                                                                                                \
-        }                                                                                                    \
+// One K step on stage CUR: 128 matrix instructions (two halves of 32 elements of K, 8 x 8 tiles each), written out
+// instruction group by instruction group with a scheduling fence after each - a lone wavefront per SIMD issues in
+// order, so what sits between two matrix instructions decides whether the matrix pipe runs dry.  Every half reads
+// the 16 fragments of the next half under its first 32 matrix instructions (one read per two).  The workgroup's one
+// barrier per step sits behind the first 32: by then every wavefront holds the fragments of both halves in
+// registers, so stage CUR is free, and the copies into the other stage have been on their way since the previous
+// step's barrier.  The 16 copies of step kb + 2 go into stage CUR behind the barrier, one per six matrix
+// instructions, which spreads them over the rest of the step: requests closer together fill the memory pipeline's
+// queue and hold up the matrix instructions behind them (gate shape, one copy per 2 / 4 / 6 matrix instructions:
+// 360 / 343 / 336 us in one run; copies behind a barrier between the halves, one per 4: 344 us).
+constexpr int kBarrierAt = 32, kCopyEvery = 6, kFragEvery = 2;
+static_assert(kBarrierAt > 15 * kFragEvery && kBarrierAt <= 64 && kBarrierAt + 16 * kCopyEvery <= 128, "placement");
+#define SNGGUF_K_STEP4(kb, CUR)                                                                                      \
+    do {                                                                                                             \
+        SNGGUF_STEP_BASE((kb) + 2, xb2_, wb2_);                                                                      \
+        _Pragma("unroll") for (int q = 0; q < 128; q++) {                                                            \
+            const int ks = q >> 6, m = q & 63;                                                                       \
+            if (q == kBarrierAt) {                                                                                   \
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                          \
+                __syncthreads();                                                                                     \
+            }                                                                                                        \
+            acc[m >> 3][m & 7] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af_[ks][m >> 3], bf_[ks][m & 7],            \
+                                                                         acc[m >> 3][m & 7], 0, 0, 0);               \
+            if (m < 16 * kFragEvery && (m % kFragEvery) == 0) {                                                      \
+                /* activation fragments first: the next half's first eight matrix instructions need all */           \
+                const int f = m / kFragEvery < 8 ? 8 + m / kFragEvery : m / kFragEvery - 8;                          \
+                if (ks == 0) SNGGUF_FRAG1(CUR, 1, 1, f);                                                             \
+                else SNGGUF_FRAG1((CUR) ^ 1, 0, 0, f);                                                               \
+            }                                                                                                        \
+            if (q >= kBarrierAt && ((q - kBarrierAt) % kCopyEvery) == kCopyEvery - 1 && (q - kBarrierAt) / kCopyEvery < 16) { \
+                const int c = (q - kBarrierAt) / kCopyEvery;                                                         \
+                if (c < 8) SNGGUF_COPY1(wb2_, woff, ws[CUR], c & 7);                                                 \
+                else SNGGUF_COPY1(xb2_, xoff, xs[CUR], c & 7);                                                       \
+            }                                                                                                        \
+            __builtin_amdgcn_sched_barrier(0);                                                                       \
+        }                                                                                                            \
     } while (0)
 
     {
         // the launcher sends only even numbers of K steps here: the loop has one body and the accumulators one home
-        bf16x8_t af_[2][4], bf_[2][4];
+        bf16x8_t af_[2][8], bf_[2][8];
         {
             SNGGUF_STEP_BASE(0, xb0_, wb0_);
             SNGGUF_STEP_BASE(1, xb1_, wb1_);
@@ -195,7 +193,7 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
                 SNGGUF_COPY1(wb0_, woff, ws[0], i);
             }
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < 8; i++) {
                 SNGGUF_COPY1(xb1_, xoff, xs[1], i);
                 SNGGUF_COPY1(wb1_, woff, ws[1], i);
             }
@@ -203,7 +201,7 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
 #pragma unroll
-        for (int f = 0; f < 8; f++) SNGGUF_FRAG1(0, 0, 0, f);
+        for (int f = 0; f < 16; f++) SNGGUF_FRAG1(0, 0, 0, f);
         for (int kd = 0; kd < ksteps; kd += 2) {
             SNGGUF_K_STEP4(kd, 0);
             SNGGUF_K_STEP4(kd + 1, 1);
@@ -218,32 +216,29 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
 #undef SNGGUF_STEP_BASE
 
     // ---- epilogue: D[i][j], i = weight row (n), j = activation row (m) ----------------------------------------
-    // lane: j = lane % 32; register v: i = 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    // lane: j = lane % 16; register v: i = 4 * (lane / 16) + v
     if constexpr (EP == 1) {
         // K split over workgroups: this slice's sums go out as fp32, to be added up by the split-K reduction
         float* part = a.partial + (int64_t)slice * a.M * a.N;
         const bool vec = (a.N & 3) == 0;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < 8; i++) {
+            const int64_t n = nb0 + wn * 128 + i * 16 + 4 * (lane >> 4);
 #pragma unroll
-            for (int vg = 0; vg < 4; vg++) {
-                const int64_t n = nb0 + wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
+            for (int j = 0; j < 8; j++) {
+                const int64_t rr = row_begin + wm * 128 + j * 16 + (lane & 15);
+                if (rr >= row_end || n >= a.N) continue;
+                const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+                float* pp = part + gr * a.N + n;
+                if (vec) {
+                    *reinterpret_cast<f32x4_t*>(pp) = acc[i][j];
+                } else {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const int64_t rr = row_begin + wm * 128 + j * 32 + (lane & 31);
-                    if (rr >= row_end || n >= a.N) continue;
-                    const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-                    float* pp = part + gr * a.N + n;
-                    if (vec) {
-                        *reinterpret_cast<f32x4_t*>(pp) = f32x4_t{acc[i][j][4 * vg], acc[i][j][4 * vg + 1], acc[i][j][4 * vg + 2], acc[i][j][4 * vg + 3]};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (n + e < a.N) pp[e] = acc[i][j][4 * vg + e];
-                    }
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < a.N) pp[e] = acc[i][j][e];
                 }
-                __builtin_amdgcn_sched_barrier(0);  // one group of accumulators at a time: they live in accumulation registers
             }
+            __builtin_amdgcn_sched_barrier(0);  // one group of accumulators at a time: they live in accumulation registers
         }
         return;
     }
@@ -251,23 +246,23 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
         // Rows of y are 16-byte aligned: stage the tile in LDS as bf16 [256 m][256 n] (the K-loop buffers are dead:
         // nothing reads them after the last barrier) and write it out as 16-byte pieces, 32 lanes along one output row.
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < 8; i++) {
+            // (an empty statement that wants this row of tiles in accumulation registers: without it the compiler moves
+            // all 256 accumulators into vector registers at the loop's exit and runs out of them)
 #pragma unroll
-            for (int vg = 0; vg < 4; vg++) {
-                const int nl = wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
-                float b[4] = {0.f, 0.f, 0.f, 0.f};
-                if (bias && nb0 + nl < a.N) {
+            for (int j = 0; j < 8; j++) asm volatile("" : "+a"(acc[i][j]));
+            const int nl = wn * 128 + i * 16 + 4 * (lane >> 4);
+            float b[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias && nb0 + nl < a.N) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) b[e] = bf16_to_f32(bias[nb0 + nl + e]);
-                }
+                for (int e = 0; e < 4; e++) b[e] = bf16_to_f32(bias[nb0 + nl + e]);
+            }
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const int ml = wm * 128 + j * 32 + (lane & 31);
-                    *reinterpret_cast<u32x2_t*>(lds + ml * kYRow + 2 * nl) =
-                        u32x2_t{pack_bf16(acc[i][j][4 * vg] + b[0], acc[i][j][4 * vg + 1] + b[1]),
-                                pack_bf16(acc[i][j][4 * vg + 2] + b[2], acc[i][j][4 * vg + 3] + b[3])};
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int j = 0; j < 8; j++) {
+                const int ml = wm * 128 + j * 16 + (lane & 15);
+                *reinterpret_cast<u32x2_t*>(lds + ml * kYRow + 2 * nl) =
+                    u32x2_t{pack_bf16(acc[i][j][0] + b[0], acc[i][j][1] + b[1]), pack_bf16(acc[i][j][2] + b[2], acc[i][j][3] + b[3])};
+                if (j & 1) __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();
@@ -295,35 +290,34 @@ __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
     }
     const bool fast = (a.N & 3) == 0;  // rows of y are 8-byte aligned and a run of four columns never straddles N
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < 8; i++) {
 #pragma unroll
-        for (int vg = 0; vg < 4; vg++) {
-            const int64_t n = nb0 + wn * 128 + i * 32 + 8 * vg + 4 * (lane >> 5);
-            float b[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
+        for (int j = 0; j < 8; j++) asm volatile("" : "+a"(acc[i][j]));  // as above: one row of tiles at a time
+        const int64_t n = nb0 + wn * 128 + i * 16 + 4 * (lane >> 4);
+        float b[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (n + e < a.N) b[e] = bf16_to_f32(bias[n + e]);
-            }
+            for (int e = 0; e < 4; e++)
+                if (n + e < a.N) b[e] = bf16_to_f32(bias[n + e]);
+        }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int64_t rr = row_begin + wm * 128 + j * 32 + (lane & 31);
-                if (rr >= row_end || n >= a.N) continue;
-                const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
-                bf16_t* yp = a.y + gr * a.N + n;
-                const int64_t yi = gr * a.N + n;
-                const float o0 = add_residual(acc[i][j][4 * vg] + b[0], a.residual, yi);
-                const float o1 = n + 1 < a.N ? add_residual(acc[i][j][4 * vg + 1] + b[1], a.residual, yi + 1) : 0.f;
-                const float o2 = n + 2 < a.N ? add_residual(acc[i][j][4 * vg + 2] + b[2], a.residual, yi + 2) : 0.f;
-                const float o3 = n + 3 < a.N ? add_residual(acc[i][j][4 * vg + 3] + b[3], a.residual, yi + 3) : 0.f;
-                if (fast) {
-                    *reinterpret_cast<u32x2_t*>(yp) = u32x2_t{pack_bf16(o0, o1), pack_bf16(o2, o3)};
-                } else {
-                    yp[0] = f32_to_bf16(o0);
-                    if (n + 1 < a.N) yp[1] = f32_to_bf16(o1);
-                    if (n + 2 < a.N) yp[2] = f32_to_bf16(o2);
-                    if (n + 3 < a.N) yp[3] = f32_to_bf16(o3);
-                }
+        for (int j = 0; j < 8; j++) {
+            const int64_t rr = row_begin + wm * 128 + j * 16 + (lane & 15);
+            if (rr >= row_end || n >= a.N) continue;
+            const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+            bf16_t* yp = a.y + gr * a.N + n;
+            const int64_t yi = gr * a.N + n;
+            const float o0 = add_residual(acc[i][j][0] + b[0], a.residual, yi);
+            const float o1 = n + 1 < a.N ? add_residual(acc[i][j][1] + b[1], a.residual, yi + 1) : 0.f;
+            const float o2 = n + 2 < a.N ? add_residual(acc[i][j][2] + b[2], a.residual, yi + 2) : 0.f;
+            const float o3 = n + 3 < a.N ? add_residual(acc[i][j][3] + b[3], a.residual, yi + 3) : 0.f;
+            if (fast) {
+                *reinterpret_cast<u32x2_t*>(yp) = u32x2_t{pack_bf16(o0, o1), pack_bf16(o2, o3)};
+            } else {
+                yp[0] = f32_to_bf16(o0);
+                if (n + 1 < a.N) yp[1] = f32_to_bf16(o1);
+                if (n + 2 < a.N) yp[2] = f32_to_bf16(o2);
+                if (n + 3 < a.N) yp[3] = f32_to_bf16(o3);
             }
         }
     }
