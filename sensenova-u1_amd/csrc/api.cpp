@@ -254,7 +254,10 @@ int linear_ws_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N
     // workspace is that large.
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
     const int64_t ksteps = K / 64;
-    const bool tile_type = qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K;
+    // (from 4096 rows on the weight pass pays for itself even here: a K step of the dense kernel takes 1.4 us against 2.0 us
+    // with the decode in the loop, and sixteen row tiles share one pass - 4096 x 1024 <- 4096: 56 against 61 us, 2048 wide
+    // 80 against 92 us; at 512 rows the pass costs more than it saves, 48 against 44 us on 4096 x 4096)
+    const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K) && M < 4096;
     const int64_t dense_bytes = tile_type ? 0 : 2 * N * K;
     if (tiles <= 128 && workspace_bytes > dense_bytes) {
         const int64_t room = (workspace_bytes - dense_bytes) / (4 * M * N);

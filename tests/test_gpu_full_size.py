@@ -88,6 +88,27 @@ def test_k_quant_mix_at_full_size(dev, qt, n, k):
         _sample_check(y2, x, packed, qt, gen, f"linear_ws qt={qt} m={m}")
 
 
+@pytest.mark.parametrize("qt", [go.Q8_0, go.Q4_K])
+def test_narrow_projection_over_image_rows_with_room_for_a_k_split(dev, qt):
+    """k / v of the generation tower (4096 -> 1024 at M = 4096: 64 output tiles) with a workspace that has room for fp32
+    partial sums behind the decoded weight, as the module's pooled workspace has: weight pass + dense kernel with K split
+    over workgroups.  The same call with the minimal workspace (no room: no split) must give the same sampled values."""
+    n, k, m = 1024, 4096, 4096
+    gen = torch.Generator().manual_seed(13 + qt)
+    packed = synthetic.make_packed(qt, n, k, seed=44, device=dev)
+    x = synthetic.make_activations(m, k, seed=61, device=dev)
+    bias = synthetic.make_activations(1, n, seed=62, device=dev).reshape(n)
+    outs = []
+    for extra in (0, 4 * 4 * m * n):
+        print(f"case full narrow qt={qt} extra workspace {extra}", flush=True)
+        ws = torch.empty(ops.linear_workspace_bytes(n, k) + extra, dtype=torch.uint8, device=dev)
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.linear_ws_into(x, packed, qt, bias, y, ws, ops.NUM_UPSTREAM_FP16)
+        _sample_check(y, x, packed, qt, gen, f"narrow qt={qt} extra={extra}", bias=bias)
+        outs.append(y)
+    assert go.rel_l2(outs[1].cpu(), outs[0].cpu()) <= 1e-4   # same bf16 weights; only the order of the fp32 sums differs
+
+
 def test_q8_0_down_projection_with_residual_at_decode(dev):
     """down_proj 12288 -> 4096 with the residual add in the epilogue, M = 1, 4, 16."""
     n, k = 4096, 12288
