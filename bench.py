@@ -618,6 +618,30 @@ def main() -> None:
         wall_st, _ = run_region(tower_stacked, gs, args.gemm_warmup)
         wall_st_ws, _ = run_region(tower_stacked_ws, gs, args.gemm_warmup)
         del qkv, y_qkv
+        # gate / up / SiLU as Qwen3MLP.forward asks for them at M = 4096: one gated launch of the dense kernel behind the
+        # two weight passes (what modality.gated_mlp runs from 2048 rows on) against two workspace launches and the
+        # elementwise product on bf16 tensors
+        gated = {}
+        for mg in (4096, 2048):
+            xg = xs[HIDDEN][:mg]
+            hg = torch.empty((mg, INTER), dtype=torch.bfloat16, device=dev)
+            y_up = torch.empty((mg, INTER), dtype=torch.bfloat16, device=dev)
+            ws_g = torch.empty(ops.gate_up_silu_workspace_bytes(INTER, HIDDEN), dtype=torch.uint8, device=dev)
+
+            def gated_fused(i):
+                ops.gate_up_silu_ws_into(xg, tower[i % 2][4], tower[i % 2][5], Q8_0, hg, ws_g, num)
+
+            def gated_separate(i):
+                ops.linear_ws_into(xg, tower[i % 2][4], Q8_0, None, ys[INTER][:mg], wtmp, num)
+                ops.linear_ws_into(xg, tower[i % 2][5], Q8_0, None, y_up, wtmp, num)
+                torch.mul(torch.nn.functional.silu(ys[INTER][:mg]), y_up, out=hg)
+
+            _, e_f = run_region(gated_fused, gs * 2, args.gemm_warmup)
+            _, e_s = run_region(gated_separate, gs * 2, args.gemm_warmup)
+            gated[f"M{mg}"] = {"one_gated_launch_us": round(e_f / (gs * 2) * 1e3, 1),
+                               "two_launches_and_product_us": round(e_s / (gs * 2) * 1e3, 1),
+                               "tflops": round(4.0 * mg * INTER * HIDDEN / (e_f / (gs * 2) * 1e-3) / 1e12, 1)}
+            del hg, y_up, ws_g
         gate_flop = 2.0 * m * INTER * HIDDEN
         gate_tflops = gate_flop / (gate_ms * 1e-3) / 1e12
         dense_tflops = gate_flop / (dense_ms * 1e-3) / 1e12
@@ -626,7 +650,7 @@ def main() -> None:
             "workload": "configs[2]: Q8_0 generation-tower projections over M=4096 image tokens "
                         "(q,o 4096^2; k,v 4096->1024; gate/up 4096->12288; down 12288->4096), seven separate linears",
             "route": "sngguf_linear_ws (what GGUFLinear.forward does beyond 64 rows): weight pass into a pooled bf16 "
-                     "workspace + the library's dense tile kernel; k / v (64 tiles) stay on the fused tile kernel",
+                     "workspace + the library's dense tile kernel; k / v (64 tiles) with K split four ways over workgroups",
             "value": round(tflops_ws, 2),
             "unit": "TFLOP/s",
             "steps": gs,
@@ -679,6 +703,12 @@ def main() -> None:
                 "workspace_value": round(flops / (wall_st_ws / gs * 1e-3) / 1e12, 2),
                 "workspace_ms_per_step": round(wall_st_ws / gs, 4),
                 "workspace_pct_of_bf16_mfma_peak": round(100 * flops / (wall_st_ws / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+            },
+            "gated_pair": {
+                "what": "silu(gate_proj(x)) * up_proj(x), 4096 -> 12288: sngguf_gate_up_silu_ws (two weight passes into one "
+                        "interleaved workspace + ONE dense launch with the gated epilogue; the projection outputs are never "
+                        "written) against sngguf_linear_ws twice + the product on bf16 tensors",
+                **gated,
             },
             "mid_rows": {
                 "what": "one projection at 128 and 512 rows (q 4096^2, k 4096->1024, gate 4096->12288, down 12288->4096): "

@@ -197,6 +197,27 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
                         int64_t N, int64_t K, void* h, int numerics, void* stream);
 
 /*
+ * The same pair beyond decode sizes (the generation tower's thousands of image rows through Qwen3MLP.forward,
+ * modeling_qwen3.py:214-216): one weight pass per matrix into the workspace - bf16 rows, the two matrices interleaved
+ * in blocks of 128 rows - and ONE launch of the dense tile kernel whose epilogue rounds the gate and the up sums to
+ * bf16, applies silu and multiplies, with the roundings above.  The two [M][N] projection outputs are never written
+ * and no elementwise pass reads them back.  Same values as sngguf_linear_ws on each matrix followed by
+ * silu(gate) * up on bf16 tensors (up to the last place of exp()).
+ *  workspace   device scratch of at least sngguf_gate_up_silu_workspace_bytes(N, K) = 512 ceil(N / 128) K bytes,
+ *              16-byte aligned; nothing in it outlives the call
+ *  M <= 16 runs sngguf_gate_up_silu (the workspace is not touched).  Otherwise the shape must satisfy
+ *  sngguf_gate_up_silu_ws_fits(qtype, M, N, K) (M >= 17, K % 128 == 0, N % 8 == 0, M K < 2^31, a packed block
+ *  format), else SNGGUF_E_BADSHAPE / SNGGUF_E_BADTYPE and the caller runs the two projections separately.  It
+ *  pays from about 1024 rows on (a launch has 2 N / 256 x M / 256 tiles and there is no K split; 12288 x 4096 at
+ *  4096 rows: 628 us against 695 us for two sngguf_linear_ws launches and the product, at 2048 rows 354 against 451).
+ */
+int64_t sngguf_gate_up_silu_workspace_bytes(int64_t N, int64_t K);
+int sngguf_gate_up_silu_ws_fits(int qtype, int64_t M, int64_t N, int64_t K);
+int sngguf_gate_up_silu_ws(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype,
+                           int64_t N, int64_t K, void* h, void* workspace, int64_t workspace_bytes,
+                           int numerics, void* stream);
+
+/*
  * RMSNorm fused in front of a decode projection.  In the decoder layer the q / k / v projections read
  * input_layernorm(hidden) and gate / up read post_attention_layernorm(hidden)
  * (src/sensenova_u1/models/neo_unify/modeling_qwen3.py:919, :938; Qwen3RMSNorm.forward at :192-197):

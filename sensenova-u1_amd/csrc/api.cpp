@@ -33,6 +33,9 @@ int launch_gemm_splitk(const void* x, int64_t M, const void* q, int qtype, int64
                        float* partial, int slices, int numerics, hipStream_t stream);
 int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_t K, const void* bias, void* y,
                       hipStream_t stream);
+int launch_dequantize_interleaved(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int second, int numerics,
+                                  hipStream_t stream);
+int launch_gemm_dense_gated(const void* x, int64_t M, const void* w2, int64_t cols, int64_t K, void* h, hipStream_t stream);
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
                 const void* residual, void* y,
                 int numerics, hipStream_t stream);
@@ -309,6 +312,34 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
     if (qtype == SNGGUF_TYPE_BF16)
         return sngguf::launch_gemv_bf16(x, M, q_gate, q_up, N, K, nullptr, nullptr, h, true, static_cast<hipStream_t>(stream));
     return sngguf::launch_gemv(x, M, q_gate, q_up, qtype, N, K, nullptr, nullptr, h, numerics, true, static_cast<hipStream_t>(stream));
+}
+
+int64_t sngguf_gate_up_silu_workspace_bytes(int64_t N, int64_t K) {
+    return N > 0 && K > 0 && N < kMaxDim && K < kMaxDim ? 2 * 256 * ((N + 127) / 128) * K : 0;
+}
+
+int sngguf_gate_up_silu_ws_fits(int qtype, int64_t M, int64_t N, int64_t K) {
+    // the dense kernel's gated epilogue: whole pairs of K steps, output rows of whole 16-byte pieces, 32-bit activation
+    // offsets; packed block formats only (plain BF16 rows are not interleaved by a weight pass)
+    return known_type(qtype) && qtype != SNGGUF_TYPE_BF16 && M >= 17 && M < kMaxDim && N > 0 && N < kMaxDim && K > 0 &&
+           K < kMaxDim && K % 128 == 0 && K % sngguf_block_size(qtype) == 0 && N % 8 == 0 && M * K < ((int64_t)1 << 31);
+}
+
+int sngguf_gate_up_silu_ws(const void* x, int64_t M, const void* q_gate, const void* q_up, int qtype, int64_t N, int64_t K,
+                           void* h, void* workspace, int64_t workspace_bytes, int numerics, void* stream) {
+    if (M >= 0 && M <= 16) return sngguf_gate_up_silu(x, M, q_gate, q_up, qtype, N, K, h, numerics, stream);
+    const int rc = check_matmul(x, M, q_gate, qtype, N, K, h, numerics);
+    if (rc != SNGGUF_OK || N == 0) return rc;
+    if (!q_up || !workspace) return SNGGUF_E_NULLPTR;
+    if (!aligned(q_up, 16) || !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
+    if (!sngguf_gate_up_silu_ws_fits(qtype, M, N, K)) return qtype == SNGGUF_TYPE_BF16 ? SNGGUF_E_BADTYPE : SNGGUF_E_BADSHAPE;
+    if (workspace_bytes < sngguf_gate_up_silu_workspace_bytes(N, K)) return SNGGUF_E_BADSHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rd = sngguf::launch_dequantize_interleaved(q_gate, qtype, N, K, workspace, 0, numerics, s);
+    if (rd != SNGGUF_OK) return rd;
+    rd = sngguf::launch_dequantize_interleaved(q_up, qtype, N, K, workspace, 1, numerics, s);
+    if (rd != SNGGUF_OK) return rd;
+    return sngguf::launch_gemm_dense_gated(x, M, workspace, N, K, h, s);
 }
 
 int64_t sngguf_lm_head_argmax_workspace_bytes(int64_t M, int64_t N) {

@@ -100,30 +100,35 @@ __device__ __forceinline__ void dequantize8(const uint8_t* __restrict__ row, int
 }
 
 // WIDE: the number of 8-element groups does not fit 32 bits (the index arithmetic then needs 64-bit divisions).
+// Row r of the input is written to output row r + ((r >> spread) << spread) + first: with spread = 63 and first = 0
+// that is row r; with spread = 7 the rows go out in blocks of 128 that leave 128 rows free behind each block (first = 0)
+// or fill those (first = 128) - two matrices interleaved in blocks of 128 rows.
 template <int QT, int NUM, int OUT, bool WIDE>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ q, int64_t rows, int64_t cols,
-                                                         int64_t row_bytes, void* __restrict__ out) {
+                                                         int64_t row_bytes, void* __restrict__ out, int spread, int64_t first) {
     const int64_t groups_per_row = cols >> 3;
     const int64_t total = rows * groups_per_row;
     if constexpr (WIDE) {
         for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (int64_t)gridDim.x * blockDim.x) {
             const int64_t r = g / groups_per_row;
             const int64_t e0 = (g - r * groups_per_row) << 3;
-            dequantize8<QT, NUM, OUT>(q + r * row_bytes, e0, out, r * cols + e0);
+            dequantize8<QT, NUM, OUT>(q + r * row_bytes, e0, out, (r + ((r >> spread) << spread) + first) * cols + e0);
         }
     } else {
         const uint32_t gpr = (uint32_t)groups_per_row, tot = (uint32_t)total, stride = gridDim.x * blockDim.x;
         for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < tot; g += stride) {
             const uint32_t r = g / gpr;
             const int64_t e0 = (int64_t)(g - r * gpr) << 3;
-            dequantize8<QT, NUM, OUT>(q + (int64_t)r * row_bytes, e0, out, (int64_t)r * cols + e0);
+            const int64_t ro = (int64_t)r + (((int64_t)r >> spread) << spread) + first;
+            dequantize8<QT, NUM, OUT>(q + (int64_t)r * row_bytes, e0, out, ro * cols + e0);
             if (g + stride < g) break;   // the next index would wrap
         }
     }
 }
 
 template <int QT, int NUM>
-static int launch_out(const uint8_t* q, int64_t rows, int64_t cols, void* out, int out_dtype, hipStream_t stream) {
+static int launch_out(const uint8_t* q, int64_t rows, int64_t cols, void* out, int out_dtype, hipStream_t stream,
+                      int spread, int64_t first) {
     const int64_t row_bytes = cols / Fmt<QT>::bs * Fmt<QT>::ts;
     const int64_t total = rows * (cols >> 3);
     if (total == 0) return SNGGUF_OK;
@@ -133,8 +138,8 @@ static int launch_out(const uint8_t* q, int64_t rows, int64_t cols, void* out, i
     const bool wide = total >= ((int64_t)1 << 32);
 #define SNGGUF_DEQ(OUT) \
     do { \
-        if (wide) dequantize_kernel<QT, NUM, OUT, true><<<grid, block, 0, stream>>>(q, rows, cols, row_bytes, out); \
-        else dequantize_kernel<QT, NUM, OUT, false><<<grid, block, 0, stream>>>(q, rows, cols, row_bytes, out); \
+        if (wide) dequantize_kernel<QT, NUM, OUT, true><<<grid, block, 0, stream>>>(q, rows, cols, row_bytes, out, spread, first); \
+        else dequantize_kernel<QT, NUM, OUT, false><<<grid, block, 0, stream>>>(q, rows, cols, row_bytes, out, spread, first); \
     } while (0)
     switch (out_dtype) {
     case SNGGUF_OUT_F32: SNGGUF_DEQ(SNGGUF_OUT_F32); break;
@@ -147,16 +152,28 @@ static int launch_out(const uint8_t* q, int64_t rows, int64_t cols, void* out, i
 }
 
 template <int QT>
-static int launch_num(const uint8_t* q, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics, hipStream_t stream) {
-    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_out<QT, SNGGUF_NUM_GGML_FP32>(q, rows, cols, out, out_dtype, stream);
-    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_out<QT, SNGGUF_NUM_UPSTREAM_FP16>(q, rows, cols, out, out_dtype, stream);
+static int launch_num(const uint8_t* q, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics, hipStream_t stream,
+                      int spread, int64_t first) {
+    if (numerics == SNGGUF_NUM_GGML_FP32) return launch_out<QT, SNGGUF_NUM_GGML_FP32>(q, rows, cols, out, out_dtype, stream, spread, first);
+    if (numerics == SNGGUF_NUM_UPSTREAM_FP16) return launch_out<QT, SNGGUF_NUM_UPSTREAM_FP16>(q, rows, cols, out, out_dtype, stream, spread, first);
     return SNGGUF_E_BADTYPE;
 }
 
 int launch_dequantize(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int out_dtype, int numerics,
                       hipStream_t stream) {
     const uint8_t* p = static_cast<const uint8_t*>(q);
-#define SNGGUF_CALL(QT) launch_num<QT>(p, rows, cols, out, out_dtype, numerics, stream)
+#define SNGGUF_CALL(QT) launch_num<QT>(p, rows, cols, out, out_dtype, numerics, stream, 63, 0)
+    SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
+#undef SNGGUF_CALL
+}
+
+// The bf16 rows of one of two matrices that share an output in blocks of 128 rows: input row r goes to output row
+// 256 (r / 128) + r % 128 (+ 128 for the second matrix).  What the gated dense GEMM reads: each of its 256-row weight
+// tiles then holds 128 gate rows and the 128 up rows of the same output columns.
+int launch_dequantize_interleaved(const void* q, int qtype, int64_t rows, int64_t cols, void* out, int second, int numerics,
+                                  hipStream_t stream) {
+    const uint8_t* p = static_cast<const uint8_t*>(q);
+#define SNGGUF_CALL(QT) launch_num<QT>(p, rows, cols, out, SNGGUF_OUT_BF16, numerics, stream, 7, second ? 128 : 0)
     SNGGUF_DISPATCH_TYPE(qtype, SNGGUF_CALL)
 #undef SNGGUF_CALL
 }

@@ -261,6 +261,24 @@ int launch_gemm_dense(const void* x, int64_t M, const void* w, int64_t N, int64_
     return launch_gemm_tiles(a, 30, SNGGUF_NUM_GGML_FP32, stream);
 }
 
+int launch_gemm_dense4(const GemmArgs& a, hipStream_t stream);
+
+// h = silu(x wg^T) * (x wu^T) with both weights already bf16 and interleaved in blocks of 128 rows (w2: rows2 =
+// 256 ceil(cols / 128) rows of K, as launch_dequantize_interleaved writes them): one launch of the four-wavefront dense
+// kernel with the gated epilogue.  Needs K % 128 == 0 (an even number of K steps), cols % 8 == 0 and M K < 2^31
+// (checked by the caller).
+int launch_gemm_dense_gated(const void* x, int64_t M, const void* w2, int64_t cols, int64_t K, void* h, hipStream_t stream) {
+    GemmArgs a{};
+    a.x = static_cast<const bf16_t*>(x);
+    a.y = static_cast<bf16_t*>(h);
+    a.M = M; a.N = 256 * ((cols + 127) / 128); a.K = K;
+    a.rowmap = nullptr; a.n0_dev = nullptr; a.n0 = M;
+    a.q[0] = a.q[1] = static_cast<const uint8_t*>(w2);
+    a.group_mask = 1;
+    a.gated_cols = cols;
+    return launch_gemm_dense4(a, stream);
+}
+
 int launch_splitk_reduce(const GemmArgs& a, const uint8_t* indicator, int64_t n_text, hipStream_t stream);
 
 // y = x W^T (+ bias) on the large-tile kernel with K split over `slices` workgroups per output tile: fp32 partial

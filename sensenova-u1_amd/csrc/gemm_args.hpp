@@ -24,6 +24,10 @@ struct GemmArgs {
     // (no bias, no residual, nothing written to y); a second kernel adds the slices up.
     float* partial;
     int ksplit;
+    // Gated pair (four-wavefront dense kernel only): the N weight rows are blocks of 128 gate rows, each followed by the
+    // 128 up rows of the same output columns, and y is [M][gated_cols]: silu(gate) * up, rounded as the decode kernels'
+    // gated pair rounds (no bias, no residual, no K split).  0 = a plain projection.
+    int64_t gated_cols;
 };
 
 }  // namespace sngguf

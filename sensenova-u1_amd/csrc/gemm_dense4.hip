@@ -40,7 +40,8 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
 
 // EP: which epilogue this instance carries (one per instance, so that the 256 accumulators of a lane are read out of
 // their accumulation registers group by group on one path instead of all at once in front of a three-way branch):
-// 0 = bf16 tile staged through LDS (N % 8 == 0), 1 = fp32 partial sums of a K slice, 2 = direct stores (any N).
+// 0 = bf16 tile staged through LDS (N % 8 == 0), 1 = fp32 partial sums of a K slice, 2 = direct stores (any N),
+// 3 = gated pair: the tile's first 128 columns are gate sums, its last 128 the up sums of the same outputs.
 template <int EP>
 __global__ __launch_bounds__(256) void gemm_dense4_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -288,6 +289,47 @@ static_assert(kBarrierAt > 15 * kFragEvery && kBarrierAt <= 64 && kBarrierAt + 1
         }
         return;
     }
+    if constexpr (EP == 3) {
+        // Stage the tile as bf16 [256 m][128 gate | 128 up] - the projections' outputs as two separate launches would
+        // round them - then every thread combines eight gate values with their eight up values: silu in fp32 rounded to
+        // bf16, product rounded to bf16 (what bf16 tensors give `act(gate) * up`, and what the decode kernels' gated
+        // pair computes).
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) asm volatile("" : "+a"(acc[i][j]));  // as above: one row of tiles at a time
+            const int nl = wn * 128 + i * 16 + 4 * (lane >> 4);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int ml = wm * 128 + j * 16 + (lane & 15);
+                *reinterpret_cast<u32x2_t*>(lds + ml * kYRow + 2 * nl) =
+                    u32x2_t{pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3])};
+                if (j & 1) __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+        const int64_t n = tn * 128 + 8 * (tid & 15);   // output column
+        if (n >= a.gated_cols) return;
+#pragma unroll 4
+        for (int p = 0; p < TM / 16; p++) {
+            const int ml = (tid >> 4) + 16 * p;
+            const int64_t rr = row_begin + ml;
+            if (rr >= row_end) break;
+            const int64_t gr = a.rowmap ? (int64_t)a.rowmap[rr] : rr;
+            const u32x4_t gt = *reinterpret_cast<const u32x4_t*>(lds + ml * kYRow + 16 * (tid & 15));
+            const u32x4_t ut = *reinterpret_cast<const u32x4_t*>(lds + ml * kYRow + 256 + 16 * (tid & 15));
+            u32x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float g0 = bf16lo_to_f32(gt[e]), g1 = bf16hi_to_f32(gt[e]);
+                const float s0 = bf16_to_f32(f32_to_bf16(g0 / (1.0f + expf(-g0))));
+                const float s1 = bf16_to_f32(f32_to_bf16(g1 / (1.0f + expf(-g1))));
+                o[e] = pack_bf16(s0 * bf16lo_to_f32(ut[e]), s1 * bf16hi_to_f32(ut[e]));
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(a.y + gr * a.gated_cols + n));
+        }
+        return;
+    }
     const bool fast = (a.N & 3) == 0;  // rows of y are 8-byte aligned and a run of four columns never straddles N
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -339,7 +381,13 @@ int launch_gemm_dense4(const GemmArgs& a, hipStream_t stream) {
         if (attr != hipSuccess) return SNGGUF_E_LAUNCH;                                                                \
         gemm_dense4_kernel<EP><<<grid, dim3(256), kLdsBytes, stream>>>(a);                                             \
     } while (0)
-    if (a.partial) SNGGUF_GO(1);
+    if (a.gated_cols > 0) {
+        // the pair's layout: whole blocks of 128 + 128 rows, output rows of whole 16-byte pieces
+        if (a.partial || a.bias[0] || a.bias[1] || a.residual || (a.N & 255) != 0 || (a.gated_cols & 7) != 0 ||
+            a.gated_cols > a.N / 2 || a.gated_cols <= a.N / 2 - 128)
+            return SNGGUF_E_BADSHAPE;
+        SNGGUF_GO(3);
+    } else if (a.partial) SNGGUF_GO(1);
     else if ((a.N & 7) == 0) SNGGUF_GO(0);
     else SNGGUF_GO(2);
 #undef SNGGUF_GO

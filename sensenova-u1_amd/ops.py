@@ -34,7 +34,7 @@ _OUT_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 EXPORTED_SYMBOLS = (
     "sngguf_version", "sngguf_strerror", "sngguf_type_size", "sngguf_block_size", "sngguf_dequantize",
-    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_linear_static_max_outputs", "sngguf_linear_static", "sngguf_gate_up_silu", "sngguf_lm_head_argmax_workspace_bytes", "sngguf_lm_head_argmax", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
+    "sngguf_linear", "sngguf_linear_residual", "sngguf_linear_workspace_bytes", "sngguf_linear_ws", "sngguf_linear_static_max_outputs", "sngguf_linear_static", "sngguf_gate_up_silu", "sngguf_gate_up_silu_workspace_bytes", "sngguf_gate_up_silu_ws_fits", "sngguf_gate_up_silu_ws", "sngguf_lm_head_argmax_workspace_bytes", "sngguf_lm_head_argmax", "sngguf_grouped_workspace_bytes", "sngguf_grouped_linear",
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_rmsnorm_fits", "sngguf_rmsnorm", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
@@ -85,6 +85,12 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_static.restype = ci
     lib.sngguf_gate_up_silu.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu.restype = ci
+    lib.sngguf_gate_up_silu_workspace_bytes.argtypes = [i64, i64]
+    lib.sngguf_gate_up_silu_workspace_bytes.restype = i64
+    lib.sngguf_gate_up_silu_ws_fits.argtypes = [ci, i64, i64, i64]
+    lib.sngguf_gate_up_silu_ws_fits.restype = ci
+    lib.sngguf_gate_up_silu_ws.argtypes = [vp, i64, vp, vp, ci, i64, i64, vp, vp, i64, ci, vp]
+    lib.sngguf_gate_up_silu_ws.restype = ci
     lib.sngguf_lm_head_argmax_workspace_bytes.argtypes = [i64, i64]
     lib.sngguf_lm_head_argmax_workspace_bytes.restype = i64
     lib.sngguf_lm_head_argmax.argtypes = [vp, i64, vp, ci, i64, i64, vp, vp, vp, ci, vp]
@@ -314,6 +320,29 @@ def gate_up_silu_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, q
                                                 h2d.shape[1], x2d.shape[1], _ptr(h2d), numerics,
                                                 _stream(dev))
     _check(rc, "sngguf_gate_up_silu")
+
+
+def gate_up_silu_workspace_bytes(n: int, k: int) -> int:
+    """Bytes of workspace ``gate_up_silu_ws_into`` needs beyond 16 rows (512 * ceil(n / 128) * k)."""
+    return int(load_library().sngguf_gate_up_silu_workspace_bytes(n, k))
+
+
+def gate_up_silu_ws_fits(quant_type: int, m: int, n: int, k: int) -> bool:
+    """Whether the dense tile kernel's gated epilogue takes ``m`` rows of this pair (shape rule of the library)."""
+    return bool(load_library().sngguf_gate_up_silu_ws_fits(quant_type, m, n, k))
+
+
+def gate_up_silu_ws_into(x2d: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, quant_type: int, h2d: torch.Tensor,
+                         workspace: torch.Tensor, numerics: int) -> None:
+    """h2d[M, N] = silu(x2d @ Wg^T) * (x2d @ Wu^T) beyond decode sizes: one weight pass per matrix into ``workspace``
+    (at least ``gate_up_silu_workspace_bytes(N, K)`` bytes) and one launch of the dense tile kernel with the gated
+    epilogue; the two projection outputs are never written."""
+    dev = x2d.device
+    with _on(dev):
+        rc = load_library().sngguf_gate_up_silu_ws(_ptr(x2d), x2d.shape[0], _ptr(gate), _ptr(up), quant_type, h2d.shape[1],
+                                                   x2d.shape[1], _ptr(h2d), _ptr(workspace),
+                                                   workspace.numel() * workspace.element_size(), numerics, _stream(dev))
+    _check(rc, "sngguf_gate_up_silu_ws")
 
 
 def lm_head_argmax_fits(quant_type: int, m: int, k: int) -> bool:
