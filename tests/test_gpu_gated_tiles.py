@@ -57,6 +57,26 @@ def test_gated_pair_on_the_dense_tile_kernel(dev, c_oracle, qt, m, n, k, num):
     assert go.rel_l2(h[rows.to(dev)].cpu(), want) <= TOL
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_gated_cases(dev, c_oracle, seed):
+    """Seeded random shapes across the tile boundaries: any of the ten packed formats, 17 ... 1300 rows, output widths
+    that are any multiple of 8, K any admissible multiple of 128; the whole output against the oracle."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    qt = [go.Q4_0, go.Q4_1, go.Q5_0, go.Q5_1, go.Q8_0, go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K][r(0, 9)]
+    m = [r(17, 64), r(65, 300), r(250, 520), r(500, 1300)][r(0, 3)]
+    n = 8 * r(1, 70)
+    k = 256 * r(1, 6) if qt in (go.Q2_K, go.Q3_K, go.Q4_K, go.Q5_K, go.Q6_K) else 128 * r(1, 12)
+    num = [ops.NUM_GGML_FP32, ops.NUM_UPSTREAM_FP16][r(0, 1)]
+    print(f"case random gated seed={seed} qt={qt} {m}x{n}x{k} num={num}", flush=True)
+    gate, up, x = _pair(dev, qt, m, n, k, seed=seed)
+    h = _fused(x, gate, up, qt, n, k, num)
+    want = c_oracle.silu_mul(go.gguf_linear_forward(x.cpu(), gate.cpu(), qt, None, numerics=num),
+                             go.gguf_linear_forward(x.cpu(), up.cpu(), qt, None, numerics=num))
+    assert bool(torch.isfinite(h.float()).all())
+    assert go.rel_l2(h.cpu(), want) <= TOL
+
+
 def test_gated_pair_at_the_mlp_shape_over_image_rows(dev, c_oracle):
     """gate / up 4096 -> 12288 at M = 4096: the generation tower's MLP.  Sampled columns against the oracle, the whole
     output against the two plain workspace launches."""
