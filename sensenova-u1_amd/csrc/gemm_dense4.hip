@@ -33,6 +33,22 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const void* p) {
     return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
 }
 
+// exp(-g) for a g with at most 16 significant bits (here: bf16 values)
+__device__ __forceinline__ float exp_neg(float g) {
+    const float e = __builtin_amdgcn_exp2f(g * -1.44268798828125f);               // exact product
+    const float c = __builtin_fmaf(e, g * -4.8884952e-06f, e);                    // x exp2(-g lo), lo ln 2 = 4.8884952e-6
+    return e == 0.f ? 0.f : c;                                                    // (0 x inf at g = +inf)
+}
+
+// g / (1 + exp(-g)): hardware reciprocal, then one correction step of the quotient with the exact remainder
+__device__ __forceinline__ float silu_f32(float g) {
+    const float d = 1.0f + exp_neg(g);
+    const float r = __builtin_amdgcn_rcpf(d);
+    const float q = g * r;
+    const float c = __builtin_fmaf(__builtin_fmaf(-d, q, g), r, q);
+    return d < __builtin_inff() ? c : q;   // exp(-g) overflows below g = -88.7: the quotient is -0 as it stands
+}
+
 // byte offset of an LDS address within the workgroup's LDS allocation (what M0 and the ds instructions take)
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
@@ -292,8 +308,8 @@ static_assert(kBarrierAt > 15 * kFragEvery && kBarrierAt <= 64 && kBarrierAt + 1
     if constexpr (EP == 3) {
         // Stage the tile as bf16 [256 m][128 gate | 128 up] - the projections' outputs as two separate launches would
         // round them - then every thread combines eight gate values with their eight up values: silu in fp32 rounded to
-        // bf16, product rounded to bf16 (what bf16 tensors give `act(gate) * up`, and what the decode kernels' gated
-        // pair computes).
+        // bf16, product rounded to bf16 (what bf16 tensors give `act(gate) * up`; the decode kernels' gated pair rounds
+        // the same way).
 #pragma unroll
         for (int i = 0; i < 8; i++) {
 #pragma unroll
@@ -321,9 +337,14 @@ static_assert(kBarrierAt > 15 * kFragEvery && kBarrierAt <= 64 && kBarrierAt + 1
             u32x4_t o;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
+                // silu on the hardware's exp2 and reciprocal (the library exp and an IEEE division here cost 8 us per
+                // tile, 7 % of the launch, against 2 - 3).  exp(-g) = exp2(-g log2(e)): the product with the upper 16 bits
+                // of log2(e) is exact for a bf16 g, the rest of log2(e) enters as a first-order correction, and the
+                // quotient gets one correction step, so the result is good to about one unit in the last place of fp32
+                // before it is rounded to bf16.
                 const float g0 = bf16lo_to_f32(gt[e]), g1 = bf16hi_to_f32(gt[e]);
-                const float s0 = bf16_to_f32(f32_to_bf16(g0 / (1.0f + expf(-g0))));
-                const float s1 = bf16_to_f32(f32_to_bf16(g1 / (1.0f + expf(-g1))));
+                const float s0 = bf16_to_f32(f32_to_bf16(silu_f32(g0)));
+                const float s1 = bf16_to_f32(f32_to_bf16(silu_f32(g1)));
                 o[e] = pack_bf16(s0 * bf16lo_to_f32(ut[e]), s1 * bf16hi_to_f32(ut[e]));
             }
             __builtin_nontemporal_store(o, reinterpret_cast<u32x4_t*>(a.y + gr * a.gated_cols + n));
