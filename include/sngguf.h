@@ -208,7 +208,8 @@ int sngguf_gate_up_silu(const void* x, int64_t M, const void* q_gate, const void
  *  M <= 16 runs sngguf_gate_up_silu (the workspace is not touched).  Otherwise the shape must satisfy
  *  sngguf_gate_up_silu_ws_fits(qtype, M, N, K) (M >= 17, K % 128 == 0, N % 8 == 0, M K < 2^31, a packed block
  *  format), else SNGGUF_E_BADSHAPE / SNGGUF_E_BADTYPE and the caller runs the two projections separately.  It
- *  pays from about 1024 rows on (a launch has 2 N / 256 x M / 256 tiles and there is no K split; 12288 x 4096 at
+ *  pays from about 512 rows on when the launch's ceil(M / 256) x ceil(N / 128) tiles come close to whole rounds of
+ *  the 256 compute units (there is no K split; 12288 x 4096 at
  *  4096 rows: 628 us against 695 us for two sngguf_linear_ws launches and the product, at 2048 rows 354 against 451).
  */
 int64_t sngguf_gate_up_silu_workspace_bytes(int64_t N, int64_t K);

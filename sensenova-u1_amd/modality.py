@@ -192,14 +192,23 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
     return down_proj(h)
 
 
-# measured on 12288 x 4096 (gated launch / two launches and the product, us): 768 rows 270 / 244, 1024 242 / 248,
-# 1280 293 / 317, 2048 365 / 453, 4096 655 / 716
-GATED_TILE_MIN_ROWS = 1024
+# The gated launch has ceil(rows / 256) x ceil(N / 128) output tiles and no K split, so it pays when those tiles come close
+# to whole rounds of the chip's 256 compute units.  Measured on 12288 x 4096 (gated launch / two launches and the product,
+# us): 512 rows (0.75 of a round) 183 / 199, 768 (1.125 rounds) 265 / 245, 1024 (1.5) 237 / 246, 1280 (1.875) 287 / 312,
+# 1536 (2.25) 368 / 460, 2048 354 / 446, 4096 631 / 706.
+GATED_TILE_MIN_ROWS = 512
+GATED_TILE_MIN_FILL = 0.7
+
+
+def gated_tile_fill(rows: int, n: int) -> float:
+    """Share of the compute units' tile slots that the gated launch's tiles fill, over its rounds."""
+    tiles = -(-rows // 256) * -(-n // 128)
+    return tiles / (256 * -(-tiles // 256))
 
 
 def _gated_tile_route(x, rows, same, gate_proj, up_proj) -> bool:
-    """Whether ``gated_mlp`` runs gate / up / SiLU as one dense GEMM launch: enough rows for the launch's tiles to fill
-    the chip (it has no K split), both weights of one packed type and shape, no bias, default GEMM policy."""
+    """Whether ``gated_mlp`` runs gate / up / SiLU as one dense GEMM launch: enough rows and tiles to fill the chip, both
+    weights of one packed type and shape, no bias, default GEMM policy."""
     if not (rows >= GATED_TILE_MIN_ROWS and same and x.is_cuda and x.dtype == torch.bfloat16):
         return False
     if gate_proj.bias is not None or up_proj.bias is not None:
@@ -209,6 +218,8 @@ def _gated_tile_route(x, rows, same, gate_proj, up_proj) -> bool:
     if getattr(gate_proj, "gemm_policy", "auto") != "auto" or getattr(up_proj, "gemm_policy", "auto") != "auto":
         return False
     if gate_proj.numerics != up_proj.numerics:
+        return False
+    if gated_tile_fill(rows, gate_proj.out_features) < GATED_TILE_MIN_FILL:
         return False
     return ops.gate_up_silu_ws_fits(int(gate_proj.weight.quant_type), rows, gate_proj.out_features, gate_proj.in_features)
 

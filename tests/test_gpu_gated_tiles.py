@@ -11,7 +11,8 @@ import torch
 
 from oracle import gguf_oracle as go
 from sensenova_u1_amd import GGUFLinear, GGUFParameter, ops, synthetic
-from sensenova_u1_amd.modality import GATED_TILE_MIN_ROWS, gated_mlp
+from sensenova_u1_amd import modality
+from sensenova_u1_amd.modality import gated_mlp
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -123,10 +124,11 @@ def test_gated_pair_entry_point_routes_and_refusals(dev):
         ops.gate_up_silu_ws_into(x, gate, up, qt, h, small, ops.NUM_UPSTREAM_FP16)
 
 
-def test_gated_mlp_takes_the_tile_route_from_its_row_limit_on(dev):
-    """``modality.gated_mlp`` (what the loader points ``Qwen3MLP.forward`` at) with enough rows: same result as the
-    three module calls and the product on bf16 tensors."""
-    n, k, m = 640, 512, GATED_TILE_MIN_ROWS
+def test_gated_mlp_takes_the_tile_route_when_its_tiles_fill_the_chip(dev, monkeypatch):
+    """``modality.gated_mlp`` (what the loader points ``Qwen3MLP.forward`` at) with enough rows and tiles: same result as
+    the three module calls and the product on bf16 tensors, and the gated entry point is what ran."""
+    n, k, m = 6144, 256, 1024
+    assert modality.gated_tile_fill(m, n) >= modality.GATED_TILE_MIN_FILL > modality.gated_tile_fill(768, 12288)
     mods = []
     for j, (o, i) in enumerate(((n, k), (n, k), (k, n))):
         lin = GGUFLinear(i, o, bias=False, compute_dtype=torch.bfloat16, device="meta")
@@ -134,7 +136,15 @@ def test_gated_mlp_takes_the_tile_route_from_its_row_limit_on(dev):
         mods.append(lin)
     gate, up, down = mods
     x = synthetic.make_activations(m, k, seed=9, device=dev).view(2, m // 2, k)
+    calls = []
+    real = ops.gate_up_silu_ws_into
+    monkeypatch.setattr(ops, "gate_up_silu_ws_into", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
     got = gated_mlp(x, gate, up, down)
+    assert calls == [m]
     want = down(torch.nn.functional.silu(gate(x)) * up(x))
     assert got.shape == want.shape
     assert go.rel_l2(got.cpu(), want.cpu()) <= 1e-4
+    # few tiles: the separate launches (with their K split) stay
+    calls.clear()
+    gated_mlp(x[:, :128], gate, up, down)
+    assert calls == []
