@@ -580,9 +580,15 @@ def main() -> None:
         def tower_resident(i):
             ws = dense[i % 2]
             for j, (_, n, k) in enumerate(shapes):
+                ops.linear_ws_into(xs[k], ws[j].view(torch.uint8), ops.BF16, None, ys[n], wtmp, num)
+
+        def tower_resident_device_library(i):
+            ws = dense[i % 2]
+            for j, (_, n, k) in enumerate(shapes):
                 torch.matmul(xs[k], ws[j].t(), out=ys[n])
 
         wall3, _ = run_region(tower_resident, gs, args.gemm_warmup)
+        wall3_dl, _ = run_region(tower_resident_device_library, gs, args.gemm_warmup)
         del dense
         # q | k | v as one [6144, 4096] matrix (rows of the three packed weights one after another, what
         # FusedProjections builds at load): 384 large tiles in one launch instead of 256 + 64 + 64
@@ -718,9 +724,12 @@ def main() -> None:
             },
             "resident": {
                 "what": "gemm_policy 'resident': the bf16 weights written once by sngguf dequantize and kept "
-                        "(2 N K bytes per linear), every call is the device library's dense GEMM alone",
+                        "(2 N K bytes per linear), every call is the library's dense tile kernel alone (sngguf_linear_ws on "
+                        "BF16 rows: K split over workgroups for k / v); device_library_*: torch.matmul on the same kept weights",
                 "value": round(flops / (wall3 / gs * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(wall3 / gs, 4),
                 "pct_of_bf16_mfma_peak": round(100 * flops / (wall3 / gs * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+                "device_library_value": round(flops / (wall3_dl / gs * 1e-3) / 1e12, 2),
+                "device_library_ms_per_step": round(wall3_dl / gs, 4),
             },
         }
         del tower, xs, ys, wtmp

@@ -247,8 +247,9 @@ int linear_ws_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N
     if (rc != SNGGUF_OK || M == 0 || N == 0) return rc;
     if (workspace && !aligned(workspace, 16)) return SNGGUF_E_ALIGN;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // everything that does not fit the dense route runs as sngguf_linear does (plain bf16 rows need no weight pass)
-    const bool fits = workspace && dense_route_fits(M, N, K) && qtype != SNGGUF_TYPE_BF16;
+    // everything that does not fit the dense route runs as sngguf_linear does
+    const bool plain = qtype == SNGGUF_TYPE_BF16;   // rows that are bf16 already: no weight pass, the dense kernel reads them
+    const bool fits = workspace && dense_route_fits(M, N, K);
     if (!fits) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     // Few output tiles (a few hundred rows, or a narrow matrix): a 256 x 256 tile takes as long per K step whether
     // or not the other compute units have work, so K is split over enough workgroups to occupy them, with the fp32
@@ -260,20 +261,21 @@ int linear_ws_impl(const void* x, int64_t M, const void* q, int qtype, int64_t N
     // (from 4096 rows on the weight pass pays for itself even here: a K step of the dense kernel takes 1.4 us against 2.0 us
     // with the decode in the loop, and sixteen row tiles share one pass - 4096 x 1024 <- 4096: 56 against 61 us, 2048 wide
     // 80 against 92 us; at 512 rows the pass costs more than it saves, 48 against 44 us on 4096 x 4096)
-    const bool tile_type = (qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K) && M < 4096;
+    const bool tile_type = plain || ((qtype == SNGGUF_TYPE_Q8_0 || qtype == SNGGUF_TYPE_Q4_K) && M < 4096);
     const int64_t dense_bytes = tile_type ? 0 : 2 * N * K;
     if (tiles <= 128 && workspace_bytes > dense_bytes) {
         const int64_t room = (workspace_bytes - dense_bytes) / (4 * M * N);
-        const int64_t slices = pick_k_slices(M, N, tiles, ksteps, room, tile_type);
+        const int64_t slices = pick_k_slices(M, N, tiles, ksteps, room, tile_type && !plain);
         if (slices >= 2) {
             float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + dense_bytes);
             if (tile_type)
-                return sngguf::launch_gemm_splitk(x, M, q, qtype, N, K, bias, y, partial, (int)slices, numerics, s);
+                return sngguf::launch_gemm_splitk(x, M, q, plain ? 30 : qtype, N, K, bias, y, partial, (int)slices, numerics, s);
             const int rd = sngguf::launch_dequantize(q, qtype, N, K, workspace, SNGGUF_OUT_BF16, numerics, s);
             if (rd != SNGGUF_OK) return rd;
             return sngguf::launch_gemm_splitk(x, M, workspace, 30, N, K, bias, y, partial, (int)slices, numerics, s);
         }
     }
+    if (plain) return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);
     // no room for a K split: row chunks through the decode kernel where they beat the few tiles of the dense kernel too
     if (workspace_bytes < 2 * N * K || row_chunks_win(M, N, K, qtype))
         return linear_impl(x, M, q, qtype, N, K, bias, nullptr, y, numerics, stream);

