@@ -55,7 +55,7 @@ def grouped_linear(hidden_states: torch.Tensor, image_gen_indicators: Optional[t
                 # the library's workspace route: each group takes the kernels its own row count calls for
                 x2d = proj._checked_rows(hidden_states)
                 proj_mot_gen._checked_rows(hidden_states)
-                ws = ops.pooled_workspace(x2d.device, ops.linear_workspace_bytes(proj.out_features, proj.in_features))
+                ws = ops.pooled_workspace(x2d.device, max(proj._workspace_bytes(split), proj._workspace_bytes(x2d.shape[0] - split)))
                 bu = proj.bias.detach().to(torch.bfloat16).contiguous() if proj.bias is not None else None
                 bg = proj_mot_gen.bias.detach().to(torch.bfloat16).contiguous() if proj_mot_gen.bias is not None else None
                 ops.grouped_linear_ws_into(x2d, None, split, proj.weight, int(proj.weight.quant_type), proj_mot_gen.weight,
