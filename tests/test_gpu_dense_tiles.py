@@ -65,3 +65,29 @@ def test_k_split_partial_sums_of_the_workspace_route(dev, m, n, k):
     want = go.gguf_linear_forward(x.cpu(), packed[cols.to(dev)].cpu(), go.Q8_0)
     assert go.rel_l2(y[:, cols.to(dev)].cpu(), want) <= TOL
     assert bool(torch.isfinite(y.float()).all())
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 4096), (4096, 1024, 1024), (300, 520, 2048)])
+def test_k_split_of_plain_bf16_rows_with_a_workspace(dev, m, n, k):
+    """Weights that are bf16 rows already (GGUF type 30, and the kept weights of the module's "resident" policy) need no
+    weight pass; with a workspace that has room for fp32 partial sums a shape with few output tiles still gets the K
+    split.  Against the oracle, and against the same call without a workspace (the dense kernel unsplit: another order
+    of the fp32 sums, same bf16 weights)."""
+    print(f"case dense split-K of bf16 rows {m}x{n}x{k}", flush=True)
+    w, wd = _bf16_rows(n, k, 3 * n + k, dev)
+    x = synthetic.make_activations(m, k, seed=m + 1)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n + 2)) * 0.5).to(torch.bfloat16)
+    xd = x.to(dev)
+    outs = []
+    for ws_bytes in (0, 16 * m * n):
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.linear_ws_into(xd, wd, go.BF16, bias.to(dev), y, ws, ops.NUM_UPSTREAM_FP16)
+        assert bool(torch.isfinite(y.float()).all())
+        outs.append(y)
+    rows = torch.randperm(m, generator=torch.Generator().manual_seed(3))[:48]
+    rows[0], rows[1] = 0, m - 1
+    want = go.gguf_linear_forward(x[rows], w.view(torch.uint8), go.BF16, bias)
+    for y in outs:
+        assert go.rel_l2(y[rows.to(dev)].cpu(), want) <= TOL
+    assert go.rel_l2(outs[1].cpu(), outs[0].cpu()) <= 5e-4
