@@ -66,6 +66,10 @@ def main() -> None:
     ap.add_argument("--gemm-warmup", type=int, default=10,
                     help="untimed tower-layer passes before the GEMM leg (about 20 ms: the shader clock settles "
                          "under the matrix-core load within that time)")
+    ap.add_argument("--settle-ms", type=float, default=20.0,
+                    help="untimed repetitions of each leg's own timed work (the captured graph) for at least this long "
+                         "before its timed region, so that a short region (--steps 20) is measured in the steady state of a "
+                         "decode loop (clocks, translation caches, graph upload) like a long one")
     ap.add_argument("--numerics", type=int, default=1, help="1 = upstream fp16 chain (drop-in), 0 = ggml fp32")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB elementwise device copies (a known-size reference for scaling the "
@@ -104,9 +108,18 @@ def main() -> None:
                        synthetic.make_packed(Q8_0, HIDDEN, INTER, seed=1002 + 3 * i, device=dev)))
     torch.cuda.synchronize()
 
-    def run_region(fn, n_steps: int, warmup: int):
+    settle_replays = []
+
+    def run_region(fn, n_steps: int, warmup: int, settle_ms: float = None):
         """W warm-up steps, then exactly n_steps steps timed (wall clock around a synchronised
-        region, and HIP events on the launch stream).  Returns (wall_ms, event_ms)."""
+        region, and HIP events on the launch stream).  Returns (wall_ms, event_ms).
+
+        Between the warm-up and the timed region the SAME work (the captured graph, or the eager loop)
+        is repeated untimed until ``settle_ms`` of wall time have passed: a region of 20 steps lasts
+        under a millisecond, in which neither the shader and memory clocks nor the translation caches
+        have reached the state every later step of a decode loop runs in.  The timed region is still
+        exactly n_steps steps; the figure is then the same whatever --steps is."""
+        settle = args.settle_ms if settle_ms is None else settle_ms
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
@@ -121,19 +134,29 @@ def main() -> None:
                 print(f"bench.py: graph capture failed ({exc}); timing eager launches", file=sys.stderr)
                 graph = None
                 torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        if graph is not None:
-            # the first launch of an instantiated graph also uploads it to the device (4 - 8 % on top of a 512-node graph of
-            # 24 us kernels, measured); torch exposes no hipGraphUpload, so one untimed replay does it
-            graph.replay()
+
+        def once():
+            if graph is not None:
+                graph.replay()
+            else:
+                for i in range(n_steps):
+                    fn(warmup + i)
+
+        # the first launch of an instantiated graph also uploads it to the device (4 - 8 % on top of a 512-node graph of
+        # 24 us kernels, measured); torch exposes no hipGraphUpload, so the untimed replays do it
+        t_settle = time.perf_counter()
+        reps = 0
+        while reps < 1 or (time.perf_counter() - t_settle) * 1e3 < settle:
+            once()
+            reps += 1
+            if reps % 8 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
+        settle_replays.append(reps)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(n_steps):
-                fn(warmup + i)
+        once()
         e1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
@@ -189,7 +212,8 @@ def main() -> None:
             "layers_rotated": L,
             "bytes_per_step": step_bytes,
             "graph": not args.no_graph,
-            "graph_upload_replays_untimed": 0 if args.no_graph else 1,
+            "settle_ms": args.settle_ms,
+            "untimed_replays_before_timed_region": settle_replays[0],
             "numerics": "upstream_fp16" if num == 1 else "ggml_fp32",
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
@@ -204,6 +228,8 @@ def main() -> None:
             "traffic": MEASURED_TRAFFIC["gemv_gate_up_m1"],
             "bytes_per_launch": gu_bytes,
             "avg_launch_us": round(gu_ms * 1e3, 3),
+            "device_ms_per_step": round(ev1 / K, 6),
+            "timing": "HIP events on the launch stream around the timed replay of a graph of `steps` gate/up launches",
         },
         "down_proj": {
             "kernel": "sngguf::gemv_q8_mfma_kernel<upstream_fp16> (down 12288->4096, M=1)",
@@ -212,6 +238,48 @@ def main() -> None:
             "avg_launch_us": round(dn_ms * 1e3, 3),
         },
     }
+
+    # ---- what the memory system gives a launch that only reads: the library's streaming-read probe over a buffer
+    # ten times the last-level cache, as one launch over all of it and as launches of the gate/up kernel's size ------
+    if not args.no_extra:
+        import ctypes
+        lib = ops.load_library()
+        chunk = (gu_bytes + 4095) // 4096 * 4096
+        n_chunks = 24
+        probe_buf = torch.empty(n_chunks * chunk, dtype=torch.uint8, device=dev)
+        probe_buf.view(torch.int64).random_()
+        probe_out = torch.empty(int(lib.sngguf_probe_stream_read_out_bytes()), dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+
+        def probe(off, nbytes, nt, wgs=0):
+            rc = lib.sngguf_probe_stream_read(ctypes.c_void_p(probe_buf.data_ptr() + off), nbytes, ctypes.c_void_p(probe_out.data_ptr()),
+                                              wgs, nt, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+            assert rc == 0, rc
+
+        pr = {}
+        for nt in (1, 0):
+            _, ev_all = run_region(lambda i: probe(0, n_chunks * chunk, nt), 8, 2)
+            _, ev_chunk = run_region(lambda i: probe((i % n_chunks) * chunk, chunk, nt), max(K, 48), 8)
+            _, ev_chunk256 = run_region(lambda i: probe((i % n_chunks) * chunk, chunk, nt, 256), max(K, 48), 8)
+            tag = "nontemporal" if nt else "plain"
+            pr[tag] = {"one_launch_over_all_GBps": round(n_chunks * chunk / (ev_all / 8 * 1e-3) / 1e9, 1),
+                       "launches_of_gate_up_size_GBps": round(chunk / (ev_chunk / max(K, 48) * 1e-3) / 1e9, 1),
+                       "launches_of_gate_up_size_us": round(ev_chunk / max(K, 48) * 1e3, 3),
+                       "launches_of_gate_up_size_256_workgroups_us": round(ev_chunk256 / max(K, 48) * 1e3, 3)}
+        best = max(v["one_launch_over_all_GBps"] for v in pr.values())
+        best_chunk = max(v["launches_of_gate_up_size_GBps"] for v in pr.values())
+        result["hbm_read_probe"] = {
+            "what": "sngguf_probe_stream_read: a kernel that only reads (16 bytes per lane and request, eight in flight, one "
+                    "word per workgroup written), over a 2.6 GB buffer: one launch over all of it, and back-to-back launches "
+                    "of the gate/up kernel's 107 MB each on distinct ranges (graph replay, HIP events)",
+            "buffer_bytes": n_chunks * chunk, "bytes_per_sized_launch": chunk, **pr,
+            "achievable_hbm_read_GBps": best, "achievable_frac_of_peak": round(best / HBM_PEAK_GBPS, 4),
+            "achievable_at_gate_up_launch_size_GBps": best_chunk,
+        }
+        result["roofline"]["achievable_hbm_read_GBps"] = best
+        result["roofline"]["achievable_at_this_launch_size_GBps"] = best_chunk
+        result["roofline"]["frac_of_achievable_at_this_launch_size"] = round(gu_gbps / best_chunk, 4)
+        del probe_buf, probe_out
 
     # ---- same MLP at M = 4 and 16 --------------------------------------------------------------
     decode = {}

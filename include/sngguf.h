@@ -169,6 +169,17 @@ int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int
                          const void* bias, void* y, int numerics, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: one launch that reads `bytes` (rounded down to 16) of device
+ * memory once - contiguous shares per workgroup, 16 bytes per lane and request, eight requests in flight per lane,
+ * with (nontemporal != 0) or without the read-once cache hint - and folds them into one word per workgroup in `out`
+ * (sngguf_probe_stream_read_out_bytes() bytes, 16-byte aligned).  `workgroups` 0 = 1024 (at most 4096).  Timed over
+ * a buffer larger than the last-level cache it gives the read rate this device sustains for a launch of that size,
+ * the ceiling the decode kernels' achieved GB/s can be read against beside the published peak.
+ */
+int64_t sngguf_probe_stream_read_out_bytes(void);
+int sngguf_probe_stream_read(const void* p, int64_t bytes, void* out, int workgroups, int nontemporal, void* stream);
+
+/*
  * lm_head followed by torch.argmax: out_index[m] = argmax_n bf16(x[m] . W[n]^T + bias[n]), the greedy next token of
  * the think loop (`torch.argmax(outputs.logits[:, -1, :], dim=-1)`, src/sensenova_u1/models/neo_unify/
  * modeling_neo_chat.py:557,586, on the logits of `self.lm_head(...)`, modeling_qwen3.py:1264).  The decode kernel's

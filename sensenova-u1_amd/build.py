@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libsngguf.so")
-SOURCES = ["api.cpp", "gguf_reader.cpp", "dequantize.hip", "plain_bf16.hip", "rmsnorm.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemv_q8_tiled.hip", "gemm.hip", "gemm_tiles.hip", "gemm_dense4.hip", "static_scratch.hip"]
+SOURCES = ["api.cpp", "gguf_reader.cpp", "dequantize.hip", "plain_bf16.hip", "rmsnorm.hip", "gemv.hip", "gemv_q8_mfma.hip", "gemv_kq_mfma.hip", "gemv_q8_tiled.hip", "gemm.hip", "gemm_tiles.hip", "gemm_dense4.hip", "static_scratch.hip", "stream_probe.hip"]
 
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIP_FLAGS = [

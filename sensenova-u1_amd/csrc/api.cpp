@@ -39,6 +39,8 @@ int launch_gemm_dense_gated(const void* x, int64_t M, const void* w2, int64_t co
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
                 const void* residual, void* y,
                 int numerics, hipStream_t stream);
+int64_t stream_probe_out_bytes();
+int launch_stream_read(const void* p, int64_t bytes, void* out, int workgroups, bool nontemporal, hipStream_t stream);
 int64_t grouped_workspace_bytes(int64_t M);
 int launch_grouped_gemm(const void* x, int64_t M, const uint8_t* indicator, int64_t n_text, const void* q_und,
                         int qtype_und, const void* q_gen, int qtype_gen, int64_t N, int64_t K, const void* bias_und,
@@ -493,6 +495,16 @@ int sngguf_rmsnorm_gate_up_silu_tiled(const void* x, int64_t M, const void* gamm
     if (!aligned(tiled_up, 16)) return SNGGUF_E_ALIGN;
     return sngguf::launch_gemv_q8_tiled(x, M, tiled_gate, tiled_up, N, K, nullptr, nullptr, h, numerics, true,
                                         static_cast<hipStream_t>(stream), gamma, eps);
+}
+
+int64_t sngguf_probe_stream_read_out_bytes(void) { return sngguf::stream_probe_out_bytes(); }
+
+int sngguf_probe_stream_read(const void* p, int64_t bytes, void* out, int workgroups, int nontemporal, void* stream) {
+    if (bytes < 0 || workgroups < 0) return SNGGUF_E_BADSHAPE;
+    if (bytes == 0) return SNGGUF_OK;
+    if (!p || !out) return SNGGUF_E_NULLPTR;
+    if (!aligned(p, 16) || !aligned(out, 16)) return SNGGUF_E_ALIGN;
+    return sngguf::launch_stream_read(p, bytes, out, workgroups, nontemporal != 0, static_cast<hipStream_t>(stream));
 }
 
 int64_t sngguf_grouped_workspace_bytes(int64_t M) { return sngguf::grouped_workspace_bytes(M); }

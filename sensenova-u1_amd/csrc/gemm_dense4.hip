@@ -46,7 +46,9 @@ __device__ __forceinline__ float silu_f32(float g) {
     const float r = __builtin_amdgcn_rcpf(d);
     const float q = g * r;
     const float c = __builtin_fmaf(__builtin_fmaf(-d, q, g), r, q);
-    return d < __builtin_inff() ? c : q;   // exp(-g) overflows below g = -88.7: the quotient is -0 as it stands
+    // exp(-g) overflows below g = -88.7: the quotient is -0 as it stands; at g = +inf the remainder inf - inf is a NaN
+    // and the quotient +inf is the value
+    return (d < __builtin_inff() && __builtin_fabsf(g) < __builtin_inff()) ? c : q;
 }
 
 // byte offset of an LDS address within the workgroup's LDS allocation (what M0 and the ds instructions take)

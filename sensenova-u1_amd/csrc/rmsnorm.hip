@@ -13,8 +13,8 @@ constexpr int kThreads = 256;
 constexpr int kPiecesPerThread = 8;   // up to 256 * 8 * 8 = 16384 elements per row in registers
 }  // namespace
 
-__global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(const bf16_t* __restrict__ x, int64_t K, const bf16_t* __restrict__ gamma,
-                                                                float eps, bf16_t* __restrict__ y) {
+__global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(const bf16_t* x, int64_t K, const bf16_t* __restrict__ gamma,
+                                                                float eps, bf16_t* y) {
     __shared__ float part[kThreads / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bf16_t* xr = x + (int64_t)blockIdx.x * K;
@@ -55,7 +55,8 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(const bf16_t* __
     }
 }
 
-// x, y [M][K] bf16, gamma [K] bf16, all 16-byte aligned, K % 8 == 0 (checked by the caller); y may be x.
+// x, y [M][K] bf16, gamma [K] bf16, all 16-byte aligned, K % 8 == 0 (checked by the caller); y may be x (neither is
+// declared restrict: every thread reads a 16-byte piece of the row before it writes that same piece and no other).
 int launch_rmsnorm(const void* x, int64_t M, int64_t K, const void* gamma, float eps, void* y, hipStream_t stream) {
     rmsnorm_rows_kernel<<<dim3((unsigned)M), dim3(kThreads), 0, stream>>>(static_cast<const bf16_t*>(x), K, static_cast<const bf16_t*>(gamma),
                                                                           eps, static_cast<bf16_t*>(y));

@@ -386,10 +386,11 @@ __device__ __forceinline__ float wave_sum(float v) {
 // ---- arg-max over output columns (lm_head followed by torch.argmax) ------------------------------------------
 // A (value, column) pair packed so that an unsigned 64-bit maximum picks the largest bf16 value and, among equal
 // values, the lowest column - what torch.argmax returns (first maximal index); a NaN counts as the largest value,
-// as it does there.  High word: the bf16 bits mapped to an unsigned number that grows with the value; low word:
-// 2^32 - 1 - column.
+// as it does there; -0 and +0 compare equal there, so both map to the key of +0.  High word: the bf16 bits mapped to
+// an unsigned number that grows with the value; low word: 2^32 - 1 - column.
 __device__ __forceinline__ uint64_t argmax_key(float v, int64_t n) {
-    const uint32_t b = f32_to_bf16(v);
+    uint32_t b = f32_to_bf16(v);
+    if ((b & 0x7FFFu) == 0) b = 0;              // a zero of either sign
     uint32_t k = (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u);
     if ((b & 0x7FFFu) > 0x7F80u) k = 0xFFFFu;   // NaN of either sign
     return ((uint64_t)k << 32) | (uint64_t)(0xFFFFFFFFu - (uint32_t)n);

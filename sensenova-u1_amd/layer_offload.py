@@ -137,6 +137,11 @@ class PackedLayerStore:
                 self._managed.add(id(t))
                 by_group.setdefault(groups.get(name, GROUP_SHARED), []).append((name, t))
             arenas = {g: _Arena(ts, pin_memory) for g, ts in by_group.items()}
+            # q / k / v that a loader stacked into one device tensor now live in the arenas: the stack lets go of its copy
+            for mod in layer.modules():
+                stack = mod.__dict__.get("_shared_stack")
+                if stack is not None:
+                    stack.release_if_moved()
             for g, a in arenas.items():
                 self._slot_bytes[g] = max(self._slot_bytes[g], a.nbytes)
             self._arenas.append(arenas)

@@ -325,13 +325,35 @@ class SharedInputStack:
         self._pending = None
 
     def intact(self) -> bool:
+        if self.stacked is None:
+            return False
         base = self.stacked.data_ptr()
         first = self.members[0]
         for mod, off in zip(self.members, self.offsets):
             w = mod.weight
             if (w.data_ptr() != base + off * self.row_bytes or w.device != self.stacked.device or mod.decode_layout != "native"
                     or mod.numerics != first.numerics or int(w.quant_type) != int(first.weight.quant_type) or mod.bias is not None):
+                self.release_if_moved()
                 return False
+        return True
+
+    def release_if_moved(self) -> bool:
+        """Drop the stacked device tensor once no member's weight lies in it any more (an offloader has rebound every
+        ``weight.data`` to its own arenas, the model went to another device): the stack would otherwise keep a second
+        copy of the packed rows alive for nothing.  The members keep whatever storage they have now and are detached;
+        returns whether the stack was released."""
+        if self.stacked is None:
+            return True
+        store = self.stacked.untyped_storage().data_ptr()
+        for mod in self.members:
+            w = mod.weight
+            if w.device == self.stacked.device and w.untyped_storage().data_ptr() == store:
+                return False
+        self.stacked = None
+        self._pending = None
+        for mod in self.members:
+            if mod.__dict__.get("_shared_stack") is self:
+                del mod.__dict__["_shared_stack"]
         return True
 
     def member_forward(self, mod: GGUFLinear, x: torch.Tensor) -> Optional[torch.Tensor]:

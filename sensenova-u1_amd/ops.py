@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_rmsnorm_fits", "sngguf_rmsnorm", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
+    "sngguf_probe_stream_read_out_bytes", "sngguf_probe_stream_read",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
 )
@@ -109,6 +110,10 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_tiled.restype = ci
     lib.sngguf_gate_up_silu_tiled.argtypes = [vp, i64, vp, vp, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu_tiled.restype = ci
+    lib.sngguf_probe_stream_read_out_bytes.argtypes = []
+    lib.sngguf_probe_stream_read_out_bytes.restype = i64
+    lib.sngguf_probe_stream_read.argtypes = [vp, i64, vp, ci, ci, vp]
+    lib.sngguf_probe_stream_read.restype = ci
     cf = ctypes.c_float
     lib.sngguf_rmsnorm_fits.argtypes = [ci, i64, i64]
     lib.sngguf_rmsnorm_fits.restype = ci

@@ -67,6 +67,29 @@ def test_argmax_ties_and_nan_follow_torch(dev):
     assert torch.equal(got, ops.linear(x.to(dev), pd, go.Q8_0, bias).argmax(dim=-1))
 
 
+def test_argmax_treats_signed_zeros_as_equal(dev):
+    """A row whose maximum is zero, with a -0 logit in front of a +0 logit: torch.argmax compares them equal and returns
+    the first.  -0 comes from a negative sum too small for bf16 (2^-120 x -2^-24); every other logit is negative."""
+    print("case argmax signed zeros", flush=True)
+    n, k = 512, 256
+    packed = torch.zeros((n, k // 32 * 34), dtype=torch.uint8)
+    one = torch.tensor([1.0], dtype=torch.float16).view(torch.uint8)
+    tiny = torch.tensor([2.0 ** -24], dtype=torch.float16).view(torch.uint8)
+    packed[:, 0:2] = one
+    packed[:, 2] = 0x9C                      # q[0] = -100: logit -100 x
+    a, b = 37, 300
+    packed[a, 0:2] = tiny
+    packed[a, 2] = 0xFF                      # q[0] = -1, d = 2^-24
+    packed[b, 2] = 0                         # all-zero row: +0
+    x = torch.zeros((2, k), dtype=torch.bfloat16)
+    x[:, 0] = 2.0 ** -120
+    for numerics in (0, 1):
+        logits = ops.linear(x.to(dev), packed.to(dev), go.Q8_0, None, numerics)
+        got = ops.lm_head_argmax(x.to(dev), packed.to(dev), go.Q8_0, None, numerics)
+        assert float(logits[0, a]) == 0.0 and float(logits[0, b]) == 0.0 and float(logits.max()) == 0.0
+        assert torch.equal(got, logits.argmax(dim=-1)), (got, logits.argmax(dim=-1), logits[0, a], logits[0, b])
+
+
 def test_vocabulary_sized_argmax_and_module_helper(dev):
     print("case argmax lm_head", flush=True)
     n, k = 151936, 4096

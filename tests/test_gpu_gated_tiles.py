@@ -58,6 +58,38 @@ def test_gated_pair_on_the_dense_tile_kernel(dev, c_oracle, qt, m, n, k, num):
     assert go.rel_l2(h[rows.to(dev)].cpu(), want) <= TOL
 
 
+def test_overflowed_and_huge_gates_follow_silu_on_bf16_tensors(dev, c_oracle):
+    """Gate sums that overflow to +-inf, or are finite and huge: silu(+inf) = +inf, silu(-inf) = NaN (-inf / inf, as
+    torch computes it), silu(-1e30) = -0.  The dense launch's own exp / reciprocal must give what the oracle and the
+    decode kernels' gated pair give on the same sums."""
+    print("case gated tiles overflow", flush=True)
+    qt, n, k = go.Q8_0, 256, 256
+    gate = synthetic.make_packed(qt, n, k, seed=71)
+    up = synthetic.make_packed(qt, n, k, seed=72)
+    big = torch.tensor([100.0], dtype=torch.float16).view(torch.uint8)
+    gate[:64, 0:2] = big                       # first block of the first 64 gate rows: weights 100 q
+    for m in (4, 130):                         # the decode kernels' pair and the dense launch
+        x = torch.zeros((m, k), dtype=torch.bfloat16)
+        x[0, 0], x[1, 0], x[2, 0] = 1e38, -1e38, 1e30
+        x[3:] = synthetic.make_activations(m - 3, k, seed=5)
+        g = go.gguf_linear_forward(x, gate, qt)
+        u = go.gguf_linear_forward(x, up, qt)
+        want = c_oracle.silu_mul(g, u)
+        assert bool(torch.isinf(g[0, :64].float()).any()) and bool(torch.isnan(want[:2].float()).any())
+        if m <= 16:
+            h = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            ops.gate_up_silu_into(x.to(dev), gate.to(dev), up.to(dev), qt, h, 1)
+        else:
+            h = _fused(x.to(dev), gate.to(dev), up.to(dev), qt, n, k)
+        h = h.cpu()
+        assert torch.equal(torch.isnan(h.float()), torch.isnan(want.float())), m
+        inf_w = torch.isinf(want.float())
+        assert torch.equal(torch.isinf(h.float()), inf_w) and torch.equal(h[inf_w].float(), want[inf_w].float()), m
+        fin = torch.isfinite(want.float())
+        assert torch.equal(torch.signbit(h[:3][fin[:3]].float()), torch.signbit(want[:3][fin[:3]].float()))
+        assert go.rel_l2(torch.where(fin, h.float(), 0.0), torch.where(fin, want.float(), 0.0)) <= TOL, m
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_random_gated_cases(dev, c_oracle, seed):
     """Seeded random shapes across the tile boundaries: any of the ten packed formats, 17 ... 1300 rows, output widths

@@ -101,3 +101,45 @@ def test_generation_tower_can_stay_resident(dev):
 
 def _padded(wrapped, group):
     return max(wrapped.store.group_nbytes(i, group) for i in range(wrapped.store.num_layers)) + 256 * 16
+
+
+def test_stacked_qkv_copy_is_released_when_the_offloader_takes_the_weights(dev):
+    """q / k / v stacked into one device tensor (what the one-call loader does by default), then wrapped for layer
+    offload: the weights move into the pinned arenas, so the stack must let go of its device copy."""
+    print("case offload releases the q|k|v stack", flush=True)
+    from sensenova_u1_amd import GGUFLinear, GGUFParameter, stack_shared_input_projections
+
+    def q(n, k, seed):
+        lin = GGUFLinear(k, n, bias=False, compute_dtype=torch.bfloat16, device="meta")
+        lin.weight = GGUFParameter(synthetic.make_packed(8, n, k, seed=seed, device=dev), quant_type=8)
+        return lin
+
+    class Attn(nn.Module):
+        def __init__(self, s):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = q(512, 512, s), q(128, 512, s + 1), q(128, 512, s + 2)
+
+        def forward(self, h):
+            return self.q_proj(h) + torch.cat([self.k_proj(h), self.v_proj(h)] * 2, dim=-1)
+
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = nn.ModuleList([Attn(10 * i) for i in range(3)])
+
+        def forward(self, h):
+            for l in self.layers:
+                h = l(h)
+            return h
+
+    model = M().eval()
+    x = synthetic.make_activations(1, 512, seed=3, device=dev)
+    want = model(x)
+    assert stack_shared_input_projections(model) == 3
+    stacks = [l.q_proj.__dict__["_shared_stack"] for l in model.layers]
+    assert torch.equal(model(x), want) and all(s.intact() for s in stacks)
+    wrapped = LayerOffloadWrapper(model, "layers", dev, prefetch_count=1)
+    assert all(s.stacked is None for s in stacks)
+    assert not any("_shared_stack" in m.__dict__ for l in model.layers for m in (l.q_proj, l.k_proj, l.v_proj))
+    assert torch.equal(wrapped(x), want)
+    wrapped.teardown()

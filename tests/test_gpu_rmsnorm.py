@@ -187,6 +187,23 @@ def test_standalone_rmsnorm_launch(dev, m, k):
     assert (got1.view(torch.int16) != go.qwen3_rms_norm(x, one, EPS).view(torch.int16)).float().mean().item() < 0.01
 
 
+@pytest.mark.parametrize("k", [4096, 16384, 20480])
+def test_standalone_rmsnorm_in_place(dev, k):
+    """y may be x: rows held in registers (K <= 16384) and rows re-read while they are written (K > 16384)."""
+    print(f"case rmsnorm in place k={k}", flush=True)
+    x = (synthetic.make_activations(3, k, seed=k).float() * 1.9).to(torch.bfloat16).to(dev)
+    gamma = _gamma(k, 4).to(dev)
+    want = ops.rms_norm(x, gamma, EPS)
+    buf = x.clone()
+    lib = ops.load_library()
+    import ctypes
+    rc = lib.sngguf_rmsnorm(ctypes.c_void_p(buf.data_ptr()), 3, k, ctypes.c_void_p(gamma.data_ptr()), ctypes.c_float(EPS),
+                            ctypes.c_void_p(buf.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(buf, want)
+
+
 def test_module_helpers_use_the_library_norm_beyond_the_fused_row_count(dev):
     from sensenova_u1_amd import GGUFLinear, GGUFParameter
     from sensenova_u1_amd.quantized_linear import rms_norm

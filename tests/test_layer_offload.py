@@ -168,3 +168,40 @@ def test_wrapper_argument_checks():
     model.norm = nn.LayerNorm(4)
     with pytest.raises(TypeError):
         LayerOffloadWrapper(model, "norm", torch.device("cuda:0"))
+
+
+def test_a_shared_input_stack_lets_go_of_its_copy_once_the_weights_have_moved():
+    """modality.SharedInputStack keeps q / k / v rows in one tensor; when a store rebinds every member's weight.data to
+    its own arena the stacked tensor has no user left and must not stay alive (the device check of the constructor is
+    side-stepped here: the bookkeeping is the same on any device)."""
+    from sensenova_u1_amd.modality import SharedInputStack
+
+    mods = [_q(64, H, 1), _q(32, H, 2), _q(32, H, 3)]
+    stack = object.__new__(SharedInputStack)
+    stack.members, stack.index = mods, {id(m): i for i, m in enumerate(mods)}
+    stack.splits = [m.out_features for m in mods]
+    stack.offsets = [0, 64, 96]
+    stack.row_bytes = mods[0].weight.shape[1]
+    stack.stacked = torch.cat([m.weight.as_tensor() for m in mods], dim=0)
+    stack._pending = None
+    for m, off in zip(mods, stack.offsets):
+        m.weight.data = stack.stacked[off:off + m.out_features]
+        m.__dict__["_shared_stack"] = stack
+    assert stack.intact() and not stack.release_if_moved() and stack.stacked is not None
+    layer = nn.Module()
+    layer.q_proj, layer.k_proj, layer.v_proj = mods
+    store = PackedLayerStore([layer], torch.device("cpu"), pin_memory=False)
+    assert stack.stacked is None and not stack.intact()
+    assert not any("_shared_stack" in m.__dict__ for m in mods)
+    assert all(id(m.weight) in store.managed_tensor_ids() for m in mods)
+    # one member moved, the others still in place: nothing is released
+    mods2 = [_q(64, H, 4), _q(32, H, 5)]
+    st2 = object.__new__(SharedInputStack)
+    st2.members, st2.index, st2.splits, st2.offsets = mods2, {id(m): i for i, m in enumerate(mods2)}, [64, 32], [0, 64]
+    st2.row_bytes, st2._pending = mods2[0].weight.shape[1], None
+    st2.stacked = torch.cat([m.weight.as_tensor() for m in mods2], dim=0)
+    for m, off in zip(mods2, st2.offsets):
+        m.weight.data = st2.stacked[off:off + m.out_features]
+        m.__dict__["_shared_stack"] = st2
+    mods2[1].weight.data = mods2[1].weight.data.clone()
+    assert not st2.intact() and st2.stacked is not None and "_shared_stack" in mods2[0].__dict__
