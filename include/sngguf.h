@@ -169,6 +169,39 @@ int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int
                          const void* bias, void* y, int numerics, void* stream);
 
 /*
+ * The SiLU-gated MLP of a decoder layer for up to 16 rows:
+ *     y = [residual +] down(silu(gate(n)) * up(n)),   n = RMSNorm(x; gamma, eps) if gamma else x
+ * i.e. Qwen3MLP.forward (src/sensenova_u1/models/neo_unify/modeling_qwen3.py:214-216) with, optionally, the
+ * post_attention_layernorm in front of it and the residual add behind it (Qwen3DecoderLayer.forward, :936-941), every
+ * rounding of the separate bf16 tensor operations kept.  x, y, residual [M][hidden], gamma [hidden] bf16;
+ * q_gate, q_up [inter][hidden], q_down [hidden][inter] packed.
+ *
+ * Where sngguf_mlp_decode_fits() says so (Q8_0 for all three, hidden 4096, inter 12288, M <= 2, one compute unit per
+ * 48-row slice of gate / up) the whole MLP is ONE launch: every workgroup computes its slice of the gated activations,
+ * hands them to the others through the workspace (8-byte words that carry the launch's generation tag beside the data)
+ * and goes on with 16 rows of the down projection as the slices it needs arrive; the down weights are requested while
+ * the slower workgroups still finish.  All workgroups of that launch must be resident
+ * together, which a device that runs nothing else at that moment guarantees.  The wait for the other workgroups is
+ * bounded (`spin_limit` polls of about a microsecond; 0 = 2^20, negative = give up at once): on giving up a workgroup
+ * sets the 32-bit word at byte sngguf_mlp_decode_status_offset() of the workspace to 1, finishes with whatever the
+ * activations hold and the launch ends normally - the caller reads that word when it synchronises, and the results
+ * of a call that set it are void.  Everything else runs as the separate launches of sngguf_[rmsnorm_]gate_up_silu
+ * and sngguf_linear[_residual] with the activations in the workspace: same values.
+ *
+ * workspace: sngguf_mlp_decode_workspace_bytes(M, hidden, inter) bytes, 256-byte aligned, all zero before the first
+ * call and the launches' own from then on (generation counter and tagged words; never cleared again, also not
+ * between replays of a captured graph).  One workspace serves one stream: calls that overlap in time on one
+ * workspace, or two one-launch calls that overlap on one device, can starve each other of compute units and time out.
+ */
+int64_t sngguf_mlp_decode_workspace_bytes(int64_t M, int64_t hidden, int64_t inter);
+int64_t sngguf_mlp_decode_status_offset(void);
+int sngguf_mlp_decode_fits(int qtype_gate_up, int qtype_down, int64_t M, int64_t hidden, int64_t inter);
+int sngguf_mlp_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up,
+                      int qtype_gate_up, const void* q_down, int qtype_down, int64_t hidden, int64_t inter,
+                      const void* residual, void* y, void* workspace, int64_t workspace_bytes, int numerics,
+                      int spin_limit, void* stream);
+
+/*
  * Measurement aid, no counterpart in the reference: one launch that reads `bytes` (rounded down to 16) of device
  * memory once - contiguous shares per workgroup, 16 bytes per lane and request, eight requests in flight per lane,
  * with (nontemporal != 0) or without the read-once cache hint - and folds them into one word per workgroup in `out`

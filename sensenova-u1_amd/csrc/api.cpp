@@ -39,6 +39,13 @@ int launch_gemm_dense_gated(const void* x, int64_t M, const void* w2, int64_t co
 int launch_gemm(const void* x, int64_t M, const void* q, int qtype, int64_t N, int64_t K, const void* bias,
                 const void* residual, void* y,
                 int numerics, hipStream_t stream);
+int64_t mlp_q8_decode_workspace_bytes(int64_t M, int64_t inter);
+int64_t mlp_q8_decode_status_offset();
+int64_t mlp_q8_decode_ctl_bytes();
+bool mlp_q8_decode_fits(int64_t M, int64_t hidden, int64_t inter);
+int launch_mlp_q8_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down,
+                         int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics, int spin_limit,
+                         hipStream_t stream);
 int64_t stream_probe_out_bytes();
 int launch_stream_read(const void* p, int64_t bytes, void* out, int workgroups, bool nontemporal, hipStream_t stream);
 int64_t grouped_workspace_bytes(int64_t M);
@@ -495,6 +502,51 @@ int sngguf_rmsnorm_gate_up_silu_tiled(const void* x, int64_t M, const void* gamm
     if (!aligned(tiled_up, 16)) return SNGGUF_E_ALIGN;
     return sngguf::launch_gemv_q8_tiled(x, M, tiled_gate, tiled_up, N, K, nullptr, nullptr, h, numerics, true,
                                         static_cast<hipStream_t>(stream), gamma, eps);
+}
+
+int64_t sngguf_mlp_decode_workspace_bytes(int64_t M, int64_t hidden, int64_t inter) {
+    if (M < 1 || M > 16 || hidden <= 0 || inter <= 0 || hidden >= kMaxDim || inter >= kMaxDim) return 0;
+    return sngguf::mlp_q8_decode_workspace_bytes(M, inter) + ((2 * M * hidden + 255) & ~(int64_t)255);
+}
+
+int64_t sngguf_mlp_decode_status_offset(void) { return sngguf::mlp_q8_decode_status_offset(); }
+
+int sngguf_mlp_decode_fits(int qtype_gate_up, int qtype_down, int64_t M, int64_t hidden, int64_t inter) {
+    return qtype_gate_up == SNGGUF_TYPE_Q8_0 && qtype_down == SNGGUF_TYPE_Q8_0 && sngguf::mlp_q8_decode_fits(M, hidden, inter);
+}
+
+int sngguf_mlp_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, int qtype_gate_up,
+                      const void* q_down, int qtype_down, int64_t hidden, int64_t inter, const void* residual, void* y,
+                      void* workspace, int64_t workspace_bytes, int numerics, int spin_limit, void* stream) {
+    int rc = check_matmul(x, M, q_gate, qtype_gate_up, inter, hidden, y, numerics);
+    if (rc != SNGGUF_OK) return rc;
+    rc = check_matmul(x, M, q_down, qtype_down, hidden, inter, y, numerics);
+    if (rc != SNGGUF_OK || M == 0 || hidden == 0 || inter == 0) return rc;
+    if (M > 16) return SNGGUF_E_BADSHAPE;
+    if (!q_up || !workspace) return SNGGUF_E_NULLPTR;
+    if (!aligned(q_up, 16) || !aligned(workspace, 256) || (residual && !aligned(residual, 16)) || (gamma && !aligned(gamma, 16)))
+        return SNGGUF_E_ALIGN;
+    if (gamma && !(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
+    if (workspace_bytes < sngguf_mlp_decode_workspace_bytes(M, hidden, inter)) return SNGGUF_E_BADSHAPE;
+    if (sngguf_mlp_decode_fits(qtype_gate_up, qtype_down, M, hidden, inter))
+        return sngguf::launch_mlp_q8_decode(x, M, gamma, eps, q_gate, q_up, q_down, hidden, inter, residual, y, workspace, numerics,
+                                            spin_limit, static_cast<hipStream_t>(stream));
+    // every other shape and type: the same arithmetic as separate launches, the gated activations (and, where the norm
+    // does not ride inside the pair's launch, the normalized rows) in the workspace
+    char* h = static_cast<char*>(workspace) + sngguf::mlp_q8_decode_ctl_bytes();
+    char* xn = static_cast<char*>(workspace) + sngguf::mlp_q8_decode_workspace_bytes(M, inter);
+    if (gamma && sngguf_rmsnorm_fits(qtype_gate_up, M, hidden)) {
+        rc = sngguf_rmsnorm_gate_up_silu(x, M, gamma, eps, q_gate, q_up, qtype_gate_up, inter, hidden, h, numerics, stream);
+    } else {
+        if (gamma) {
+            rc = sngguf_rmsnorm(x, M, hidden, gamma, eps, xn, stream);
+            if (rc != SNGGUF_OK) return rc;
+        }
+        rc = sngguf_gate_up_silu(gamma ? xn : x, M, q_gate, q_up, qtype_gate_up, inter, hidden, h, numerics, stream);
+    }
+    if (rc != SNGGUF_OK) return rc;
+    return residual ? sngguf_linear_residual(h, M, q_down, qtype_down, hidden, inter, nullptr, residual, y, numerics, stream)
+                    : sngguf_linear(h, M, q_down, qtype_down, hidden, inter, nullptr, y, numerics, stream);
 }
 
 int64_t sngguf_probe_stream_read_out_bytes(void) { return sngguf::stream_probe_out_bytes(); }

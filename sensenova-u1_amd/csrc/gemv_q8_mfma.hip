@@ -17,26 +17,42 @@
 //     depend on M and the cross-lane reduction happens inside the matrix core.
 // Nothing dequantized is written to memory.
 
+#include <stddef.h>
+
 #include "sngguf_common.hpp"
 
 namespace sngguf {
 
 // CB: blocks per step.  GATED: wavefronts [0, W) work on qa (gate), [W, 2W) on qb (up).
-// XN: RMSNorm(x) with weight `gamma` is what gets contracted.  Each wavefront stages the K range it works on
-// (all M rows) in LDS behind the slabs, the workgroup adds up the sums of squares, and every wavefront then
-// normalizes its own share in place; the B fragments come from there.
-template <int NUM, int CB, bool GATED, int WMAX, bool XN = false>
-__global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,
-                                                            const uint8_t* __restrict__ qa,
-                                                            const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                            const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                            const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
-    constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
-    constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
-    constexpr int kPieces = 16 * kRowPieces;      // per slab
-    constexpr int kLoads = (kPieces + 63) / 64;   // per lane (5 or 9; the last one is partial)
-    constexpr int kSlab = 16 * kRowStep;          // LDS bytes per wavefront (4352 or 8704)
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+// XS: where the B operand comes from.  0: fragments fetched from global memory one step ahead.  1: RMSNorm(x) with
+// weight `gamma` is what gets contracted - each wavefront stages the K range it works on (all M rows) in LDS behind
+// the slabs, the workgroup adds up the sums of squares, and every wavefront then normalizes its own share in place;
+// the B fragments come from there.  2: the same wavefront-private staging without a norm, read with agent-scope loads:
+// x was written by other workgroups of the SAME launch (the one-launch MLP below).
+template <int CB>
+struct CbGeom {
+    static constexpr int kRowStep = CB * 34;             // bytes of one row per step (272 or 544)
+    static constexpr int kRowPieces = kRowStep / 16;     // 16-byte pieces per row and step (17 or 34)
+    static constexpr int kPieces = 16 * kRowPieces;      // per slab
+    static constexpr int kLoads = (kPieces + 63) / 64;   // per lane (5 or 9; the last one is partial)
+    static constexpr int kSlab = 16 * kRowStep;          // LDS bytes per wavefront (4352 or 8704)
+};
+
+// The body of the block-aligned kernel for workgroup `bid` of `nblocks`, all `blockDim.x / 64` wavefronts taking part.
+// `pre` holds the first step's slab pieces if `have_pre` (requested by the caller with cb_first_fetch, so that the
+// request can be made long before the activations exist); otherwise the body requests them itself.
+template <int NUM, int CB, bool GATED, int WMAX, int XS>
+__device__ __forceinline__ void gemv_q8_cb_body(uint8_t* lds, const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
+                                                const uint8_t* __restrict__ qb, int64_t N, int64_t K, const bf16_t* __restrict__ bias,
+                                                const bf16_t* residual, bf16_t* __restrict__ y, const bf16_t* __restrict__ gamma, float eps,
+                                                uint64_t* __restrict__ amax, const int bid, const int nblocks,
+                                                u32x4_t (&pre)[CbGeom<CB>::kLoads], const bool have_pre) {
+    constexpr bool XN = XS != 0;
+    constexpr int kRowStep = CbGeom<CB>::kRowStep;
+    constexpr int kRowPieces = CbGeom<CB>::kRowPieces;
+    constexpr int kPieces = CbGeom<CB>::kPieces;
+    constexpr int kLoads = CbGeom<CB>::kLoads;
+    constexpr int kSlab = CbGeom<CB>::kSlab;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int waves = blockDim.x >> 6;
@@ -45,7 +61,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
     const uint8_t* __restrict__ q = (GATED && wave >= W) ? qb : qa;
     const int r = lane & 15, g = lane >> 4;
     const int64_t row_bytes = (K >> 5) * 34;
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t n0 = (int64_t)bid * 16;
 
     // this wavefront's share of the K steps
     const int steps = (int)(K / (32 * CB));
@@ -67,7 +83,6 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
     uint8_t* slab = lds + wave * kSlab;
 
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    u32x4_t pre[kLoads];
     auto fetch = [&](int s) {
         const uint8_t* p = base + (int64_t)s * kRowStep;
 #pragma unroll
@@ -132,9 +147,21 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
 #pragma unroll
             for (int b = 0; b < CB; b++) xa[b] = *reinterpret_cast<const u32x4_t*>(xrow + ((int64_t)s0 * CB + b) * 32);
         }
-        fetch(s0);
+        if (!have_pre) fetch(s0);
     }
-    if constexpr (XN) {
+    if constexpr (XS == 2) {
+        // this wavefront's share of the activations, written earlier in this launch by other workgroups: 8-byte
+        // agent-scope loads (they bypass whatever this compute unit's caches hold), into the wavefront's own LDS rows
+        const int pieces8 = (s1 - s0) * CB * 8;            // 8-byte pieces per row in this wavefront's K range
+        const int64_t k0 = (int64_t)s0 * CB * 32;
+        for (int m = 0; m < M; m++)
+            for (int c = lane; c < pieces8; c += 64) {
+                const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(x + (int64_t)m * K + k0 + 4 * c), __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+                *reinterpret_cast<uint64_t*>(xw + m * xrow_b + 8 * c) = v;
+            }
+    }
+    if constexpr (XS == 1) {
         // the first slab is on its way; stage and normalize this wavefront's activations underneath
         float* ssum = reinterpret_cast<float*>(lds + waves * kSlab + waves * (M * xrow_b));  // [M][waves]
         const int pieces = (s1 - s0) * CB * 4;             // 16-byte pieces per row in this wavefront's K range
@@ -203,7 +230,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
 #pragma unroll
             for (int v = 0; v < 4; v++)
                 if (n + v < N) key = u64_max(key, argmax_key(o[v], n + v));
-            argmax_store(key, g, amax, m, blockIdx.x, gridDim.x);
+            argmax_store(key, g, amax, m, bid, nblocks);
             return;
         }
     }
@@ -215,6 +242,40 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* _
         for (int v = 0; v < 4; v++)
             if (n + v < N) yr[v] = f32_to_bf16(o[v]);
     }
+}
+
+// The first step's slab pieces of wavefront `wave` of `waves` (not gated), as gemv_q8_cb_body wants them in `pre`.
+template <int CB>
+__device__ __forceinline__ void cb_first_fetch(const uint8_t* __restrict__ q, int64_t N, int64_t K, int bid, int wave, int waves, int lane,
+                                               u32x4_t (&pre)[CbGeom<CB>::kLoads]) {
+    constexpr int kRowStep = CbGeom<CB>::kRowStep, kRowPieces = CbGeom<CB>::kRowPieces, kPieces = CbGeom<CB>::kPieces,
+                  kLoads = CbGeom<CB>::kLoads;
+    const int64_t row_bytes = (K >> 5) * 34;
+    const int64_t n0 = (int64_t)bid * 16;
+    const int steps = (int)(K / (32 * CB));
+    const int s0 = (int)((int64_t)wave * steps / waves);
+    const uint8_t* p = q + n0 * row_bytes + (int64_t)s0 * kRowStep;
+#pragma unroll
+    for (int i = 0; i < kLoads; i++) {
+        const int f = lane + 64 * i;
+        const bool ok = f < kPieces;
+        const int fr = ok ? f / kRowPieces : 0, fp = ok ? f % kRowPieces : 0;
+        int64_t n = n0 + fr;
+        if (n >= N) n = N - 1;
+        if (ok) pre[i] = *reinterpret_cast<const u32x4_t*>(p + (n - n0) * row_bytes + 16 * fp);
+    }
+}
+
+template <int NUM, int CB, bool GATED, int WMAX, bool XN = false>
+__global__ __launch_bounds__(64 * WMAX) void gemv_q8_mfma_kernel(const bf16_t* __restrict__ x, int M,
+                                                            const uint8_t* __restrict__ qa,
+                                                            const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                            const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
+                                                            const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    u32x4_t pre[CbGeom<CB>::kLoads];
+    gemv_q8_cb_body<NUM, CB, GATED, WMAX, XN ? 1 : 0>(lds, x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax, (int)blockIdx.x,
+                                                      (int)gridDim.x, pre, false);
 }
 
 
@@ -239,14 +300,19 @@ constexpr int kSpanBytes = 2176;  // 64 blocks = 17 lines
 // PAIRED (gated only): one wavefront works on the gate AND the up matrix of its K range, so that each activation
 // fragment is fetched once for both - with several activation rows those fetches, not the weights, fill the
 // vector memory path (16 rows x 64 bytes per matrix instruction against 544 bytes of weights).
-template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED = false>
-__global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
-                                                                 const uint8_t* __restrict__ qa,
-                                                                 const uint8_t* __restrict__ qb, int64_t N, int64_t K,
-                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
-                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax,
-                                                                 int gpw, int skew) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+// The body of the line-aligned kernel for workgroup `bid`.  `after_loop(stores)` is called by every wavefront when it
+// has left its K loop, before the workgroup adds up the partial sums; `stores` tells whether this wavefront will write
+// outputs.  AGENT_STORES: for consumers inside the same launch, and the wavefronts of a workgroup leave the body one by
+// one instead of together (`red_lds` must then be room for the partial sums plus 64 bytes that nothing else uses).  y is then an array of 8-byte words, word (m N + n) / 2
+// = { outputs n, n + 1 of row m as two bf16, tag }, each written with one agent-scope store (it reaches memory that every
+// compute unit of the device reads): a reader that finds `tag` in a word has that word's data, whatever else has or has
+// not arrived.
+template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED, bool AGENT_STORES, typename AfterLoop>
+__device__ __forceinline__ void gemv_q8_span_body(uint8_t* lds, const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
+                                                  const uint8_t* __restrict__ qb, int64_t N, int64_t K, const bf16_t* __restrict__ bias,
+                                                  const bf16_t* residual, bf16_t* __restrict__ y, const bf16_t* __restrict__ gamma, float eps,
+                                                  uint64_t* __restrict__ amax, int gpw, int skew, const int bid, AfterLoop&& after_loop,
+                                                  const uint32_t tag = 0, const int ring_stride = 0, uint8_t* red_lds = nullptr) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     static_assert(!PAIRED || GATED, "a pair is the gate and the up matrix");
     constexpr int NQ = PAIRED ? 2 : 1;   // matrices per wavefront
@@ -275,7 +341,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     const uint8_t* __restrict__ q = (GATED && !PAIRED && lw >= W) ? qb : qa;
     const int r = lane & 15, g = lane >> 4;
     const int64_t row_bytes = (K >> 5) * 34;
-    const int64_t n0 = ((int64_t)blockIdx.x * gpw + grp) * 16;
+    const int64_t n0 = ((int64_t)bid * gpw + grp) * 16;
     const bool live = n0 < N;            // the last workgroup's row groups may lie past the end: those wavefronts idle
     const int spans = (int)(K >> 11);
     const int t0 = live ? (int)((int64_t)kw * spans / W) : 0, t1 = live ? (int)((int64_t)(kw + 1) * spans / W) : 0;
@@ -307,7 +373,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     const uint8_t* __restrict__ base = q + n0 * row_bytes;
     const uint8_t* __restrict__ base2 = qb + n0 * row_bytes;           // PAIRED: the second matrix
     constexpr int kSlab = 16 * kRingRow;
-    uint8_t* slab = lds + wave * (NQ * kSlab);                         // PAIRED: two rings per wavefront
+    // (ring_stride: bytes between the rings of consecutive wavefronts when the caller wants them further apart than
+    // they are long; red_lds: where the partial sums are added up when the caller wants the rings left alone)
+    const int wave_lds = ring_stride > 0 ? ring_stride : NQ * kSlab;
+    uint8_t* slab = lds + wave * wave_lds;                             // PAIRED: two rings per wavefront
     uint8_t* lw2 = slab + (lane >> 4) * kRingRow + 16 * (lane & 15);  // + 4 i rows, + 256 for odd groups
     uint8_t* lw1 = slab + (lane >> 3) * kRingRow + 16 * (lane & 7);   // + 8 i rows (line 16 -> ring slot 0)
     const uint8_t* lr = slab + r * kRingRow;                           // this lane's weight row
@@ -320,7 +389,7 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
     // workgroup and the B fragments come from there; otherwise they are fetched from global
     // memory one step ahead.
     const int64_t xs_stride = 2 * K + 64;   // bytes per activation row in LDS (+64: rows on different banks)
-    uint8_t* xs = lds + waves * (NQ * kSlab);
+    uint8_t* xs = lds + waves * wave_lds;
     const uint8_t* xsrow = xs + (has_x ? r : M - 1) * xs_stride + 16 * g;
 
     f32x4_t acc[NQ];
@@ -355,6 +424,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         }
     };
 
+    if constexpr (AGENT_STORES) {
+        static_assert(XLDS && !PAIRED, "the barrier of the activation staging orders the counters' reset");
+        if (tid < 16) (reinterpret_cast<uint32_t*>(reinterpret_cast<f32x4_t*>(red_lds ? red_lds : lds) + waves * 64))[tid] = 0;
+    }
     if constexpr (XLDS) {
         // weights of the first step are requested before the activations are staged
         if (npre > 0) {
@@ -491,14 +564,25 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         }
     }
 
+    after_loop(lw == 0 && live);
     // ---- add the wavefronts' partial sums (the rings are dead: reuse them) ---------------------------
-    __syncthreads();
     // per row group: [gate partial sums of the W K ranges | up partial sums][64]; the paired mode keeps the up sums of
     // all wavefronts behind the gate sums of all wavefronts
-    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);
-    red[lwave * 64 + lane] = acc[0];
-    if constexpr (PAIRED) red[(waves + lwave) * 64 + lane] = acc[NQ - 1];
-    __syncthreads();
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(red_lds ? red_lds : lds);
+    if constexpr (AGENT_STORES) {
+        // no workgroup barrier: a wavefront leaves its partial sums, counts itself in for its row group and is free; the
+        // group's storing wavefront waits for the group's count only (its partners are running and wait for nothing)
+        uint32_t* cnt = reinterpret_cast<uint32_t*>(red + waves * 64) + grp;
+        red[lwave * 64 + lane] = acc[0];
+        if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lw != 0 || !live) return;
+        while (__hip_atomic_load(cnt, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)wpg) __builtin_amdgcn_s_sleep(1);
+    } else {
+        __syncthreads();
+        red[lwave * 64 + lane] = acc[0];
+        if constexpr (PAIRED) red[(waves + lwave) * 64 + lane] = acc[NQ - 1];
+        __syncthreads();
+    }
     if (lw != 0 || !has_x || !live) return;
     f32x4_t sum = red[wbase * 64 + lane];
     for (int w = 1; w < W; w++) {
@@ -514,6 +598,12 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
         for (int w = 1; w < W; w++) {
             const f32x4_t v = red[(ubase + w) * 64 + lane];
             up[0] += v[0]; up[1] += v[1]; up[2] += v[2]; up[3] += v[3];
+        }
+        if constexpr (AGENT_STORES) {
+            // this group's partial sums have been read: counted in word 15 behind them (the caller may reuse their memory
+            // once every group of the workgroup has counted itself)
+            if (lane == 0)
+                __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(red + waves * 64) + 15, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
@@ -531,18 +621,352 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 #pragma unroll
             for (int v = 0; v < 4; v++)
                 if (n + v < N) key = u64_max(key, argmax_key(o[v], n + v));
-            argmax_store(key, g, amax, m, (int64_t)blockIdx.x * gpw + grp, (N + 15) >> 4);
+            argmax_store(key, g, amax, m, (int64_t)bid * gpw + grp, (N + 15) >> 4);
             return;
         }
     }
     bf16_t* yr = y + (int64_t)m * N + n;
     if (n + 3 < N && (N & 3) == 0) {
-        *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+        if constexpr (AGENT_STORES) {
+            uint64_t* yt = reinterpret_cast<uint64_t*>(y) + (((int64_t)m * N + n) >> 1);
+            __hip_atomic_store(yt, (uint64_t)pack_bf16(o[0], o[1]) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(yt + 1, (uint64_t)pack_bf16(o[2], o[3]) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            *reinterpret_cast<u32x2_t*>(yr) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+        }
     } else {
+        // (a ragged N: plain stores; the one caller with AGENT_STORES has N % 4 == 0)
 #pragma unroll
         for (int v = 0; v < 4; v++)
             if (n + v < N) yr[v] = f32_to_bf16(o[v]);
     }
+}
+
+template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED = false>
+__global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* __restrict__ x, int M,
+                                                                 const uint8_t* __restrict__ qa,
+                                                                 const uint8_t* __restrict__ qb, int64_t N, int64_t K,
+                                                                 const bf16_t* __restrict__ bias, const bf16_t* residual, bf16_t* __restrict__ y,
+                                                                 const bf16_t* __restrict__ gamma, float eps, uint64_t* __restrict__ amax,
+                                                                 int gpw, int skew) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    gemv_q8_span_body<NUM, GATED, WMAX, XLDS, PAIRED, false>(lds, x, M, qa, qb, N, K, bias, residual, y, gamma, eps, amax, gpw, skew,
+                                                             (int)blockIdx.x, [](bool) {});
+}
+
+// ---- the SiLU-gated MLP of a decoder layer at decode sizes in ONE launch --------------------------------------
+// down(silu(gate(x)) * up(x)) (Qwen3MLP.forward, modeling_qwen3.py:214-216), optionally with the RMSNorm in front
+// (post_attention_layernorm, :938) and the residual add behind it (:941).  Workgroup b first works as workgroup b of
+// the line-aligned gated pair (three 16-row groups of the gate / up matrices, twelve wavefronts) and writes its 48 gated
+// activations; then it contracts 16 rows of the down matrix with ALL gated activations, K split over its twelve
+// wavefronts, four steps of 8 blocks each.  The down-projection weights do not depend on the activations:
+//   * a wavefront requests its first two steps into registers the moment it leaves the first loop; the first six of
+//     a workgroup to get there also move them into LDS and decode them to matrix-core operands right away;
+//   * once the whole workgroup has left the first phase (one barrier) every wavefront requests steps 3 and 4 and
+//     decodes what it has not decoded yet - all of it while the slowest compute units still deliver activations;
+//   * when the activations of its K range are there, 32 matrix instructions and the reduction over the twelve
+//     wavefronts are all that is left.
+// So the memory system and the vector ALU stay busy through what would be the tail of one kernel, the launch gap
+// and the start of the next (35.9 us against 38.8 us for the two launches at M = 1, same process).
+//
+// Hand-over between workgroups of one launch: the activations travel as 8-byte words { two bf16, generation tag },
+// each written with one agent-scope store, so a word that shows this launch's tag carries this launch's data whatever
+// order the stores arrive in.  Behind its 16 outputs a row group also stores the tag into its flag.  A consumer
+// wavefront polls the 64 flags of the row groups its K range needs (one 4-byte agent-scope load per lane and poll, at
+// most `spin_limit` polls), then reads the words and checks every tag (a flag may overtake data; then it reads again).
+// The generation comes from MlpCtl at the start of the workspace (zero before its first use); the last workgroup to
+// finish the kernel (a trailing counter that nobody waits for) advances it, so replays of a captured launch need no
+// clearing in between.  All workgroups must be resident together (one per compute unit: the launcher checks the
+// device's unit count and the kernel's occupancy); if the poll limit is hit - another launch holding compute units for
+// that long - the wavefront sets `status`, goes on with whatever the words hold and the kernel still ends normally.
+// Inside a workgroup the first phase uses no barrier either: a wavefront leaves its partial sums in LDS and counts
+// itself in for its row group, and only that group's storing wavefront waits for the count.
+struct MlpCtl {
+    uint32_t gen, done, status, pad[61];
+    uint32_t flags[1024];   // per 16-row group of gate / up
+};
+constexpr int64_t kMlpCtlBytes = 8192;   // the tagged activation words [M][inter / 2] follow at this offset
+
+#ifdef SNGGUF_MLP_TRACE
+__device__ uint64_t g_mlp_trace[256 * 12 * 8];
+#define MLP_TRACE(slot) do { if (lane == 0) g_mlp_trace[((int)blockIdx.x * 12 + wave) * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define MLP_TRACE(slot) do { } while (0)
+#endif
+
+constexpr int kMlpWaveLds = 2 * CbGeom<8>::kSlab;   // per wavefront: its ring of the first phase, two slabs of the second
+constexpr int kEarlyDecoders = 6;                   // wavefronts per workgroup that decode two steps while the others finish
+
+template <int NUM>
+__global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q_gate,
+                                                            const uint8_t* __restrict__ q_up, const uint8_t* __restrict__ q_down,
+                                                            int64_t hidden, int64_t inter, const bf16_t* __restrict__ gamma, float eps,
+                                                            const bf16_t* residual, bf16_t* __restrict__ y, MlpCtl* ctl,
+                                                            uint64_t* ht, int spin_limit) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int CB = 8, kWaves = 12;
+    constexpr int kRowStep = CbGeom<CB>::kRowStep, kLoads = CbGeom<CB>::kLoads, kSlab = CbGeom<CB>::kSlab;
+    static_assert(kMlpWaveLds >= 16 * kRingRow, "a wavefront's two slabs take the place of its ring");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bid = (int)blockIdx.x, nb = (int)gridDim.x;
+    const int r = lane & 15, g = lane >> 4;
+    MLP_TRACE(0);
+    // this launch's tag: nobody advances the generation before every workgroup, this one included, has finished
+    const uint32_t gen = __hip_atomic_load(&ctl->gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t tag = gen + 1u;
+
+    // LDS: [12 x (ring | two slabs)] [x staged for the first phase (M rows)] [partial sums of the first phase];
+    // the second phase's activations go where the last two were
+    uint8_t* const after_rings = lds + kWaves * kMlpWaveLds;
+    uint8_t* const red_a = after_rings + (((size_t)M * (2 * hidden + 64) + (gamma ? 4 * M * kWaves : 0) + 255) & ~(size_t)255);
+
+    // ---- down projection, geometry: rows [16 bid, +16), this wavefront's steps [s0, s0 + nst) of 8 blocks ----
+    constexpr int kSteps = 4;   // steps per wavefront: inter = 12 wavefronts x 4 steps x 256 elements (the launcher checks)
+    const int s0 = wave * kSteps;
+    const int64_t drow_bytes = (inter >> 5) * 34;
+    const uint8_t* __restrict__ dbase = q_down + (int64_t)bid * 16 * drow_bytes;
+    u32x4_t pre[kLoads], pre2[kLoads];
+    auto dfetch = [&](int s, u32x4_t (&dst)[kLoads]) {
+        const uint8_t* p = dbase + (int64_t)s * kRowStep;
+#pragma unroll
+        for (int i = 0; i < kLoads; i++) {
+            const int f = lane + 64 * i;
+            const bool ok = f < CbGeom<CB>::kPieces;
+            const int fr = ok ? f / CbGeom<CB>::kRowPieces : 0, fp = ok ? f % CbGeom<CB>::kRowPieces : 0;
+            if (ok) dst[i] = *reinterpret_cast<const u32x4_t*>(p + fr * drow_bytes + 16 * fp);
+        }
+    };
+    uint8_t* const slab0 = lds + wave * kMlpWaveLds;
+    auto to_slab = [&](int which, const u32x4_t (&src)[kLoads]) {
+#pragma unroll
+        for (int i = 0; i < kLoads; i++)
+            if (lane + 64 * i < CbGeom<CB>::kPieces) *reinterpret_cast<u32x4_t*>(slab0 + which * kSlab + 16 * (lane + 64 * i)) = src[i];
+    };
+
+    // ---- decode the four steps into matrix-core operands while the activations are still on their way ----
+    // (this wavefront's ring is its own again; the vector ALU has room while other wavefronts wait for memory, and once
+    // the activations are there only the 32 matrix instructions are left)
+    u32x4_t afrag[kSteps * CB];
+    auto decode = [&](int i, int which) {
+        const uint8_t* sl = slab0 + which * kSlab;
+        const uint8_t* lrow = sl + r * kRowStep + 8 * g;
+#pragma unroll
+        for (int b = 0; b < CB; b++) {
+            const uint16_t d = *reinterpret_cast<const uint16_t*>(sl + r * kRowStep + 34 * b);
+            uint32_t q0, q1;
+            if ((b & 1) == 0) {
+                const uint32_t* w = reinterpret_cast<const uint32_t*>(lrow + 34 * b);
+                const uint32_t w0v = w[0], w1v = w[1], w2v = w[2];
+                q0 = __builtin_amdgcn_alignbit(w1v, w0v, 16);
+                q1 = __builtin_amdgcn_alignbit(w2v, w1v, 16);
+            } else {
+                const uint32_t* w = reinterpret_cast<const uint32_t*>(lrow + 34 * b + 2);
+                q0 = w[0];
+                q1 = w[1];
+            }
+            uint32_t a0, a1, a2, a3;
+            q8_dword_bf16<NUM>(d, q0, a0, a1);
+            q8_dword_bf16<NUM>(d, q1, a2, a3);
+            afrag[i * CB + b] = u32x4_t{a0, a1, a2, a3};
+        }
+    };
+    int did_early = 0;
+    // ---- gate / up / SiLU: activations [48 bid, +48) of every row, as tagged words ----
+    // Measured on 12288 x 4096 at M = 1 against the two separate launches in one process (37.3 / 38.8 us on two devices):
+    // no barrier between the phases, every wavefront fetching and decoding its four steps as soon as it is free, 40.4 us -
+    // the early traffic and arithmetic slow the first phase's last wavefronts, which everything waits for; a workgroup
+    // barrier before steps 2 and 3 are requested 36.6 / 37.1 us; with the first six wavefronts decoding steps 0 and 1
+    // in front of that barrier 35.9 us (eight: 36.1, ten: 36.6).
+    __builtin_amdgcn_s_setprio(2);   // the first phase is what every other workgroup waits for
+    gemv_q8_span_body<NUM, true, 12, true, false, true>(
+        lds, x, M, q_gate, q_up, inter, hidden, nullptr, nullptr, reinterpret_cast<bf16_t*>(ht), gamma, eps, nullptr, 3, 1, bid,
+        [&](bool stores) {
+            MLP_TRACE(1);
+            // the first two down-projection steps, requested the moment this wavefront leaves the loop
+            dfetch(s0, pre);
+            dfetch(s0 + 1, pre2);
+            // the first kEarlyDecoders wavefronts of the workgroup to get here have microseconds until the last one does:
+            // they decode those two steps now, at the lowest priority, instead of idling at the barrier
+            uint32_t* order = reinterpret_cast<uint32_t*>(red_a + kWaves * 64 * 16) + 14;
+            uint32_t nth = 0;
+            if (lane == 0) nth = __hip_atomic_fetch_add(order, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            nth = __builtin_amdgcn_readfirstlane(nth);
+            if (nth < (uint32_t)kEarlyDecoders) {
+                __builtin_amdgcn_s_setprio(0);
+                to_slab(0, pre);
+                to_slab(1, pre2);
+                decode(0, 0);
+                decode(1, 1);
+                did_early = 1;
+            }
+        },
+        tag, kMlpWaveLds, red_a);
+    // a wavefront that wrote a row group's activations also raises that group's flag (behind the data, unordered)
+    {
+        // the body's storing wavefronts are those with lw == 0 in its [group][matrix][K half] order: recomputed here
+        const int slot = wave >> 2, i4 = wave & 3;
+        const int pair = slot == 1 ? 4 + (i4 >> 1) : i4;
+        const int khalf = slot == 1 ? (i4 & 1) : (slot >> 1);
+        const int lwave = 2 * pair + khalf;
+        if ((lwave & 3) == 0 && lane == 0)
+            __hip_atomic_store(&ctl->flags[3 * bid + (lwave >> 2)], tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    MLP_TRACE(2);
+    __syncthreads();   // (all of the workgroup's first-phase requests have been served: now the rest of the second phase's)
+
+    did_early = __builtin_amdgcn_readfirstlane(did_early);
+    if (!did_early) {
+        to_slab(0, pre);
+        to_slab(1, pre2);
+    }
+    dfetch(s0 + 2, pre);
+    dfetch(s0 + 3, pre2);
+    if (!did_early) {
+        decode(0, 0);
+        decode(1, 1);
+    }
+    to_slab(0, pre);
+    to_slab(1, pre2);
+    decode(2, 0);
+    decode(3, 1);
+    MLP_TRACE(6);
+    MLP_TRACE(3);
+
+    // ---- wait for this wavefront's K range of the activations ----
+    // staged (tags stripped) as [M][xrow_b] bytes; fragment (step i, block b) of row m at ((i CB + b) 64 + 16 g)
+    const int xrow_b = kSteps * CB * 64 + 16;
+    uint8_t* xw = after_rings + wave * (M * xrow_b);
+    {
+        const int pairs = kSteps * CB * 8;            // 16-byte pairs of words per row in this wavefront's K range (256)
+        const int64_t w0 = (int64_t)s0 * CB * 16;     // first word of the range within a row
+        const int64_t row_words = inter >> 1;
+        // the row groups whose outputs are this range: 16 outputs each
+        const int g0 = (s0 * CB * 32) >> 4, ng = (kSteps * CB * 32) >> 4;
+        int polls = 0;
+        bool gave_up = false;
+        for (;;) {
+            bool all = true;
+            for (int j = lane; j < ng; j += 64) all = all && __hip_atomic_load(&ctl->flags[g0 + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+            if (__builtin_amdgcn_ballot_w64(!all) == 0) break;
+            if (++polls > spin_limit) { gave_up = true; break; }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        // the staged copy goes where the first phase kept x and its partial sums: every wavefront of THIS workgroup must
+        // have left that phase and its three storing wavefronts must have read the sums (they count themselves in LDS;
+        // all of them are running and wait for nothing, so this wait ends)
+        {
+            const uint32_t* done_reading = reinterpret_cast<const uint32_t*>(red_a + kWaves * 64 * 16) + 15;
+            while (__hip_atomic_load(done_reading, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < 3u) __builtin_amdgcn_s_sleep(1);
+        }
+        for (;;) {
+            bool all = true;
+            for (int m = 0; m < M; m++)
+                for (int c = lane; c < pairs; c += 64) {
+                    const uint64_t* src = ht + (int64_t)m * row_words + w0 + 2 * c;
+                    const uint64_t a = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint64_t b = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    all = all && (uint32_t)(a >> 32) == tag && (uint32_t)(b >> 32) == tag;
+                    *reinterpret_cast<uint64_t*>(xw + m * xrow_b + 8 * c) = (uint64_t)(uint32_t)a | (b << 32);
+                }
+            if (gave_up || __builtin_amdgcn_ballot_w64(!all) == 0) break;
+            if (++polls > spin_limit) { gave_up = true; break; }
+        }
+        if (gave_up && lane == 0) __hip_atomic_store(&ctl->status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    MLP_TRACE(4);
+
+    // ---- contract ----
+    __builtin_amdgcn_s_setprio(3);
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const bool has_x = r < M;
+    const uint8_t* xwrow = xw + (has_x ? r : M - 1) * xrow_b + 16 * g;
+#pragma unroll
+    for (int i = 0; i < kSteps * CB; i++) {
+        const u32x4_t xfrag = *reinterpret_cast<const u32x4_t*>(xwrow + i * 64);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afrag[i]), __builtin_bit_cast(bf16x8_t, xfrag), acc, 0, 0, 0);
+    }
+
+    // ---- add the wavefronts' partial sums, residual, store ----
+    __syncthreads();
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [waves][64]
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == 0 && has_x) {
+        f32x4_t sum = red[lane];
+        for (int w = 1; w < kWaves; w++) {
+            const f32x4_t t = red[w * 64 + lane];
+            sum[0] += t[0]; sum[1] += t[1]; sum[2] += t[2]; sum[3] += t[3];
+        }
+        const int64_t n = (int64_t)bid * 16 + 4 * g;
+        float o[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = add_residual(sum[v], residual, (int64_t)r * hidden + n + v);
+        *reinterpret_cast<u32x2_t*>(y + (int64_t)r * hidden + n) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+    }
+    MLP_TRACE(5);
+    if (tid == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&ctl->done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == (uint32_t)nb - 1u) {
+            __hip_atomic_store(&ctl->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&ctl->gen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+#ifdef SNGGUF_MLP_TRACE
+extern "C" int sngguf_debug_mlp_trace(void* host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_mlp_trace), sizeof(g_mlp_trace));
+}
+#endif
+
+int64_t mlp_q8_decode_workspace_bytes(int64_t M, int64_t inter) { return kMlpCtlBytes + ((4 * M * inter + 255) & ~(int64_t)255); }
+int64_t mlp_q8_decode_ctl_bytes() { return kMlpCtlBytes; }
+int64_t mlp_q8_decode_status_offset() { return (int64_t)offsetof(MlpCtl, status); }
+
+// Shapes the one-launch form takes: Q8_0 everywhere; hidden = 4096 (two spans per row: the twelve-wavefront form of
+// the gated pair); inter = 3 hidden (as many 48-row slices of gate / up as 16-row groups of down: one of each per
+// workgroup) and a multiple of 12 x 256 (whole steps per wavefront of the down projection); one or two rows (their
+// staged copies fit beside two slabs per wavefront); as many compute units as workgroups and the kernel resident on each.
+bool mlp_q8_decode_fits(int64_t M, int64_t hidden, int64_t inter) {
+    if (M < 1 || M > 2 || hidden != 4096 || inter != 3 * hidden || inter != 12 * 4 * 256) return false;
+    static const int ok = [] {
+        int dev = 0, cus = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        for (const void* k : {reinterpret_cast<const void*>(&mlp_q8_decode_kernel<0>), reinterpret_cast<const void*>(&mlp_q8_decode_kernel<1>)}) {
+            if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) return 0;
+        }
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mlp_q8_decode_kernel<1>, 768, 160 * 1024) != hipSuccess) return 0;
+        return per_cu >= 1 ? cus : 0;
+    }();
+    return ok >= inter / 48;
+}
+
+// x [M][hidden], y [M][hidden], residual (may be null) [M][hidden] bf16; gamma (may be null) [hidden]; workspace as
+// mlp_q8_decode_workspace_bytes says, its first kMlpCtlBytes zero before the first use and left alone between calls.
+int launch_mlp_q8_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down,
+                         int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics, int spin_limit,
+                         hipStream_t stream) {
+    if (!mlp_q8_decode_fits(M, hidden, inter)) return SNGGUF_E_BADSHAPE;
+    // [12 x two slabs] + max(x staged + sums of squares + partial sums and counters of the first phase, activations of the second)
+    const size_t first = (((size_t)M * (2 * hidden + 64) + (gamma ? (size_t)4 * M * 12 : 0) + 255) & ~(size_t)255) + (size_t)12 * 64 * 16 + 64;
+    const size_t second = (size_t)12 * M * ((size_t)(inter / 256 / 12) * 8 * 64 + 16);
+    const size_t lds_bytes = (size_t)12 * kMlpWaveLds + (first > second ? first : second);
+    if (lds_bytes > 160 * 1024) return SNGGUF_E_BADSHAPE;
+    MlpCtl* ctl = static_cast<MlpCtl*>(workspace);
+    uint64_t* h = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(workspace) + kMlpCtlBytes);
+    const dim3 grid((unsigned)(inter / 48)), block(768);
+    const int limit = spin_limit == 0 ? 1 << 20 : spin_limit < 0 ? 0 : spin_limit;
+#define SNGGUF_MLP(NUMV) \
+    mlp_q8_decode_kernel<NUMV><<<grid, block, lds_bytes, stream>>>(static_cast<const bf16_t*>(x), (int)M, static_cast<const uint8_t*>(q_gate), \
+        static_cast<const uint8_t*>(q_up), static_cast<const uint8_t*>(q_down), hidden, inter, static_cast<const bf16_t*>(gamma), eps, \
+        static_cast<const bf16_t*>(residual), static_cast<bf16_t*>(y), ctl, h, limit)
+    if (numerics == SNGGUF_NUM_GGML_FP32) SNGGUF_MLP(0);
+    else SNGGUF_MLP(1);
+#undef SNGGUF_MLP
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
 }
 
 template <int NUM>

@@ -136,15 +136,67 @@ class FusedProjections(nn.Module):
         return torch.split(y, self.splits, dim=-1)
 
 
+# Whether ``gated_mlp`` may run the whole MLP as ONE launch where the library offers it (``ops.mlp_decode_fits``: Q8_0,
+# hidden 4096, intermediate 12288, one or two rows).  That launch needs every compute unit of the device at once; a
+# process that runs kernels on several streams at the same time should switch it off.
+ONE_LAUNCH_MLP = True
+
+
+def _one_launch_mlp(x, rows, gate_proj, up_proj, down_proj, norm_weight, residual) -> bool:
+    if not (ONE_LAUNCH_MLP and 0 < rows <= 2 and x.is_cuda and x.dtype == torch.bfloat16):
+        return False
+    mods = (gate_proj, up_proj, down_proj)
+    if any(m.bias is not None or m.decode_layout != "native" or m.numerics != gate_proj.numerics or not m.weight.is_cuda
+           or (m.compute_dtype or x.dtype) != torch.bfloat16 for m in mods):
+        return False
+    if norm_weight is not None and (norm_weight.dtype != torch.bfloat16 or norm_weight.numel() != gate_proj.in_features):
+        return False
+    if residual is not None and (residual.dtype != torch.bfloat16 or tuple(residual.shape) != (*x.shape[:-1], down_proj.out_features)):
+        return False
+    if int(gate_proj.weight.quant_type) != int(up_proj.weight.quant_type):
+        return False
+    if (up_proj.in_features, up_proj.out_features) != (gate_proj.in_features, gate_proj.out_features) \
+            or (down_proj.in_features, down_proj.out_features) != (gate_proj.out_features, gate_proj.in_features):
+        return False
+    return ops.mlp_decode_fits(int(gate_proj.weight.quant_type), int(down_proj.weight.quant_type), rows, gate_proj.in_features,
+                               gate_proj.out_features)
+
+
 def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_proj: GGUFLinear,
-              norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:
+              norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``down_proj(silu(gate_proj(x)) * up_proj(x))`` (``Qwen3MLP.forward``, modeling_qwen3.py:214-216).
 
     For decode (at most 16 rows, same quant type on gate and up, no bias) the gate and up
     projections and the SiLU product run as one fused GEMV launch.  With ``norm_weight`` the MLP reads
     ``RMSNorm(x)`` (``post_attention_layernorm``, modeling_qwen3.py:938); where ``ops.rmsnorm_fits`` allows, the norm
-    is part of that same launch."""
+    is part of that same launch.  With ``residual`` the result is ``residual + mlp`` (modeling_qwen3.py:940-941), added
+    in the down projection's epilogue.  One or two rows of the 8B model's shape in Q8_0 run as ONE launch
+    (``sngguf_mlp_decode``; see ``ONE_LAUNCH_MLP``): same values as the separate launches up to the order in which the
+    down projection's partial sums are added."""
     rows = x.numel() // x.shape[-1] if x.numel() else 0
+    if _one_launch_mlp(x, rows, gate_proj, up_proj, down_proj, norm_weight, residual):
+        x2d = gate_proj._checked_rows(x, norm_weight, residual)
+        up_proj._checked_rows(x)
+        # (the down projection's input never exists as a tensor here: its packed weight is checked by itself)
+        ops._require_device(x, down_proj.weight)
+        _, dn, dk = ops._packed_2d(down_proj.weight, down_proj._weight_type())
+        if (dn, dk) != (down_proj.out_features, down_proj.in_features) or not down_proj.weight.is_contiguous():
+            raise ops.SnGgufError("gated_mlp: the down projection's packed weight does not match the module")
+        out = torch.empty((*x.shape[:-1], down_proj.out_features), dtype=torch.bfloat16, device=x.device)
+        res2d = residual.reshape(-1, down_proj.out_features).contiguous() if residual is not None else None
+        ws = ops.mlp_decode_workspace(x.device, rows, gate_proj.in_features, gate_proj.out_features)
+        ops.mlp_decode_into(x2d, norm_weight.contiguous() if norm_weight is not None else None, eps, gate_proj.weight, up_proj.weight,
+                            int(gate_proj.weight.quant_type), down_proj.weight, int(down_proj.weight.quant_type), res2d,
+                            out.view(-1, down_proj.out_features), ws, gate_proj.numerics)
+        return out
+    if residual is not None:
+        return down_proj.forward_residual(_gated_activations(x, rows, gate_proj, up_proj, norm_weight, eps), residual)
+    return down_proj(_gated_activations(x, rows, gate_proj, up_proj, norm_weight, eps))
+
+
+def _gated_activations(x, rows, gate_proj, up_proj, norm_weight, eps) -> torch.Tensor:
+    """``silu(gate_proj(n)) * up_proj(n)``, n = RMSNorm(x) if ``norm_weight`` is given else x."""
     same = int(gate_proj.weight.quant_type) == int(up_proj.weight.quant_type)
     decode = 0 < rows <= 16 and same and gate_proj.bias is None and up_proj.bias is None and x.dtype == torch.bfloat16
     if norm_weight is not None:
@@ -164,7 +216,7 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
                 ops.rmsnorm_gate_up_silu_into(x2d, norm_weight.contiguous(), eps, gate_proj.weight, up_proj.weight,
                                               int(gate_proj.weight.quant_type), h.view(-1, gate_proj.out_features),
                                               gate_proj.numerics)
-            return down_proj(h)
+            return h
         x = rms_norm(x, norm_weight, eps)
     tg = gate_proj.tiled_weight() if decode else None
     tu = up_proj.tiled_weight() if decode and tg is not None else None
@@ -189,7 +241,7 @@ def gated_mlp(x: torch.Tensor, gate_proj: GGUFLinear, up_proj: GGUFLinear, down_
                                  gate_proj.numerics)
     else:
         h = torch.nn.functional.silu(gate_proj(x)) * up_proj(x)
-    return down_proj(h)
+    return h
 
 
 # The gated launch has ceil(rows / 256) x ceil(N / 128) output tiles and no K split, so it pays when those tiles come close

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "sngguf_grouped_linear_ws", "sngguf_q8_0_tiled_bytes", "sngguf_q8_0_tile", "sngguf_linear_tiled", "sngguf_gate_up_silu_tiled",
     "sngguf_rmsnorm_fits", "sngguf_rmsnorm", "sngguf_rmsnorm_linear", "sngguf_rmsnorm_gate_up_silu",
     "sngguf_rmsnorm_linear_tiled", "sngguf_rmsnorm_gate_up_silu_tiled",
+    "sngguf_mlp_decode_workspace_bytes", "sngguf_mlp_decode_status_offset", "sngguf_mlp_decode_fits", "sngguf_mlp_decode",
     "sngguf_probe_stream_read_out_bytes", "sngguf_probe_stream_read",
     "sngguf_file_open", "sngguf_file_close", "sngguf_file_version", "sngguf_file_alignment", "sngguf_file_tensor_count",
     "sngguf_file_tensor", "sngguf_file_metadata_count", "sngguf_file_metadata", "sngguf_file_read_tensors",
@@ -110,6 +111,14 @@ def load_library() -> ctypes.CDLL:
     lib.sngguf_linear_tiled.restype = ci
     lib.sngguf_gate_up_silu_tiled.argtypes = [vp, i64, vp, vp, i64, i64, vp, ci, vp]
     lib.sngguf_gate_up_silu_tiled.restype = ci
+    lib.sngguf_mlp_decode_workspace_bytes.argtypes = [i64, i64, i64]
+    lib.sngguf_mlp_decode_workspace_bytes.restype = i64
+    lib.sngguf_mlp_decode_status_offset.argtypes = []
+    lib.sngguf_mlp_decode_status_offset.restype = i64
+    lib.sngguf_mlp_decode_fits.argtypes = [ci, ci, i64, i64, i64]
+    lib.sngguf_mlp_decode_fits.restype = ci
+    lib.sngguf_mlp_decode.argtypes = [vp, i64, vp, ctypes.c_float, vp, vp, ci, vp, ci, i64, i64, vp, vp, vp, i64, ci, ci, vp]
+    lib.sngguf_mlp_decode.restype = ci
     lib.sngguf_probe_stream_read_out_bytes.argtypes = []
     lib.sngguf_probe_stream_read_out_bytes.restype = i64
     lib.sngguf_probe_stream_read.argtypes = [vp, i64, vp, ci, ci, vp]
@@ -269,6 +278,60 @@ def pooled_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
 def release_workspaces() -> None:
     """Drop the pooled workspaces (they are reallocated on the next call that needs one)."""
     _workspaces.clear()
+    _mlp_workspaces.clear()
+
+
+_mlp_workspaces: dict = {}
+_MLP_CTL_BYTES = 8192
+
+
+def mlp_decode_fits(qt_gate_up: int, qt_down: int, m: int, hidden: int, inter: int) -> bool:
+    """Whether ``mlp_decode_into`` runs this MLP as one launch (else it runs the separate launches, same values)."""
+    return bool(load_library().sngguf_mlp_decode_fits(int(qt_gate_up), int(qt_down), m, hidden, inter))
+
+
+def mlp_decode_workspace_bytes(m: int, hidden: int, inter: int) -> int:
+    return int(load_library().sngguf_mlp_decode_workspace_bytes(m, hidden, inter))
+
+
+def mlp_decode_workspace(dev: torch.device, m: int, hidden: int, inter: int) -> torch.Tensor:
+    """The persistent workspace of ``mlp_decode_into`` for ``dev`` (one per device, grown on demand): its first 8 KB are
+    zero when it is created and belong to the launches from then on.  Calls that may overlap in time on one device
+    (several streams) need workspaces of their own: allocate them with ``torch.zeros``."""
+    nbytes = mlp_decode_workspace_bytes(m, hidden, inter)
+    if nbytes <= 0:
+        raise SnGgufError(f"mlp_decode: no workspace for {m} rows, hidden {hidden}, intermediate {inter}")
+    key = dev.index if dev.index is not None else torch.cuda.current_device()
+    ws = _mlp_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        # (created while a graph is being captured, the tensor lives in the graph's pool and is zeroed by every replay:
+        # still a valid start state; the reference kept here keeps the pool from handing its memory out again)
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        _mlp_workspaces[key] = ws
+    return ws
+
+
+def mlp_decode_gave_up(workspace: torch.Tensor) -> bool:
+    """Whether a one-launch call on this workspace ever gave up waiting for the other workgroups (its results are void
+    then).  Reads device memory: synchronises."""
+    off = int(load_library().sngguf_mlp_decode_status_offset())
+    return bool(int(workspace[off:off + 4].view(torch.int32).item()) != 0)
+
+
+def mlp_decode_into(x2d: torch.Tensor, gamma: Optional[torch.Tensor], eps: float, gate: torch.Tensor, up: torch.Tensor,
+                    qt_gate_up: int, down: torch.Tensor, qt_down: int, residual: Optional[torch.Tensor], y2d: torch.Tensor,
+                    workspace: torch.Tensor, numerics: int, spin_limit: int = 0) -> None:
+    """y2d[M, hidden] = [residual +] down(silu(gate(n)) * up(n)), n = RMSNorm(x2d; gamma, eps) if gamma is given else
+    x2d: Qwen3MLP.forward (modeling_qwen3.py:214-216) with the layer's second norm and residual add (:936-941), for up
+    to 16 rows; ONE launch where ``mlp_decode_fits`` says so."""
+    dev = x2d.device
+    m, hidden = x2d.shape
+    inter = gate.shape[0]
+    with _on(dev):
+        rc = load_library().sngguf_mlp_decode(_ptr(x2d), m, _ptr(gamma), float(eps), _ptr(gate), _ptr(up), int(qt_gate_up), _ptr(down),
+                                              int(qt_down), hidden, inter, _ptr(residual), _ptr(y2d), _ptr(workspace),
+                                              workspace.numel() * workspace.element_size(), numerics, int(spin_limit), _stream(dev))
+    _check(rc, "sngguf_mlp_decode")
 
 
 def linear_workspace_bytes(n: int, k: int) -> int:
