@@ -31,7 +31,7 @@ HIDDEN, INTER, KV = 4096, 12288, 1024
 # HBM bytes per launch of the dominant kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
 # each scaled by what the same counter reads for the plain 256 MiB elementwise copy that
 # --calibrate-copy runs in the same process; None = not measured for this build.
-MEASURED_TRAFFIC = {"gemv_gate_up_m1": 107505775, "gemm_gate_m4096": 516228558, "gemm_dense_gate_m4096": 705144046}
+MEASURED_TRAFFIC = {"mlp_one_launch_m1": None, "gemv_gate_up_m1": 107505775, "gemm_gate_m4096": 516228558, "gemm_dense_gate_m4096": 705144046}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -163,6 +163,7 @@ def main() -> None:
         return (t1 - t0) * 1e3, e0.elapsed_time(e1)
 
     def mlp_leg(m: int, n_steps: int, warmup: int, layers=layers, gate_up_type: int = Q8_0, down_type: int = Q8_0):
+        """The MLP step as two launches (fused gate/up + SiLU, then down), and each of the two alone."""
         x = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
         h = torch.empty((m, INTER), dtype=torch.bfloat16, device=dev)
         y = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
@@ -185,13 +186,66 @@ def main() -> None:
         _, ev_dn = run_region(down_only, n_steps, warmup)
         return wall, ev, ev_gu / n_steps, ev_dn / n_steps
 
-    wall1, ev1, gu_ms, dn_ms = mlp_leg(1, K, W)
+    def mlp_one_launch_leg(m: int, n_steps: int, warmup: int):
+        """The MLP step as modality.gated_mlp runs it by default for one or two rows: sngguf_mlp_decode, ONE launch."""
+        x = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
+        y = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
+        ws = torch.zeros(ops.mlp_decode_workspace_bytes(m, HIDDEN, INTER), dtype=torch.uint8, device=dev)
+        nl = len(layers)
+
+        def step(i):
+            gate, up, down = layers[i % nl]
+            ops.mlp_decode_into(x, None, 1e-6, gate, up, Q8_0, down, Q8_0, None, y, ws, num)
+
+        wall, ev = run_region(step, n_steps, warmup)
+        torch.cuda.synchronize()
+        if ops.mlp_decode_gave_up(ws):
+            raise RuntimeError("bench.py: a one-launch MLP gave up waiting for its workgroups; the figure would be void")
+        return wall, ev
+
+    one_launch = ops.mlp_decode_fits(Q8_0, Q8_0, 1, HIDDEN, INTER)
+    wall2, ev2, gu_ms, dn_ms = mlp_leg(1, K, W)
     step_bytes = mlp_bytes(1)
+    if one_launch:
+        wall1, ev1 = mlp_one_launch_leg(1, K, W)
+    else:
+        wall1, ev1 = wall2, ev2
     ms_per_step = wall1 / K
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     gu_bytes = 2 * linear_bytes(1, INTER, HIDDEN)
     gu_gbps = gu_bytes / (gu_ms * 1e-3) / 1e9
     dn_bytes = linear_bytes(1, HIDDEN, INTER)
+    dev_gbps = step_bytes / (ev1 / K * 1e-3) / 1e9
+    two_gbps = step_bytes / (wall2 / K * 1e-3) / 1e9
+
+    if one_launch:
+        roofline = {
+            "kernel": "sngguf::mlp_q8_decode_kernel<upstream_fp16> (gate/up + SiLU + down of the M=1 MLP in one launch: the whole step)",
+            "bound": "hbm",
+            "achieved": round(dev_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dev_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC["mlp_one_launch_m1"],
+            "bytes_per_launch": step_bytes,
+            "avg_launch_us": round(ev1 / K * 1e3, 3),
+            "device_ms_per_step": round(ev1 / K, 6),
+            "timing": "HIP events on the launch stream around the timed replay of the graph of `steps` launches",
+        }
+    else:
+        roofline = {
+            "kernel": "sngguf::gemv_q8_span_kernel<upstream_fp16, gated> (fused gate/up + SiLU, M=1)",
+            "bound": "hbm",
+            "achieved": round(gu_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gu_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC["gemv_gate_up_m1"],
+            "bytes_per_launch": gu_bytes,
+            "avg_launch_us": round(gu_ms * 1e3, 3),
+            "device_ms_per_step": round(ev1 / K, 6),
+            "timing": "HIP events on the launch stream around the timed replay of a graph of `steps` gate/up launches",
+        }
 
     result = {
         "metric": "Q8_0 dequant-GEMV HBM GB/s (% of peak); M=4096 dequant-GEMM TFLOP/s",
@@ -208,7 +262,9 @@ def main() -> None:
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: Q8_0 MLP of one decoder layer, text decode M=1 "
-                        "(gate/up 4096->12288 fused with SiLU, down 12288->4096)",
+                        "(gate/up 4096->12288 with SiLU, down 12288->4096)",
+            "route": ("sngguf_mlp_decode: the whole MLP in one launch (what modality.gated_mlp runs by default for one or two rows)"
+                      if one_launch else "sngguf_gate_up_silu + sngguf_linear: two launches"),
             "layers_rotated": L,
             "bytes_per_step": step_bytes,
             "graph": not args.no_graph,
@@ -218,24 +274,22 @@ def main() -> None:
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "device_ms_per_step": round(ev1 / K, 6),
-        "roofline": {
-            "kernel": "sngguf::gemv_q8_span_kernel<upstream_fp16, gated> (fused gate/up + SiLU, M=1)",
-            "bound": "hbm",
-            "achieved": round(gu_gbps, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(gu_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC["gemv_gate_up_m1"],
-            "bytes_per_launch": gu_bytes,
-            "avg_launch_us": round(gu_ms * 1e3, 3),
-            "device_ms_per_step": round(ev1 / K, 6),
-            "timing": "HIP events on the launch stream around the timed replay of a graph of `steps` gate/up launches",
-        },
-        "down_proj": {
-            "kernel": "sngguf::gemv_q8_mfma_kernel<upstream_fp16> (down 12288->4096, M=1)",
-            "achieved": round(dn_bytes / (dn_ms * 1e-3) / 1e9, 1),
-            "unit": "GB/s",
-            "avg_launch_us": round(dn_ms * 1e3, 3),
+        "roofline": roofline,
+        "two_launches": {
+            "what": "the same step as sngguf_gate_up_silu + sngguf_linear (modality.ONE_LAUNCH_MLP = False, and every row count "
+                    "beyond two): the fused gate/up + SiLU kernel, then the down projection",
+            "value": round(two_gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100.0 * two_gbps / HBM_PEAK_GBPS, 2),
+            "ms_per_step": round(wall2 / K, 6), "device_ms_per_step": round(ev2 / K, 6),
+            "gate_up": {
+                "kernel": "sngguf::gemv_q8_span_kernel<upstream_fp16, gated> (fused gate/up + SiLU, M=1)",
+                "achieved": round(gu_gbps, 1), "unit": "GB/s", "frac": round(gu_gbps / HBM_PEAK_GBPS, 4),
+                "traffic": MEASURED_TRAFFIC["gemv_gate_up_m1"], "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_ms * 1e3, 3),
+            },
+            "down_proj": {
+                "kernel": "sngguf::gemv_q8_mfma_kernel<upstream_fp16> (down 12288->4096, M=1)",
+                "achieved": round(dn_bytes / (dn_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "frac": round(dn_bytes / (dn_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "bytes_per_launch": dn_bytes, "avg_launch_us": round(dn_ms * 1e3, 3),
+            },
         },
     }
 
@@ -277,8 +331,9 @@ def main() -> None:
             "achievable_at_gate_up_launch_size_GBps": best_chunk,
         }
         result["roofline"]["achievable_hbm_read_GBps"] = best
-        result["roofline"]["achievable_at_this_launch_size_GBps"] = best_chunk
-        result["roofline"]["frac_of_achievable_at_this_launch_size"] = round(gu_gbps / best_chunk, 4)
+        result["roofline"]["frac_of_achievable"] = round(result["roofline"]["achieved"] / best, 4)
+        result["two_launches"]["gate_up"]["achievable_at_this_launch_size_GBps"] = best_chunk
+        result["two_launches"]["gate_up"]["frac_of_achievable_at_this_launch_size"] = round(gu_gbps / best_chunk, 4)
         del probe_buf, probe_out
 
     # ---- same MLP at M = 4 and 16 --------------------------------------------------------------
@@ -462,6 +517,15 @@ def main() -> None:
             ops.rmsnorm_gate_up_silu_into(hid, gammas[1], eps, gate, up, Q8_0, h1, num)
             ops.linear_residual_into(h1, down, Q8_0, None, hid, yo, num)
 
+        # ... with the MLP, its norm and its residual add as ONE launch: three launches per layer
+        ws_l = torch.zeros(ops.mlp_decode_workspace_bytes(1, HIDDEN, INTER), dtype=torch.uint8, device=dev)
+
+        def layer_three_launches(i):
+            ops.rmsnorm_linear_into(x1, gammas[0], eps, qkv[i % nl], Q8_0, None, yqkv, num)
+            gate, up, down = layers[i % len(layers)]
+            ops.linear_residual_into(yq, attn[i % nl][3], Q8_0, None, res, hid, num)
+            ops.mlp_decode_into(hid, gammas[1], eps, gate, up, Q8_0, down, Q8_0, hid, yo, ws_l, num)
+
         # ... and on the tiled copies of all seven weights
         t_mlp = [tuple(ops.q8_0_tile(t) for t in layer) for layer in layers]
         t_qkv = [ops.q8_0_tile(w) for w in qkv]
@@ -482,6 +546,8 @@ def main() -> None:
                                    ("stacked_qkv_fused_residual", layer_stacked_residual, "4 linears"),
                                    ("with_norms_separate", layer_norms_separate, "4 linears + 2 torch rms_norm"),
                                    ("with_norms_fused", layer_norms_fused, "4 linears, both RMSNorms inside the q|k|v and gate/up launches"),
+                                   ("with_norms_fused_one_launch_mlp", layer_three_launches,
+                                    "q|k|v with its norm, o with its residual add, and the whole MLP with norm and residual add as one launch: 3 launches"),
                                    ("tiled_with_norms_fused", layer_tiled_norms_fused,
                                     "as with_norms_fused on the operand-order (tiled) copies of the seven weights")):
             wall_l, _ = run_region(fn, k3, min(W, 16))
