@@ -660,10 +660,10 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 // the line-aligned gated pair (three 16-row groups of the gate / up matrices, twelve wavefronts) and writes its 48 gated
 // activations; then it contracts 16 rows of the down matrix with ALL gated activations, K split over its twelve
 // wavefronts, four steps of 8 blocks each.  The down-projection weights do not depend on the activations:
-//   * a wavefront requests its first two steps into registers the moment it leaves the first loop; the first six of
-//     a workgroup to get there also move them into LDS and decode them to matrix-core operands right away;
+//   * a wavefront requests its first two steps into registers the moment it leaves the first loop, hands in its
+//     partial sums, moves the two steps into LDS and decodes them to matrix-core operands;
 //   * once the whole workgroup has left the first phase (one barrier) every wavefront requests steps 3 and 4 and
-//     decodes what it has not decoded yet - all of it while the slowest compute units still deliver activations;
+//     decodes them too - all of it while the slowest compute units still deliver activations;
 //   * when the activations of its K range are there, 32 matrix instructions and the reduction over the twelve
 //     wavefronts are all that is left.
 // So the memory system and the vector ALU stay busy through what would be the tail of one kernel, the launch gap
@@ -695,7 +695,6 @@ __device__ uint64_t g_mlp_trace[256 * 12 * 8];
 #endif
 
 constexpr int kMlpWaveLds = 2 * CbGeom<8>::kSlab;   // per wavefront: its ring of the first phase, two slabs of the second
-constexpr int kEarlyDecoders = 6;                   // wavefronts per workgroup that decode two steps while the others finish
 
 template <int NUM>
 __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q_gate,
@@ -771,13 +770,12 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
             afrag[i * CB + b] = u32x4_t{a0, a1, a2, a3};
         }
     };
-    int did_early = 0;
     // ---- gate / up / SiLU: activations [48 bid, +48) of every row, as tagged words ----
-    // Measured on 12288 x 4096 at M = 1 against the two separate launches in one process (37.3 / 38.8 us on two devices):
-    // no barrier between the phases, every wavefront fetching and decoding its four steps as soon as it is free, 40.4 us -
-    // the early traffic and arithmetic slow the first phase's last wavefronts, which everything waits for; a workgroup
-    // barrier before steps 2 and 3 are requested 36.6 / 37.1 us; with the first six wavefronts decoding steps 0 and 1
-    // in front of that barrier 35.9 us (eight: 36.1, ten: 36.6).
+    // Measured on 12288 x 4096 at M = 1 against the two separate launches in one process (37.3 ... 39.5 us, by device):
+    // every wavefront fetching and decoding all four steps as soon as it is free, no barrier, 40.4 us (56 us when only
+    // the first few to arrive do so); a workgroup barrier before steps 2 and 3 are requested and all decoding behind it
+    // 36.6 ... 37.1 us; steps 0 and 1 decoded in front of that barrier by every wavefront 35.5 us (by the first six or
+    // eight to arrive only: 36.4 us).
     __builtin_amdgcn_s_setprio(2);   // the first phase is what every other workgroup waits for
     gemv_q8_span_body<NUM, true, 12, true, false, true>(
         lds, x, M, q_gate, q_up, inter, hidden, nullptr, nullptr, reinterpret_cast<bf16_t*>(ht), gamma, eps, nullptr, 3, 1, bid,
@@ -786,20 +784,6 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
             // the first two down-projection steps, requested the moment this wavefront leaves the loop
             dfetch(s0, pre);
             dfetch(s0 + 1, pre2);
-            // the first kEarlyDecoders wavefronts of the workgroup to get here have microseconds until the last one does:
-            // they decode those two steps now, at the lowest priority, instead of idling at the barrier
-            uint32_t* order = reinterpret_cast<uint32_t*>(red_a + kWaves * 64 * 16) + 14;
-            uint32_t nth = 0;
-            if (lane == 0) nth = __hip_atomic_fetch_add(order, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            nth = __builtin_amdgcn_readfirstlane(nth);
-            if (nth < (uint32_t)kEarlyDecoders) {
-                __builtin_amdgcn_s_setprio(0);
-                to_slab(0, pre);
-                to_slab(1, pre2);
-                decode(0, 0);
-                decode(1, 1);
-                did_early = 1;
-            }
         },
         tag, kMlpWaveLds, red_a);
     // a wavefront that wrote a row group's activations also raises that group's flag (behind the data, unordered)
@@ -814,19 +798,16 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     }
     __builtin_amdgcn_s_setprio(0);
     MLP_TRACE(2);
-    __syncthreads();   // (all of the workgroup's first-phase requests have been served: now the rest of the second phase's)
-
-    did_early = __builtin_amdgcn_readfirstlane(did_early);
-    if (!did_early) {
-        to_slab(0, pre);
-        to_slab(1, pre2);
-    }
+    // steps 0 and 1 move into LDS and are decoded at once, at the lowest priority (this wavefront's partial sums are
+    // counted in: nobody waits for it); steps 2 and 3 are requested only when the whole workgroup has left the first
+    // phase - requested earlier, their traffic slows the first phase's last wavefronts, which every workgroup waits for
+    to_slab(0, pre);
+    to_slab(1, pre2);
+    decode(0, 0);
+    decode(1, 1);
+    __syncthreads();
     dfetch(s0 + 2, pre);
     dfetch(s0 + 3, pre2);
-    if (!did_early) {
-        decode(0, 0);
-        decode(1, 1);
-    }
     to_slab(0, pre);
     to_slab(1, pre2);
     decode(2, 0);
