@@ -303,10 +303,10 @@ constexpr int kSpanBytes = 2176;  // 64 blocks = 17 lines
 // The body of the line-aligned kernel for workgroup `bid`.  `after_loop(stores)` is called by every wavefront when it
 // has left its K loop, before the workgroup adds up the partial sums; `stores` tells whether this wavefront will write
 // outputs.  AGENT_STORES: for consumers inside the same launch, and the wavefronts of a workgroup leave the body one by
-// one instead of together (`red_lds` must then be room for the partial sums plus 64 bytes that nothing else uses).  y is then an array of 8-byte words, word (m N + n) / 2
-// = { outputs n, n + 1 of row m as two bf16, tag }, each written with one agent-scope store (it reaches memory that every
-// compute unit of the device reads): a reader that finds `tag` in a word has that word's data, whatever else has or has
-// not arrived.
+// one instead of together (`red_lds` must then be room for the partial sums plus 64 bytes that nothing else uses).
+// y is then an array of 8-byte words, word (m N + n) / 2 = { outputs n, n + 1 of row m as two bf16, tag }, each written
+// with one agent-scope store (it reaches memory that every compute unit of the device reads): a reader that finds
+// `tag` in a word has that word's data, whatever else has or has not arrived.
 template <int NUM, bool GATED, int WMAX, bool XLDS, bool PAIRED, bool AGENT_STORES, typename AfterLoop>
 __device__ __forceinline__ void gemv_q8_span_body(uint8_t* lds, const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ qa,
                                                   const uint8_t* __restrict__ qb, int64_t N, int64_t K, const bf16_t* __restrict__ bias,
@@ -599,12 +599,6 @@ __device__ __forceinline__ void gemv_q8_span_body(uint8_t* lds, const bf16_t* __
             const f32x4_t v = red[(ubase + w) * 64 + lane];
             up[0] += v[0]; up[1] += v[1]; up[2] += v[2]; up[3] += v[3];
         }
-        if constexpr (AGENT_STORES) {
-            // this group's partial sums have been read: counted in word 15 behind them (the caller may reuse their memory
-            // once every group of the workgroup has counted itself)
-            if (lane == 0)
-                __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(red + waves * 64) + 15, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const float gt = bf16_to_f32(f32_to_bf16(sum[v]));
@@ -694,7 +688,8 @@ __device__ uint64_t g_mlp_trace[256 * 12 * 8];
 #define MLP_TRACE(slot) do { } while (0)
 #endif
 
-constexpr int kMlpWaveLds = 2 * CbGeom<8>::kSlab;   // per wavefront: its ring of the first phase, two slabs of the second
+constexpr int kMlpWaveLds = 16 * kRingRow;   // per wavefront: its ring of the first phase; in the second phase one slab
+                                             // (4352 bytes) and the staged activations of rows 0 and 1 (2 x 2048 bytes)
 
 template <int NUM>
 __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q_gate,
@@ -705,7 +700,7 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int CB = 8, kWaves = 12;
     constexpr int kRowStep = CbGeom<CB>::kRowStep, kLoads = CbGeom<CB>::kLoads, kSlab = CbGeom<CB>::kSlab;
-    static_assert(kMlpWaveLds >= 16 * kRingRow, "a wavefront's two slabs take the place of its ring");
+    static_assert(kMlpWaveLds == kSlab + 2 * 2048, "a slab and two staged activation rows take the place of a wavefront's ring");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = (int)blockIdx.x, nb = (int)gridDim.x;
@@ -715,8 +710,8 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     const uint32_t gen = __hip_atomic_load(&ctl->gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t tag = gen + 1u;
 
-    // LDS: [12 x (ring | two slabs)] [x staged for the first phase (M rows)] [partial sums of the first phase];
-    // the second phase's activations go where the last two were
+    // LDS: [12 x (ring of the first phase | slab and staged activation rows of the second)] [x staged for the first
+    // phase (M rows)] [partial sums and counters of the first phase]
     uint8_t* const after_rings = lds + kWaves * kMlpWaveLds;
     uint8_t* const red_a = after_rings + (((size_t)M * (2 * hidden + 64) + (gamma ? 4 * M * kWaves : 0) + 255) & ~(size_t)255);
 
@@ -737,18 +732,18 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
         }
     };
     uint8_t* const slab0 = lds + wave * kMlpWaveLds;
-    auto to_slab = [&](int which, const u32x4_t (&src)[kLoads]) {
+    auto to_slab = [&](const u32x4_t (&src)[kLoads]) {
 #pragma unroll
         for (int i = 0; i < kLoads; i++)
-            if (lane + 64 * i < CbGeom<CB>::kPieces) *reinterpret_cast<u32x4_t*>(slab0 + which * kSlab + 16 * (lane + 64 * i)) = src[i];
+            if (lane + 64 * i < CbGeom<CB>::kPieces) *reinterpret_cast<u32x4_t*>(slab0 + 16 * (lane + 64 * i)) = src[i];
     };
 
     // ---- decode the four steps into matrix-core operands while the activations are still on their way ----
     // (this wavefront's ring is its own again; the vector ALU has room while other wavefronts wait for memory, and once
     // the activations are there only the 32 matrix instructions are left)
     u32x4_t afrag[kSteps * CB];
-    auto decode = [&](int i, int which) {
-        const uint8_t* sl = slab0 + which * kSlab;
+    auto decode = [&](int i) {
+        const uint8_t* sl = slab0;
         const uint8_t* lrow = sl + r * kRowStep + 8 * g;
 #pragma unroll
         for (int b = 0; b < CB; b++) {
@@ -801,24 +796,25 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     // steps 0 and 1 move into LDS and are decoded at once, at the lowest priority (this wavefront's partial sums are
     // counted in: nobody waits for it); steps 2 and 3 are requested only when the whole workgroup has left the first
     // phase - requested earlier, their traffic slows the first phase's last wavefronts, which every workgroup waits for
-    to_slab(0, pre);
-    to_slab(1, pre2);
-    decode(0, 0);
-    decode(1, 1);
+    to_slab(pre);
+    decode(0);
+    to_slab(pre2);
+    decode(1);
     __syncthreads();
     dfetch(s0 + 2, pre);
     dfetch(s0 + 3, pre2);
-    to_slab(0, pre);
-    to_slab(1, pre2);
-    decode(2, 0);
-    decode(3, 1);
+    to_slab(pre);
+    decode(2);
+    to_slab(pre2);
+    decode(3);
     MLP_TRACE(6);
     MLP_TRACE(3);
 
     // ---- wait for this wavefront's K range of the activations ----
-    // staged (tags stripped) as [M][xrow_b] bytes; fragment (step i, block b) of row m at ((i CB + b) 64 + 16 g)
-    const int xrow_b = kSteps * CB * 64 + 16;
-    uint8_t* xw = after_rings + wave * (M * xrow_b);
+    // staged (tags stripped), 2048 bytes per row, behind this wavefront's slab (at most two rows: the launcher checks);
+    // fragment (step i, block b) of a row at ((i CB + b) 64 + 16 g)
+    constexpr int xrow_b = kSteps * CB * 64;
+    auto xw_row = [&](int m) -> uint8_t* { return slab0 + kSlab + m * xrow_b; };
     {
         const int pairs = kSteps * CB * 8;            // 16-byte pairs of words per row in this wavefront's K range (256)
         const int64_t w0 = (int64_t)s0 * CB * 16;     // first word of the range within a row
@@ -834,13 +830,6 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
             if (++polls > spin_limit) { gave_up = true; break; }
             __builtin_amdgcn_s_sleep(2);
         }
-        // the staged copy goes where the first phase kept x and its partial sums: every wavefront of THIS workgroup must
-        // have left that phase and its three storing wavefronts must have read the sums (they count themselves in LDS;
-        // all of them are running and wait for nothing, so this wait ends)
-        {
-            const uint32_t* done_reading = reinterpret_cast<const uint32_t*>(red_a + kWaves * 64 * 16) + 15;
-            while (__hip_atomic_load(done_reading, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < 3u) __builtin_amdgcn_s_sleep(1);
-        }
         for (;;) {
             bool all = true;
             for (int m = 0; m < M; m++)
@@ -849,7 +838,7 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
                     const uint64_t a = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     const uint64_t b = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     all = all && (uint32_t)(a >> 32) == tag && (uint32_t)(b >> 32) == tag;
-                    *reinterpret_cast<uint64_t*>(xw + m * xrow_b + 8 * c) = (uint64_t)(uint32_t)a | (b << 32);
+                    *reinterpret_cast<uint64_t*>(xw_row(m) + 8 * c) = (uint64_t)(uint32_t)a | (b << 32);
                 }
             if (gave_up || __builtin_amdgcn_ballot_w64(!all) == 0) break;
             if (++polls > spin_limit) { gave_up = true; break; }
@@ -862,7 +851,7 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     __builtin_amdgcn_s_setprio(3);
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     const bool has_x = r < M;
-    const uint8_t* xwrow = xw + (has_x ? r : M - 1) * xrow_b + 16 * g;
+    const uint8_t* xwrow = xw_row(has_x ? r : M - 1) + 16 * g;
 #pragma unroll
     for (int i = 0; i < kSteps * CB; i++) {
         const u32x4_t xfrag = *reinterpret_cast<const u32x4_t*>(xwrow + i * 64);
@@ -908,8 +897,9 @@ int64_t mlp_q8_decode_status_offset() { return (int64_t)offsetof(MlpCtl, status)
 
 // Shapes the one-launch form takes: Q8_0 everywhere; hidden = 4096 (two spans per row: the twelve-wavefront form of
 // the gated pair); inter = 3 hidden (as many 48-row slices of gate / up as 16-row groups of down: one of each per
-// workgroup) and a multiple of 12 x 256 (whole steps per wavefront of the down projection); one or two rows (their
-// staged copies fit beside two slabs per wavefront); as many compute units as workgroups and the kernel resident on each.
+// workgroup) and 12 wavefronts x 4 steps x 256 elements of it per row of the down projection; one or two rows (their staged
+// copies fit behind a wavefront's slab; with three and four rows, tried with the copies elsewhere in LDS, the separate
+// launches were 3 - 6 % faster: polling and reading the tagged words grows with the rows); as many compute units as workgroups and the kernel resident on each.
 bool mlp_q8_decode_fits(int64_t M, int64_t hidden, int64_t inter) {
     if (M < 1 || M > 2 || hidden != 4096 || inter != 3 * hidden || inter != 12 * 4 * 256) return false;
     static const int ok = [] {
@@ -931,10 +921,9 @@ int launch_mlp_q8_decode(const void* x, int64_t M, const void* gamma, float eps,
                          int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics, int spin_limit,
                          hipStream_t stream) {
     if (!mlp_q8_decode_fits(M, hidden, inter)) return SNGGUF_E_BADSHAPE;
-    // [12 x two slabs] + max(x staged + sums of squares + partial sums and counters of the first phase, activations of the second)
-    const size_t first = (((size_t)M * (2 * hidden + 64) + (gamma ? (size_t)4 * M * 12 : 0) + 255) & ~(size_t)255) + (size_t)12 * 64 * 16 + 64;
-    const size_t second = (size_t)12 * M * ((size_t)(inter / 256 / 12) * 8 * 64 + 16);
-    const size_t lds_bytes = (size_t)12 * kMlpWaveLds + (first > second ? first : second);
+    // [12 x ring] + x staged + sums of squares + partial sums and counters of the first phase
+    const size_t lds_bytes = (size_t)12 * kMlpWaveLds + (((size_t)M * (2 * hidden + 64) + (gamma ? (size_t)4 * M * 12 : 0) + 255) & ~(size_t)255) +
+                             (size_t)12 * 64 * 16 + 64;
     if (lds_bytes > 160 * 1024) return SNGGUF_E_BADSHAPE;
     MlpCtl* ctl = static_cast<MlpCtl*>(workspace);
     uint64_t* h = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(workspace) + kMlpCtlBytes);

@@ -1,5 +1,5 @@
 """GPU: the decode MLP as one entry point (``sngguf_mlp_decode``): one launch at the 8B model's shape in Q8_0 for up to
-four rows, the separate launches everywhere else.  Against the separate launches of the library (the gated activations
+two rows, the separate launches everywhere else.  Against the separate launches of the library (the gated activations
 are the same kernel's, so only the down projection's order of summation differs) and against the CPU oracle on sampled
 output columns; consecutive calls, graph replays (the hand-over state advances by itself), the bounded wait."""
 import pytest
@@ -183,7 +183,7 @@ def test_gated_mlp_takes_the_one_launch_route_and_can_be_told_not_to(dev, monkey
     calls = []
     real = ops.mlp_decode_into
     monkeypatch.setattr(ops, "mlp_decode_into", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
-    for m in (1, 2, 3):
+    for m in (1, 3, 5):
         x = synthetic.make_activations(m, H, seed=m, device=dev).reshape(1, m, H)
         res = synthetic.make_activations(m, H, seed=10 + m, device=dev).reshape(1, m, H)
         for gm, rs in ((None, None), (gamma, res)):
