@@ -341,14 +341,22 @@ class SharedInputStack:
     ``modeling_qwen3.py:444,450,456`` and the ``_mot_gen`` triple at ``:602,608,614``), with their packed rows stored one
     after another in ONE device tensor and every module's ``weight.data`` a view of its rows.
 
-    The modules stay separate ``GGUFLinear`` objects and the model code stays as it is.  For a single activation row (a
-    decode step) the first member's forward runs one launch over all rows - packed GGUF rows are independent, so the stacked rows are a valid
-    weight of ``sum(out_features)`` rows - and keeps the result; the following members, called with the same tensor
-    (same storage, shape, strides and version counter), return their columns of it.  Anything else - another input,
-    more than one row, a weight that no longer lies where the stack put it (``.to()``, an offloader's rebinding) -
-    falls back to the member's own launch, so the stack never changes what a call returns, only how many launches
-    a decode step needs (three -> one: the 4096 -> 1024 k / v launches cost more in launch overhead than in bytes).
-    Outputs of one step are ranges of one buffer: contiguous and disjoint, but not separately allocated."""
+    The modules stay separate ``GGUFLinear`` objects and the model code stays as it is.  The first member's forward runs
+    one launch over all rows - packed GGUF rows are independent, so the stacked rows are a valid weight of
+    ``sum(out_features)`` rows - and keeps the result; the following members, called with the same tensor (same
+    storage, shape, strides and version counter), return their columns of it.  Anything else - another input, a weight
+    that no longer lies where the stack put it (``.to()``, an offloader's rebinding) - falls back to the member's own
+    launch.  At decode that is one launch instead of three (the 4096 -> 1024 k / v launches cost more in launch overhead
+    than in bytes); over thousands of image rows one launch of 384 large tiles instead of 256 + 64 + 64 (k / v alone have
+    too few tiles to fill the chip).  Every output is the same dot product of the same rounded operands as the member's
+    own launch computes; beyond 64 rows the order in which the K steps' fp32 sums are added can differ (the narrow
+    members' own launches split K over workgroups), i.e. the last place of a bf16 output now and then.
+    Outputs of one step are ranges of one buffer: disjoint, every row contiguous, but not separately allocated - with
+    several rows they are strided views (see ``member_forward``).  The pending result is recognised by the input's
+    address, shape, strides and version counter: a write into the input that bypasses the version counter (through
+    ``x.data`` or a raw pointer) between the members' calls is not seen."""
+
+    MULTI_ROW = True   # serve inputs of several rows too (outputs are then column ranges of one buffer)
 
     def __init__(self, members) -> None:
         members = list(members)
@@ -412,9 +420,11 @@ class SharedInputStack:
         """The member's output if the stack can supply it, else None (the member then runs its own launch)."""
         i = self.index[id(mod)]
         rows = x.numel() // mod.in_features if x.numel() else 0
-        # one row only: the members' outputs are then contiguous tensors like those of their own launches (with several
-        # rows they would be strided column ranges, which `.view(...)` calls that merge dimensions refuse)
-        if not (rows == 1 and x.is_cuda and x.dtype == torch.bfloat16):
+        # several rows: the members' outputs are column ranges of one [rows, sum(out_features)] buffer - every row
+        # contiguous, rows a fixed stride apart.  Splitting the last dimension into heads (`.view(*shape[:-1], -1, head_dim)`,
+        # modeling_qwen3.py:444,450,456) works on such a tensor; merging dimensions would need `.reshape`.  One row gives
+        # plain contiguous tensors.  MULTI_ROW switches the several-row form off.
+        if not (rows >= 1 and (rows == 1 or self.MULTI_ROW) and x.is_cuda and x.dtype == torch.bfloat16):
             if i == 0:
                 self._pending = None
             return None
@@ -424,7 +434,20 @@ class SharedInputStack:
             if len(self.members) == 1 or not self.intact():
                 return None
             first = self.members[0]
-            y = ops.linear(x, self.stacked, int(first.weight.quant_type), None, first.numerics)
+            qt = int(first.weight.quant_type)
+            if rows <= 16 or (rows <= 64 and first.in_features % 256 == 0) or first.gemm_policy == "fused" or qt == ops.BF16:
+                y = ops.linear(x, self.stacked, qt, None, first.numerics)
+            elif first.gemm_policy == "auto" and x.is_contiguous():
+                # the workspace route of a single module (quantized_linear.GGUFLinear.forward), on the stacked rows
+                n, k = self.stacked.shape[0], first.in_features
+                nbytes = ops.linear_workspace_bytes(n, k)
+                if -(-rows // 256) * -(-n // 256) <= 128:
+                    nbytes += 16 * rows * n
+                x2d = first._checked_rows(x)
+                y = torch.empty((*x.shape[:-1], n), dtype=torch.bfloat16, device=x.device)
+                ops.linear_ws_into(x2d, self.stacked, qt, None, y.view(-1, n), ops.pooled_workspace(x.device, nbytes), first.numerics)
+            else:
+                return None
             # x itself is kept with the result: while it is alive no other tensor can take its address, so an equal key
             # can only come from a tensor that shares its storage, shape, strides and version - the same values
             self._pending = (key, y, x)

@@ -445,9 +445,9 @@ def test_loader_fused_mlp_forward_matches_the_three_module_calls(tmp_path, dev):
 
 def test_loader_stacks_qkv_into_one_decode_launch(tmp_path, dev):
     """q_proj / k_proj / v_proj of an attention-shaped module loaded through load_gguf_model share one weight tensor; at
-    a single row the q call runs one launch over all rows and k / v return their ranges of it.  Every output
-    holds the tolerance against the oracle; other inputs, an input changed in place between the calls, more than one
-    row and a weight moved away from the stack all take the member's own launch."""
+    the q call runs one launch over all rows and k / v return their ranges of it (contiguous tensors for one row, strided
+    column ranges of one buffer for several).  Every output holds the tolerance against the oracle; other inputs, an
+    input changed in place between the calls and a weight moved away from the stack all take the member's own launch."""
     from sensenova_u1_amd import load_gguf_model
     from sensenova_u1_amd.gguf_file import write_gguf
     print("case loader-stacked qkv", flush=True)
@@ -495,11 +495,26 @@ def test_loader_stacks_qkv_into_one_decode_launch(tmp_path, dev):
         q.view(1, m, -1, 64), k.view(-1)                               # any reshape of the outputs works
         for name, got in (("q_proj", q), ("k_proj", k), ("v_proj", v)):
             assert go.rel_l2(got.cpu().reshape(m, -1), want(name, x.reshape(m, HK))) <= 1e-3, (name, m)
-    # several rows: the members' own launches, separate contiguous tensors
+    # several rows (decode kernel, decode kernel's 17 .. 64-row form, workspace route): still one launch; the outputs are
+    # column ranges of one buffer, whose last dimension splits into heads as the model code does it
+    for m in (5, 40, 300):
+        xm = (torch.randn(1, m, HK, generator=torch.Generator().manual_seed(m)) * 0.8).to(torch.bfloat16).to(dev)
+        q = att.q_proj(xm)
+        assert stack._pending is not None
+        k, v = att.k_proj(xm), att.v_proj(xm)
+        assert stack._pending is None
+        assert q.shape == (1, m, NQ) and k.shape == (1, m, NKV) and q.stride(-2) == NQ + 2 * NKV and not k.is_contiguous()
+        assert k.data_ptr() == q.data_ptr() + 2 * NQ and v.data_ptr() == k.data_ptr() + 2 * NKV
+        assert q.view(1, m, -1, 64).shape == (1, m, NQ // 64, 64) and v.view(1, m, -1, 64).transpose(1, 2).shape == (1, NKV // 64, m, 64)
+        for name, got in (("q_proj", q), ("k_proj", k), ("v_proj", v)):
+            assert go.rel_l2(got.cpu().reshape(m, -1), want(name, xm.reshape(m, HK))) <= 1e-3, (name, m)
+    # ... unless told not to: the members' own launches, separate contiguous tensors
     x5 = (torch.randn(1, 5, HK, generator=torch.Generator().manual_seed(5)) * 0.8).to(torch.bfloat16).to(dev)
+    stack.MULTI_ROW = False
     q, k = att.q_proj(x5), att.k_proj(x5)
     assert stack._pending is None and q.is_contiguous() and k.is_contiguous()
     assert go.rel_l2(k.cpu().reshape(5, -1), want("k_proj", x5.reshape(5, HK))) <= 1e-3
+    stack.MULTI_ROW = True
     # another tensor for k: its own launch on that tensor
     x1 = (torch.randn(1, HK, generator=torch.Generator().manual_seed(50)) * 0.8).to(torch.bfloat16).to(dev)
     x2 = (torch.randn(1, HK, generator=torch.Generator().manual_seed(51)) * 0.8).to(torch.bfloat16).to(dev)
@@ -511,10 +526,6 @@ def test_loader_stacks_qkv_into_one_decode_launch(tmp_path, dev):
     x1.mul_(0.5)
     k = att.k_proj(x1)
     assert go.rel_l2(k.cpu(), want("k_proj", x1)) <= 1e-3
-    # more rows than the decode kernels take: three launches, separate tensors
-    xl = (torch.randn(40, HK, generator=torch.Generator().manual_seed(52)) * 0.8).to(torch.bfloat16).to(dev)
-    q, k = att.q_proj(xl), att.k_proj(xl)
-    assert q.is_contiguous() and k.is_contiguous() and go.rel_l2(k.cpu(), want("k_proj", xl)) <= 1e-3
     # a weight that left the stack (an offloader's rebinding): no stacked launch, same results
     att.k_proj.weight.data = att.k_proj.weight.data.clone()
     assert not stack.intact()
