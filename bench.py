@@ -186,16 +186,17 @@ def main() -> None:
         _, ev_dn = run_region(down_only, n_steps, warmup)
         return wall, ev, ev_gu / n_steps, ev_dn / n_steps
 
-    def mlp_one_launch_leg(m: int, n_steps: int, warmup: int):
+    def mlp_one_launch_leg(m: int, n_steps: int, warmup: int, lay=None, qt_gu=Q8_0, qt_down=Q8_0):
         """The MLP step as modality.gated_mlp runs it by default for one or two rows: sngguf_mlp_decode, ONE launch."""
+        lay = layers if lay is None else lay
         x = synthetic.make_activations(m, HIDDEN, seed=7, device=dev)
         y = torch.empty((m, HIDDEN), dtype=torch.bfloat16, device=dev)
         ws = torch.zeros(ops.mlp_decode_workspace_bytes(m, HIDDEN, INTER), dtype=torch.uint8, device=dev)
-        nl = len(layers)
+        nl = len(lay)
 
         def step(i):
-            gate, up, down = layers[i % nl]
-            ops.mlp_decode_into(x, None, 1e-6, gate, up, Q8_0, down, Q8_0, None, y, ws, num)
+            gate, up, down = lay[i % nl]
+            ops.mlp_decode_into(x, None, 1e-6, gate, up, qt_gu, down, qt_down, None, y, ws, num)
 
         wall, ev = run_region(step, n_steps, warmup)
         torch.cuda.synchronize()
@@ -913,6 +914,13 @@ def main() -> None:
             kq[f"mlp_M{m}"] = {"value": round(gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
                                "bytes_per_step": nbytes, "ms_per_step": round(wall / k2, 6),
                                "gate_up_us": round(gu * 1e3, 3), "down_us": round(dn * 1e3, 3)}
+            if m == 1 and ops.mlp_decode_fits(Q4_K, Q6_K, 1, HIDDEN, INTER):
+                # the route modality.gated_mlp takes for one or two rows; the two launches stay beside it
+                wall1k, _ = mlp_one_launch_leg(1, k2, min(W, 16), klayers, Q4_K, Q6_K)
+                g1 = nbytes / (wall1k / k2 * 1e-3) / 1e9
+                kq["mlp_M1"] = {"what": "sngguf_mlp_decode, one launch", "value": round(g1, 1), "unit": "GB/s",
+                                "pct_of_hbm_peak": round(100 * g1 / HBM_PEAK_GBPS, 2), "bytes_per_step": nbytes,
+                                "ms_per_step": round(wall1k / k2, 6), "two_launches": kq["mlp_M1"]}
         # post_attention_layernorm in front of the Q4_K gate/up pair at M = 1: one torch rms_norm launch + the pair,
         # against the norm folded into the pair's launch
         xk = synthetic.make_activations(1, HIDDEN, seed=21, device=dev)

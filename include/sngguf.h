@@ -176,8 +176,8 @@ int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int
  * rounding of the separate bf16 tensor operations kept.  x, y, residual [M][hidden], gamma [hidden] bf16;
  * q_gate, q_up [inter][hidden], q_down [hidden][inter] packed.
  *
- * Where sngguf_mlp_decode_fits() says so (Q8_0 for all three, hidden 4096, inter 12288, M <= 2, one compute unit per
- * 48-row slice of gate / up) the whole MLP is ONE launch: every workgroup computes its slice of the gated activations,
+ * Where sngguf_mlp_decode_fits() says so (Q8_0 for all three, or Q4_K gate / up with a Q6_K or Q4_K down projection;
+ * hidden 4096, inter 12288, M <= 2, one compute unit per 48-row slice of gate / up) the whole MLP is ONE launch: every workgroup computes its slice of the gated activations,
  * hands them to the others through the workspace (8-byte words that carry the launch's generation tag beside the data)
  * and goes on with 16 rows of the down projection as the slices it needs arrive; the down weights are requested while
  * the slower workgroups still finish.  All workgroups of that launch must be resident
@@ -186,7 +186,9 @@ int sngguf_linear_static(const void* x, int64_t M, const void* q, int qtype, int
  * sets the 32-bit word at byte sngguf_mlp_decode_status_offset() of the workspace to 1, finishes with whatever the
  * activations hold and the launch ends normally - the caller reads that word when it synchronises, and the results
  * of a call that set it are void.  Everything else runs as the separate launches of sngguf_[rmsnorm_]gate_up_silu
- * and sngguf_linear[_residual] with the activations in the workspace: same values.
+ * and sngguf_linear[_residual] with the activations in the workspace: same values.  (The one launch against the
+ * separate ones: equal up to the order in which fp32 partial sums are added - the down projection's K split and, for
+ * the K-quant mixes with gamma, the sum of squares.)
  *
  * workspace: sngguf_mlp_decode_workspace_bytes(M, hidden, inter) bytes, 256-byte aligned, all zero before the first
  * call and the launches' own from then on (generation counter and tagged words; never cleared again, also not

@@ -46,6 +46,10 @@ bool mlp_q8_decode_fits(int64_t M, int64_t hidden, int64_t inter);
 int launch_mlp_q8_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down,
                          int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics, int spin_limit,
                          hipStream_t stream);
+bool mlp_kq_decode_fits(int qtype_gate_up, int qtype_down, int64_t M, int64_t hidden, int64_t inter);
+int launch_mlp_kq_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down,
+                         int qtype_down, int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics,
+                         int spin_limit, hipStream_t stream);
 int64_t stream_probe_out_bytes();
 int launch_stream_read(const void* p, int64_t bytes, void* out, int workgroups, bool nontemporal, hipStream_t stream);
 int64_t grouped_workspace_bytes(int64_t M);
@@ -512,7 +516,8 @@ int64_t sngguf_mlp_decode_workspace_bytes(int64_t M, int64_t hidden, int64_t int
 int64_t sngguf_mlp_decode_status_offset(void) { return sngguf::mlp_q8_decode_status_offset(); }
 
 int sngguf_mlp_decode_fits(int qtype_gate_up, int qtype_down, int64_t M, int64_t hidden, int64_t inter) {
-    return qtype_gate_up == SNGGUF_TYPE_Q8_0 && qtype_down == SNGGUF_TYPE_Q8_0 && sngguf::mlp_q8_decode_fits(M, hidden, inter);
+    if (qtype_gate_up == SNGGUF_TYPE_Q8_0 && qtype_down == SNGGUF_TYPE_Q8_0) return sngguf::mlp_q8_decode_fits(M, hidden, inter);
+    return sngguf::mlp_kq_decode_fits(qtype_gate_up, qtype_down, M, hidden, inter);
 }
 
 int sngguf_mlp_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, int qtype_gate_up,
@@ -528,9 +533,13 @@ int sngguf_mlp_decode(const void* x, int64_t M, const void* gamma, float eps, co
         return SNGGUF_E_ALIGN;
     if (gamma && !(eps >= 0.f)) return SNGGUF_E_BADSHAPE;
     if (workspace_bytes < sngguf_mlp_decode_workspace_bytes(M, hidden, inter)) return SNGGUF_E_BADSHAPE;
-    if (sngguf_mlp_decode_fits(qtype_gate_up, qtype_down, M, hidden, inter))
-        return sngguf::launch_mlp_q8_decode(x, M, gamma, eps, q_gate, q_up, q_down, hidden, inter, residual, y, workspace, numerics,
-                                            spin_limit, static_cast<hipStream_t>(stream));
+    if (sngguf_mlp_decode_fits(qtype_gate_up, qtype_down, M, hidden, inter)) {
+        if (qtype_gate_up == SNGGUF_TYPE_Q8_0)
+            return sngguf::launch_mlp_q8_decode(x, M, gamma, eps, q_gate, q_up, q_down, hidden, inter, residual, y, workspace, numerics,
+                                                spin_limit, static_cast<hipStream_t>(stream));
+        return sngguf::launch_mlp_kq_decode(x, M, gamma, eps, q_gate, q_up, q_down, qtype_down, hidden, inter, residual, y, workspace,
+                                            numerics, spin_limit, static_cast<hipStream_t>(stream));
+    }
     // every other shape and type: the same arithmetic as separate launches, the gated activations (and, where the norm
     // does not ride inside the pair's launch, the normalized rows) in the workspace
     char* h = static_cast<char*>(workspace) + sngguf::mlp_q8_decode_ctl_bytes();

@@ -730,7 +730,372 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
     return launch_r<QT, NUM, 1>(x, M, qa, qb, N, K, bias, residual, y, gated, gamma, eps, stream, amax);
 }
 
+// ---- the SiLU-gated MLP of a decoder layer at decode sizes in ONE launch, K-quant weights ---------------------
+// The organisation of mlp_q8_decode_kernel (gemv_q8_mfma.hip) with this file's decoders: 256 workgroups of twelve
+// wavefronts, one per compute unit.  Phase A: workgroup b computes the gated activations of rows [48 b, +48) - three
+// 16-row groups, each with four wavefronts as in the gated pair's own launch (gate / up x two K halves of eight
+// super-blocks), the activations staged once per workgroup in LDS (normalized there if `gamma` is given) - and writes
+// them as 8-byte words { two bf16, generation tag } with agent-scope stores, then the group's flag.  No barrier inside
+// the phase: a wavefront leaves its partial sums in LDS and counts itself in for its row group; the group's storing
+// wavefront waits for that count only.  Phase B: 16 rows of the down matrix, K = inter split over the twelve
+// wavefronts, four super-blocks each; two of them are requested the moment the wavefront leaves phase A's loop, the
+// other two after one workgroup barrier (requested earlier, their traffic slows phase A's last wavefronts, which the
+// whole device waits for), and all four wait as raw bytes in registers; the first is decoded into matrix-core operands
+// while the activations are on their way.  Then the wavefront polls the flags of the 64 row groups its K range needs,
+// reads the tagged words (every tag checked), contracts the decoded super-block, decodes and contracts the other three,
+// and the twelve partial sums are added.  Bounded wait, status word, generation counter and workspace layout as in the
+// Q8_0 kernel (MlpCtl).  Without `gamma` the gated activations are bit-identical to the gated pair's own launch (same
+// fragments, same order of accumulation), and so is the output (the down projection's own launch splits K over eight
+// wavefronts, not twelve: equal up to the order of twelve fp32 additions, which the tests allow for).
+// The decode arithmetic, not memory, bounds these formats: the launch is worth 1 - 3 % over the two separate ones
+// (34.1 against 34.3 us with a Q6_K down projection, 31.9 against 33.0 with Q4_K), where the Q8_0 kernel gains 11 %.
+template <int QT>
+struct SlabIo {
+    typedef Slab<QT> S;
+    static constexpr int kPieces = 16 * S::pieces;
+    static constexpr int kLoads = (kPieces + 63) / 64;
+    static constexpr int kSlab = 16 * S::stride;
+    static constexpr bool kQ6 = QT == SNGGUF_TYPE_Q6_K;
+    uint32_t off[kLoads], dst[kLoads];
+    uint32_t doff;
+    bool tail_lane;
+    __device__ __forceinline__ void init(int lane, int64_t row_bytes) {
+#pragma unroll
+        for (int i = 0; i < kLoads; i++) {
+            const int f = lane + 64 * i;
+            const bool ok = f < kPieces;
+            const int fr = ok ? f / S::pieces : 0, fp = ok ? f % S::pieces : 0;
+            off[i] = (uint32_t)(fr * row_bytes + (fp == S::pieces - 1 ? S::last_src : 16 * fp));
+            dst[i] = (uint32_t)(fr * S::stride + 16 * fp);
+        }
+        tail_lane = lane + 64 * (kLoads - 1) < kPieces;
+        doff = (uint32_t)((lane < 16 ? lane : 0) * row_bytes + 208);
+    }
+    __device__ __forceinline__ void fetch(const uint8_t* __restrict__ base, int s, int lane, u32x4_t (&pre)[kLoads], uint16_t& pre_d) const {
+        const uint8_t* p = base + (int64_t)s * S::ts;
+#pragma unroll
+        for (int i = 0; i < kLoads - 1; i++) pre[i] = ld_piece<S::align>(p + off[i]);
+        if (tail_lane) pre[kLoads - 1] = ld_piece<S::align>(p + off[kLoads - 1]);
+        if constexpr (kQ6) {
+            if (lane < 16) pre_d = ld_u16(p + doff);
+        }
+    }
+    __device__ __forceinline__ void store(uint8_t* slab, int lane, const u32x4_t (&pre)[kLoads], uint16_t pre_d) const {
+#pragma unroll
+        for (int i = 0; i < kLoads - 1; i++) *reinterpret_cast<u32x4_t*>(slab + dst[i]) = pre[i];
+        if (tail_lane) *reinterpret_cast<u32x4_t*>(slab + dst[kLoads - 1]) = pre[kLoads - 1];
+        if constexpr (kQ6) {
+            if (lane < 16) *reinterpret_cast<uint16_t*>(slab + lane * S::stride + 208) = pre_d;
+        }
+    }
+};
+
+constexpr int kMlpKqWaves = 12;
+// Super-blocks of the down matrix that a wavefront decodes into registers while it waits for the activations: one (32
+// registers of operands beside a decoder's ~100 of temporaries is what 168 registers per lane hold; two spill).
+#ifndef SNGGUF_MLPKQ_AHEAD
+#define SNGGUF_MLPKQ_AHEAD 1
+#endif
+constexpr int kMlpKqSteps = 4;   // super-blocks of the down matrix per wavefront: inter = 12 x 4 x 256 (the launcher checks)
+
+template <int QA, int QB>
+struct MlpKqLds {
+    // [12 slabs of phase A][x staged (M rows) + sums of squares][partial sums of phase A + counters][12 x (slab of phase B, two staged activation rows)]
+    static constexpr int kSlabsA = kMlpKqWaves * SlabIo<QA>::kSlab;
+    static constexpr int kWaveB = SlabIo<QB>::kSlab + 2 * kMlpKqSteps * 512;
+    __host__ __device__ static size_t xs_bytes(int M, int64_t hidden, bool norm) {
+        return (((size_t)M * (2 * (size_t)hidden + 64) + (norm ? (size_t)4 * M * kMlpKqWaves : 0)) + 255) & ~(size_t)255;
+    }
+    __host__ __device__ static size_t total(int M, int64_t hidden, bool norm) {
+        return (size_t)kSlabsA + xs_bytes(M, hidden, norm) + (size_t)kMlpKqWaves * 64 * 16 + 64 + (size_t)kMlpKqWaves * kWaveB;
+    }
+};
+
+template <int QA, int QB, int NUM>
+__global__ __launch_bounds__(64 * kMlpKqWaves) void mlp_kq_decode_kernel(const bf16_t* __restrict__ x, int M, const uint8_t* __restrict__ q_gate,
+                                                                         const uint8_t* __restrict__ q_up, const uint8_t* __restrict__ q_down,
+                                                                         int64_t hidden, int64_t inter, const bf16_t* __restrict__ gamma, float eps,
+                                                                         const bf16_t* residual, bf16_t* __restrict__ y, MlpCtl* ctl, uint64_t* ht,
+                                                                         int spin_limit) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    typedef SlabIo<QA> IA;
+    typedef SlabIo<QB> IB;
+    typedef MlpKqLds<QA, QB> L;
+    constexpr int kWaves = kMlpKqWaves, kSteps = kMlpKqSteps;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bid = (int)blockIdx.x, nb = (int)gridDim.x;
+    const int r = lane & 15, g = lane >> 4;
+    const half4_t ident = identity_row(lane);
+    // this launch's tag: nobody advances the generation before every workgroup, this one included, has finished
+    const uint32_t tag = __hip_atomic_load(&ctl->gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+
+    uint8_t* const xs = lds + L::kSlabsA;
+    const int64_t xs_stride = 2 * hidden + 64;
+    f32x4_t* const red_a = reinterpret_cast<f32x4_t*>(xs + L::xs_bytes(M, hidden, gamma != nullptr));
+    uint32_t* const cnt = reinterpret_cast<uint32_t*>(red_a + kWaves * 64);
+    uint8_t* const slab_b = reinterpret_cast<uint8_t*>(cnt + 16) + wave * L::kWaveB;
+    uint8_t* const xw = slab_b + IB::kSlab;   // [2][kSteps * 512] bytes
+
+    // ---- phase A: row group 3 bid + grp, matrix mat (0 gate, 1 up), K half kh ----
+    __builtin_amdgcn_s_setprio(2);
+    const int grp = wave >> 2, lw = wave & 3, mat = lw >> 1, kh = lw & 1;
+    const int nsb = (int)(hidden >> 8);
+    const int sa0 = kh * (nsb >> 1), sa1 = sa0 + (nsb >> 1);
+    const int64_t arow_bytes = (int64_t)nsb * IA::S::ts;
+    const uint8_t* __restrict__ abase = (mat ? q_up : q_gate) + (int64_t)(3 * bid + grp) * 16 * arow_bytes;
+    IA ia;
+    ia.init(lane, arow_bytes);
+    uint8_t* const slab_a = lds + wave * IA::kSlab;
+    u32x4_t pre_a[IA::kLoads];
+    uint16_t pre_ad = 0;
+    ia.fetch(abase, sa0, lane, pre_a, pre_ad);
+    if (tid < 16) cnt[tid] = 0;
+    // the activations, staged once for the workgroup (normalized in place if gamma is given)
+    {
+        const int pieces_per_row = (int)(hidden >> 3);
+        if (gamma == nullptr) {
+            for (int f = tid; f < M * pieces_per_row; f += 64 * kWaves) {
+                const int m = f / pieces_per_row, c = f - m * pieces_per_row;
+                *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * hidden + 8 * c);
+            }
+        } else {
+            float* ssum = reinterpret_cast<float*>(xs + M * xs_stride);   // [M][waves]
+            for (int m = 0; m < M; m++) {
+                float ss = 0.f;
+                for (int c = tid; c < pieces_per_row; c += 64 * kWaves) {
+                    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)m * hidden + 8 * c);
+                    *reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c) = v;
+                    ss += sumsq_piece(v);
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) ssum[m * kWaves + wave] = ss;
+            }
+            __syncthreads();
+            for (int m = 0; m < M; m++) {
+                float tot = 0.f;
+                for (int w = 0; w < kWaves; w++) tot += ssum[m * kWaves + w];
+                const float rstd = rms_rstd(tot, hidden, eps);
+                for (int c = tid; c < pieces_per_row; c += 64 * kWaves) {
+                    u32x4_t* cell = reinterpret_cast<u32x4_t*>(xs + m * xs_stride + 16 * c);
+                    *cell = rmsnorm_piece(*cell, *reinterpret_cast<const u32x4_t*>(gamma + 8 * c), rstd);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const bool has_x = r < M;
+    const uint8_t* xsrow = xs + (has_x ? r : M - 1) * xs_stride + 16 * g;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = sa0; s < sa1; s++) {
+        ia.store(slab_a, lane, pre_a, pre_ad);
+        if (s + 1 < sa1) ia.fetch(abase, s + 1, lane, pre_a, pre_ad);
+        const uint8_t* row = slab_a + r * IA::S::stride;
+        auto emit0 = [&](int jj, const u32x4_t& a) {
+            const u32x4_t xf = *reinterpret_cast<const u32x4_t*>(xsrow + (s * 8 + jj) * 64);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xf), acc, 0, 0, 0);
+        };
+        decode_half<QA, NUM, 0>(ident, row, g, emit0);
+        auto emit1 = [&](int jj, const u32x4_t& a) {
+            const u32x4_t xf = *reinterpret_cast<const u32x4_t*>(xsrow + (s * 8 + 4 + jj) * 64);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xf), acc, 0, 0, 0);
+        };
+        decode_half<QA, NUM, 1>(ident, row, g, emit1);
+    }
+
+    // ---- phase B geometry: rows [16 bid, +16) of down, super-blocks [4 wave, +4) ----
+    const int sb0 = wave * kSteps;
+    const int64_t brow_bytes = (inter >> 8) * IB::S::ts;
+    const uint8_t* __restrict__ bbase = q_down + (int64_t)bid * 16 * brow_bytes;
+    IB ib;
+    ib.init(lane, brow_bytes);
+    u32x4_t raw[kSteps][IB::kLoads];
+    uint16_t raw_d[kSteps] = {};
+    ib.fetch(bbase, sb0, lane, raw[0], raw_d[0]);
+    ib.fetch(bbase, sb0 + 1, lane, raw[1], raw_d[1]);
+
+    // ---- phase A epilogue: partial sums, per-group count, the storing wavefront's SiLU and tagged stores ----
+    red_a[wave * 64 + lane] = acc;
+    if (lane == 0) __hip_atomic_fetch_add(cnt + grp, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (lw == 0) {
+        while (__hip_atomic_load(cnt + grp, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < 4u) __builtin_amdgcn_s_sleep(1);
+        if (has_x) {
+            // wavefronts 4 grp + {0, 1}: gate K halves, + {2, 3}: up K halves; D[i][j]: j = lane % 16 the activation row
+            f32x4_t gs = red_a[(4 * grp) * 64 + lane], us = red_a[(4 * grp + 2) * 64 + lane];
+            const f32x4_t g1 = red_a[(4 * grp + 1) * 64 + lane], u1 = red_a[(4 * grp + 3) * 64 + lane];
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float gt = bf16_to_f32(f32_to_bf16(gs[v] + g1[v]));
+                const float ut = bf16_to_f32(f32_to_bf16(us[v] + u1[v]));
+                const float sl = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+                o[v] = sl * ut;
+            }
+            const int64_t n = (int64_t)(3 * bid + grp) * 16 + 4 * g;
+            uint64_t* yt = ht + (((int64_t)r * inter + n) >> 1);
+            __hip_atomic_store(yt, (uint64_t)pack_bf16(o[0], o[1]) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(yt + 1, (uint64_t)pack_bf16(o[2], o[3]) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) __hip_atomic_store(&ctl->flags[3 * bid + grp], tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_setprio(0);
+
+    // ---- phase B: decode the first kAhead super-blocks into matrix-core operands while the activations are on their
+    // way (what the register file holds beside a decoder's temporaries); the others wait as raw bytes in registers ----
+    constexpr int kAhead = SNGGUF_MLPKQ_AHEAD;
+    u32x4_t afrag[kAhead > 0 ? kAhead * 8 : 1];
+    const uint8_t* const brow = slab_b + r * IB::S::stride;
+    auto decode = [&](int i) {
+        ib.store(slab_b, lane, raw[i], raw_d[i]);
+        auto e0 = [&](int jj, const u32x4_t& a) { afrag[i * 8 + jj] = a; };
+        decode_half<QB, NUM, 0>(ident, brow, g, e0);
+        auto e1 = [&](int jj, const u32x4_t& a) { afrag[i * 8 + 4 + jj] = a; };
+        decode_half<QB, NUM, 1>(ident, brow, g, e1);
+    };
+    if constexpr (kAhead > 0) decode(0);
+    if constexpr (kAhead > 1) decode(1);
+    __syncthreads();   // the whole workgroup has left phase A: now the other two steps' traffic
+    ib.fetch(bbase, sb0 + 2, lane, raw[2], raw_d[2]);
+    ib.fetch(bbase, sb0 + 3, lane, raw[3], raw_d[3]);
+    if constexpr (kAhead > 2) decode(2);
+    if constexpr (kAhead > 3) decode(3);
+
+    // ---- wait for this wavefront's K range of the activations: flags of its 64 row groups, then the tagged words ----
+    constexpr int xrow_b = kSteps * 512;
+    {
+        const int pairs = kSteps * 64;                    // 16-byte pairs of words per row in this wavefront's K range
+        const int64_t w0 = (int64_t)sb0 * 128;            // first word of the range within a row
+        const int64_t row_words = inter >> 1;
+        const int g0 = sb0 * 16, ng = kSteps * 16;        // row groups of 16 outputs
+        int polls = 0;
+        bool gave_up = false;
+        for (;;) {
+            bool all = true;
+            for (int j = lane; j < ng; j += 64) all = all && __hip_atomic_load(&ctl->flags[g0 + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+            if (__builtin_amdgcn_ballot_w64(!all) == 0) break;
+            if (++polls > spin_limit) { gave_up = true; break; }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        for (;;) {
+            bool all = true;
+            for (int m = 0; m < M; m++)
+                for (int c = lane; c < pairs; c += 64) {
+                    const uint64_t* src = ht + (int64_t)m * row_words + w0 + 2 * c;
+                    const uint64_t a = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint64_t b = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    all = all && (uint32_t)(a >> 32) == tag && (uint32_t)(b >> 32) == tag;
+                    *reinterpret_cast<uint64_t*>(xw + m * xrow_b + 8 * c) = (uint64_t)(uint32_t)a | (b << 32);
+                }
+            if (gave_up || __builtin_amdgcn_ballot_w64(!all) == 0) break;
+            if (++polls > spin_limit) { gave_up = true; break; }
+        }
+        if (gave_up && lane == 0) __hip_atomic_store(&ctl->status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- contract, add the twelve partial sums, residual, store ----
+    __builtin_amdgcn_s_setprio(3);
+    f32x4_t yacc = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t* xwrow = xw + (has_x ? r : M - 1) * xrow_b + 16 * g;
+#pragma unroll
+    for (int i = 0; i < kAhead * 8; i++) {
+        const u32x4_t xf = *reinterpret_cast<const u32x4_t*>(xwrow + i * 64);
+        yacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afrag[i]), __builtin_bit_cast(bf16x8_t, xf), yacc, 0, 0, 0);
+    }
+    auto decode_contract = [&](int i) {
+        ib.store(slab_b, lane, raw[i], raw_d[i]);
+        auto e0 = [&](int jj, const u32x4_t& a) {
+            const u32x4_t xf = *reinterpret_cast<const u32x4_t*>(xwrow + (i * 8 + jj) * 64);
+            yacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xf), yacc, 0, 0, 0);
+        };
+        decode_half<QB, NUM, 0>(ident, brow, g, e0);
+        auto e1 = [&](int jj, const u32x4_t& a) {
+            const u32x4_t xf = *reinterpret_cast<const u32x4_t*>(xwrow + (i * 8 + 4 + jj) * 64);
+            yacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, xf), yacc, 0, 0, 0);
+        };
+        decode_half<QB, NUM, 1>(ident, brow, g, e1);
+    };
+    if constexpr (kAhead <= 0) decode_contract(0);
+    if constexpr (kAhead <= 1) decode_contract(1);
+    if constexpr (kAhead <= 2) decode_contract(2);
+    if constexpr (kAhead <= 3) decode_contract(3);
+    __syncthreads();   // every wavefront is past phase A's epilogue: its partial-sum area is free
+    red_a[wave * 64 + lane] = yacc;
+    __syncthreads();
+    if (wave == 0 && has_x) {
+        f32x4_t sum = red_a[lane];
+        for (int w = 1; w < kWaves; w++) {
+            const f32x4_t t = red_a[w * 64 + lane];
+            sum[0] += t[0]; sum[1] += t[1]; sum[2] += t[2]; sum[3] += t[3];
+        }
+        const int64_t n = (int64_t)bid * 16 + 4 * g;
+        float o[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = add_residual(sum[v], residual, (int64_t)r * hidden + n + v);
+        *reinterpret_cast<u32x2_t*>(y + (int64_t)r * hidden + n) = u32x2_t{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+    }
+    if (tid == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&ctl->done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == (uint32_t)nb - 1u) {
+            __hip_atomic_store(&ctl->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&ctl->gen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+template <int QA, int QB, int NUM>
+int launch_mlp_kq(const void* x, int M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down, int64_t hidden,
+                  int64_t inter, const void* residual, void* y, void* workspace, int spin_limit, hipStream_t stream) {
+    const size_t lds_bytes = MlpKqLds<QA, QB>::total(M, hidden, gamma != nullptr);
+    if (lds_bytes > 160 * 1024) return SNGGUF_E_BADSHAPE;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&mlp_kq_decode_kernel<QA, QB, NUM>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess) return SNGGUF_E_LAUNCH;
+    MlpCtl* ctl = static_cast<MlpCtl*>(workspace);
+    uint64_t* h = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(workspace) + kMlpCtlBytes);
+    const int limit = spin_limit == 0 ? 1 << 20 : spin_limit < 0 ? 0 : spin_limit;
+    mlp_kq_decode_kernel<QA, QB, NUM><<<dim3((unsigned)(inter / 48)), dim3(64 * kMlpKqWaves), lds_bytes, stream>>>(
+        static_cast<const bf16_t*>(x), M, static_cast<const uint8_t*>(q_gate), static_cast<const uint8_t*>(q_up),
+        static_cast<const uint8_t*>(q_down), hidden, inter, static_cast<const bf16_t*>(gamma), eps, static_cast<const bf16_t*>(residual),
+        static_cast<bf16_t*>(y), ctl, h, limit);
+    return hipGetLastError() == hipSuccess ? SNGGUF_OK : SNGGUF_E_LAUNCH;
+}
+
 }  // namespace
+
+// The K-quant mixes the one-launch MLP takes: Q4_K gate / up with a Q6_K or Q4_K down projection (the "Q4_K_M" recipe),
+// hidden 4096, inter 12288 (48 rows of gate / up and 16 rows of down per workgroup, 12 x 4 super-blocks per down row),
+// one or two rows, one resident workgroup per compute unit.
+bool mlp_kq_decode_fits(int qtype_gate_up, int qtype_down, int64_t M, int64_t hidden, int64_t inter) {
+    if (qtype_gate_up != SNGGUF_TYPE_Q4_K || (qtype_down != SNGGUF_TYPE_Q6_K && qtype_down != SNGGUF_TYPE_Q4_K)) return false;
+    if (M < 1 || M > 2 || hidden != 4096 || inter != 12 * kMlpKqSteps * 256) return false;
+    static const int cus = [] {
+        int dev = 0, n = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        const void* k = reinterpret_cast<const void*>(&mlp_kq_decode_kernel<SNGGUF_TYPE_Q4_K, SNGGUF_TYPE_Q6_K, 1>);
+        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) return 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mlp_kq_decode_kernel<SNGGUF_TYPE_Q4_K, SNGGUF_TYPE_Q6_K, 1>, 64 * kMlpKqWaves,
+                                                         160 * 1024) != hipSuccess)
+            return 0;
+        return per_cu >= 1 ? n : 0;
+    }();
+    return cus >= inter / 48;
+}
+
+int launch_mlp_kq_decode(const void* x, int64_t M, const void* gamma, float eps, const void* q_gate, const void* q_up, const void* q_down,
+                         int qtype_down, int64_t hidden, int64_t inter, const void* residual, void* y, void* workspace, int numerics,
+                         int spin_limit, hipStream_t stream) {
+    if (!mlp_kq_decode_fits(SNGGUF_TYPE_Q4_K, qtype_down, M, hidden, inter)) return SNGGUF_E_BADSHAPE;
+#define SNGGUF_GO(QB, NUMV) \
+    return launch_mlp_kq<SNGGUF_TYPE_Q4_K, QB, NUMV>(x, (int)M, gamma, eps, q_gate, q_up, q_down, hidden, inter, residual, y, workspace, spin_limit, stream)
+    if (qtype_down == SNGGUF_TYPE_Q6_K) {
+        if (numerics == SNGGUF_NUM_GGML_FP32) SNGGUF_GO(SNGGUF_TYPE_Q6_K, 0);
+        SNGGUF_GO(SNGGUF_TYPE_Q6_K, 1);
+    }
+    if (numerics == SNGGUF_NUM_GGML_FP32) SNGGUF_GO(SNGGUF_TYPE_Q4_K, 0);
+    SNGGUF_GO(SNGGUF_TYPE_Q4_K, 1);
+#undef SNGGUF_GO
+}
 
 // Workgroups of a plain decode launch = (value, column) slots per activation row that its arg-max form writes.
 int64_t gemv_argmax_slots(int qtype, int64_t M, int64_t N) {

@@ -675,12 +675,6 @@ __global__ __launch_bounds__(64 * WMAX) void gemv_q8_span_kernel(const bf16_t* _
 // that long - the wavefront sets `status`, goes on with whatever the words hold and the kernel still ends normally.
 // Inside a workgroup the first phase uses no barrier either: a wavefront leaves its partial sums in LDS and counts
 // itself in for its row group, and only that group's storing wavefront waits for the count.
-struct MlpCtl {
-    uint32_t gen, done, status, pad[61];
-    uint32_t flags[1024];   // per 16-row group of gate / up
-};
-constexpr int64_t kMlpCtlBytes = 8192;   // the tagged activation words [M][inter / 2] follow at this offset
-
 #ifdef SNGGUF_MLP_TRACE
 __device__ uint64_t g_mlp_trace[256 * 12 * 8];
 #define MLP_TRACE(slot) do { if (lane == 0) g_mlp_trace[((int)blockIdx.x * 12 + wave) * 8 + (slot)] = wall_clock64(); } while (0)

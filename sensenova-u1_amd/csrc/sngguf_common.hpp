@@ -448,4 +448,15 @@ __device__ __forceinline__ u32x4_t rmsnorm_piece(u32x4_t xv, u32x4_t gv, float r
     return o;
 }
 
+
+// ---- hand-over state of the one-launch decode MLP kernels ----------------------------------------------------
+// At the start of the caller's workspace, zero before its first use: the generation counter that tags the activation
+// words of a launch (advanced by the last workgroup to finish, through the trailing `done` counter), a sticky status word
+// (1: some wavefront gave up waiting), and one flag per 16-row group of gate / up.
+struct MlpCtl {
+    uint32_t gen, done, status, pad[61];
+    uint32_t flags[1024];
+};
+constexpr int64_t kMlpCtlBytes = 8192;   // the tagged activation words [M][inter / 2] follow at this offset
+
 }  // namespace sngguf

@@ -1,7 +1,9 @@
-"""GPU: the decode MLP as one entry point (``sngguf_mlp_decode``): one launch at the 8B model's shape in Q8_0 for up to
-two rows, the separate launches everywhere else.  Against the separate launches of the library (the gated activations
-are the same kernel's, so only the down projection's order of summation differs) and against the CPU oracle on sampled
-output columns; consecutive calls, graph replays (the hand-over state advances by itself), the bounded wait."""
+"""GPU: the decode MLP as one entry point (``sngguf_mlp_decode``): one launch at the 8B model's shape for up to two rows
+in Q8_0 and in the K-quant mixes (Q4_K gate / up with a Q6_K or Q4_K down projection), the separate launches everywhere
+else.  Against the separate launches of the library (the gated activations come out of the same arithmetic in the same
+order, so only the down projection's order of summation differs - and, for the K-quants with the norm folded in, the
+order in which the sum of squares is added) and against the CPU oracle on sampled output columns; consecutive calls,
+graph replays (the hand-over state advances by itself), the bounded wait."""
 import pytest
 import torch
 
@@ -42,12 +44,16 @@ def _separate(x, gamma, gate, up, down, qt_gu, qt_d, residual, num):
     return y, h
 
 
+ONE_LAUNCH_TYPES = [(go.Q8_0, go.Q8_0), (go.Q4_K, go.Q6_K), (go.Q4_K, go.Q4_K)]
+
+
 @pytest.mark.parametrize("m", [1, 2])
 @pytest.mark.parametrize("num", [ops.NUM_GGML_FP32, ops.NUM_UPSTREAM_FP16])
-def test_one_launch_mlp_matches_the_separate_launches_and_the_oracle(dev, c_oracle, m, num):
-    print(f"case mlp_decode m={m} num={num}", flush=True)
-    assert ops.mlp_decode_fits(go.Q8_0, go.Q8_0, m, H, I)
-    gate, up, down = _weights(dev, seed=10 * m)
+@pytest.mark.parametrize("qt_gu,qt_d", ONE_LAUNCH_TYPES)
+def test_one_launch_mlp_matches_the_separate_launches_and_the_oracle(dev, c_oracle, m, num, qt_gu, qt_d):
+    print(f"case mlp_decode {qt_gu}/{qt_d} m={m} num={num}", flush=True)
+    assert ops.mlp_decode_fits(qt_gu, qt_d, m, H, I)
+    gate, up, down = _weights(dev, qt_gu, qt_d, seed=10 * m)
     ws = torch.zeros(ops.mlp_decode_workspace_bytes(m, H, I), dtype=torch.uint8, device=dev)
     gen = torch.Generator().manual_seed(m)
     gamma = (torch.rand(H, generator=gen) * 1.5 + 0.25).to(torch.bfloat16).to(dev)
@@ -57,13 +63,19 @@ def test_one_launch_mlp_matches_the_separate_launches_and_the_oracle(dev, c_orac
             res = synthetic.make_activations(m, H, seed=200 + m, device=dev) if use_res else None
             g = gamma if use_gamma else None
             y = torch.full((m, H), float("nan"), dtype=torch.bfloat16, device=dev)
-            ops.mlp_decode_into(x, g, EPS, gate, up, go.Q8_0, down, go.Q8_0, res, y, ws, num)
-            want, h_sep = _separate(x, g, gate, up, down, go.Q8_0, go.Q8_0, res, num)
+            ops.mlp_decode_into(x, g, EPS, gate, up, qt_gu, down, qt_d, res, y, ws, num)
+            want, h_sep = _separate(x, g, gate, up, down, qt_gu, qt_d, res, num)
             assert bool(torch.isfinite(y.float()).all())
-            # the gated activations the launch left in the workspace are the pair kernel's own
+            # the gated activations the launch left in the workspace are the pair kernel's own (K-quants with the norm
+            # folded in: the workgroup adds the sum of squares over twelve wavefronts where the pair's launch adds it
+            # over two, so 1 / rms may differ in its last bits and a normalized value that sat on a bf16 tie with it)
             h_ws = _activations_left_in(ws, m)
-            assert torch.equal(h_ws, h_sep), (use_gamma, use_res)
-            assert go.rel_l2(y.cpu(), want.cpu()) <= 1e-4, (use_gamma, use_res)
+            if qt_gu == go.Q8_0 or not use_gamma:
+                assert torch.equal(h_ws, h_sep), (use_gamma, use_res)
+                assert go.rel_l2(y.cpu(), want.cpu()) <= 1e-4, (use_gamma, use_res)
+            else:
+                assert go.rel_l2(h_ws.cpu(), h_sep.cpu()) <= 3e-4, (use_gamma, use_res)
+                assert go.rel_l2(y.cpu(), want.cpu()) <= 5e-4, (use_gamma, use_res)
             assert not ops.mlp_decode_gave_up(ws)
             # the oracle, stage by stage (the tolerance is stated per linear): the gated activations on sampled columns
             # against oracle norm + gate / up / SiLU, and sampled outputs against the oracle's down projection of the
@@ -71,27 +83,28 @@ def test_one_launch_mlp_matches_the_separate_launches_and_the_oracle(dev, c_orac
             cols = torch.randint(0, H, (40,), generator=gen)
             icols = torch.randint(0, I, (64,), generator=gen)
             xn = go.qwen3_rms_norm(x.cpu(), gamma.cpu(), EPS) if use_gamma else x.cpu()
-            hg = c_oracle.silu_mul(go.gguf_linear_forward(xn, gate[icols.to(dev)].cpu(), go.Q8_0, None, numerics=num),
-                                   go.gguf_linear_forward(xn, up[icols.to(dev)].cpu(), go.Q8_0, None, numerics=num))
+            hg = c_oracle.silu_mul(go.gguf_linear_forward(xn, gate[icols.to(dev)].cpu(), qt_gu, None, numerics=num),
+                                   go.gguf_linear_forward(xn, up[icols.to(dev)].cpu(), qt_gu, None, numerics=num))
             assert go.rel_l2(h_ws[:, icols.to(dev)].cpu(), hg) <= TOL, (use_gamma, use_res)
-            yo = go.gguf_linear_forward(h_ws.cpu(), down[cols.to(dev)].cpu(), go.Q8_0, None, numerics=num)
+            yo = go.gguf_linear_forward(h_ws.cpu(), down[cols.to(dev)].cpu(), qt_d, None, numerics=num)
             if use_res:
                 yo = (res.cpu()[:, cols].float() + yo.float()).to(torch.bfloat16)
             assert go.rel_l2(y[:, cols.to(dev)].cpu(), yo) <= TOL, (use_gamma, use_res)
 
 
-def test_consecutive_calls_and_graph_replays_advance_the_hand_over_state(dev):
-    print("case mlp_decode replays", flush=True)
+@pytest.mark.parametrize("qt_gu,qt_d", ONE_LAUNCH_TYPES[:2])
+def test_consecutive_calls_and_graph_replays_advance_the_hand_over_state(dev, qt_gu, qt_d):
+    print(f"case mlp_decode replays {qt_gu}/{qt_d}", flush=True)
     m = 1
-    sets = [_weights(dev, seed=50 + 10 * i) for i in range(3)]
+    sets = [_weights(dev, qt_gu, qt_d, seed=50 + 10 * i) for i in range(3)]
     ws = torch.zeros(ops.mlp_decode_workspace_bytes(m, H, I), dtype=torch.uint8, device=dev)
     x = synthetic.make_activations(m, H, seed=7, device=dev)
     ys = [torch.empty((m, H), dtype=torch.bfloat16, device=dev) for _ in sets]
-    wants = [_separate(x, None, *w, go.Q8_0, go.Q8_0, None, 1)[0] for w in sets]
+    wants = [_separate(x, None, *w, qt_gu, qt_d, None, 1)[0] for w in sets]
 
     def run():
         for w, y in zip(sets, ys):
-            ops.mlp_decode_into(x, None, EPS, *w[:2], go.Q8_0, w[2], go.Q8_0, None, y, ws, 1)
+            ops.mlp_decode_into(x, None, EPS, *w[:2], qt_gu, w[2], qt_d, None, y, ws, 1)
 
     for _ in range(3):
         run()
@@ -111,33 +124,35 @@ def test_consecutive_calls_and_graph_replays_advance_the_hand_over_state(dev):
         torch.cuda.synchronize()
         for y, f in zip(ys, first):
             assert torch.equal(y, f), rep
-        ops.linear(x, sets[0][0], go.Q8_0)          # eager work between the replays
+        ops.linear(x, sets[0][0], qt_gu)            # eager work between the replays
         torch.cuda.synchronize()
     assert gen_word() == 9 + 3 * 4 and not ops.mlp_decode_gave_up(ws)
 
 
-def test_a_bounded_wait_that_gives_up_still_ends_the_launch(dev):
+@pytest.mark.parametrize("qt_gu,qt_d", ONE_LAUNCH_TYPES[:2])
+def test_a_bounded_wait_that_gives_up_still_ends_the_launch(dev, qt_gu, qt_d):
     """spin_limit < 0: a workgroup that does not find every flag set at its first poll gives up at once, says so in the
     status word and finishes; the state still advances and a following ordinary call on the workspace is right."""
-    print("case mlp_decode give-up", flush=True)
+    print(f"case mlp_decode give-up {qt_gu}/{qt_d}", flush=True)
     m = 1
-    gate, up, down = _weights(dev, seed=90)
+    gate, up, down = _weights(dev, qt_gu, qt_d, seed=90)
     ws = torch.zeros(ops.mlp_decode_workspace_bytes(m, H, I), dtype=torch.uint8, device=dev)
     x = synthetic.make_activations(m, H, seed=8, device=dev)
     y = torch.empty((m, H), dtype=torch.bfloat16, device=dev)
-    ops.mlp_decode_into(x, None, EPS, gate, up, go.Q8_0, down, go.Q8_0, None, y, ws, 1, spin_limit=-1)
+    ops.mlp_decode_into(x, None, EPS, gate, up, qt_gu, down, qt_d, None, y, ws, 1, spin_limit=-1)
     torch.cuda.synchronize()
     assert int(ws[0:4].view(torch.int32).item()) == 1          # generation advanced: every workgroup came through
     gave_up = ops.mlp_decode_gave_up(ws)
     print(f"  gave up: {gave_up}", flush=True)
     off = int(ops.load_library().sngguf_mlp_decode_status_offset())
     ws[off:off + 4].zero_()
-    ops.mlp_decode_into(x, None, EPS, gate, up, go.Q8_0, down, go.Q8_0, None, y, ws, 1)
-    want = _separate(x, None, gate, up, down, go.Q8_0, go.Q8_0, None, 1)[0]
+    ops.mlp_decode_into(x, None, EPS, gate, up, qt_gu, down, qt_d, None, y, ws, 1)
+    want = _separate(x, None, gate, up, down, qt_gu, qt_d, None, 1)[0]
     assert go.rel_l2(y.cpu(), want.cpu()) <= 1e-4 and not ops.mlp_decode_gave_up(ws)
 
 
-@pytest.mark.parametrize("qt_gu,qt_d,m,hidden,inter", [(go.Q8_0, go.Q8_0, 3, H, I), (go.Q8_0, go.Q8_0, 16, H, I), (go.Q4_K, go.Q6_K, 1, H, I),
+@pytest.mark.parametrize("qt_gu,qt_d,m,hidden,inter", [(go.Q8_0, go.Q8_0, 3, H, I), (go.Q8_0, go.Q8_0, 16, H, I), (go.Q4_K, go.Q6_K, 3, H, I),
+                                                        (go.Q6_K, go.Q6_K, 1, H, I), (go.Q8_0, go.Q6_K, 1, H, I), (go.Q4_K, go.Q8_0, 2, H, I),
                                                         (go.Q8_0, go.Q8_0, 2, 2048, 6144), (go.Q4_K, go.Q4_K, 3, 1024, 2816),
                                                         (go.Q8_0, go.Q8_0, 1, 512, 1536)])
 def test_other_shapes_and_types_run_the_separate_launches(dev, qt_gu, qt_d, m, hidden, inter):
