@@ -55,16 +55,31 @@ __device__ __forceinline__ f32x4_t widen_f16x4(half4_t ident, half2_t lo, half2_
 // integer is formed without a convert); NUM 0: exact fp32 products, one rounding in the subtraction
 // (the - 1024 - zero rides on the accumulator input of the widening instruction).  Must be called
 // by all 64 lanes; `ident` is identity_row(lane).
-template <int NUM, bool HAS_MIN>
+// FUSED (formats with a minimum and zero = 0): the product and the operation next to it as one fused multiply-add
+// where that gives the same bits.  NUM 0: D * q is exact in fp32 (at most 11 + 6 + 5 significant bits), so
+// fma(D, q, -DM) rounds once exactly where D * q - DM does.  NUM 1: (1024 + q) * D - 1024 * D, exact inside the
+// fused operation, rounds once to fp16(q * D); -1024 * D is exact in fp16 unless it overflows, so the caller takes
+// this form only where every |D| of the wavefront is below 64 (a scale product that large has not been seen in a
+// file; the plain form stays for it).
+template <int NUM, bool HAS_MIN, bool FUSED = false>
 __device__ __forceinline__ void kq_dword_bf16(half4_t ident, uint32_t v, float zero, typename Num<NUM>::T D,
                                               typename Num<NUM>::T DM, uint32_t& p01, uint32_t& p23) {
     const half2_t h01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u));
     const half2_t h23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u));
     if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
-        const _Float16 off = (_Float16)(1024.0f + zero);
-        const half2_t off2 = {off, off};
         const half2_t D2 = {D, D};
-        half2_t a = (h01 - off2) * D2, b = (h23 - off2) * D2;
+        half2_t a, b;
+        if constexpr (FUSED) {
+            const _Float16 c = (_Float16)(-1024.0f) * D;
+            const half2_t C2 = {c, c};
+            a = __builtin_elementwise_fma(h01, D2, C2);
+            b = __builtin_elementwise_fma(h23, D2, C2);
+        } else {
+            const _Float16 off = (_Float16)(1024.0f + zero);
+            const half2_t off2 = {off, off};
+            a = (h01 - off2) * D2;
+            b = (h23 - off2) * D2;
+        }
         if constexpr (HAS_MIN) {
             const half2_t M2 = {DM, DM};
             a = a - M2;
@@ -76,10 +91,17 @@ __device__ __forceinline__ void kq_dword_bf16(half4_t ident, uint32_t v, float z
     } else {
         const float c = -(1024.0f + zero);
         const f32x4_t qf = widen_f16x4(ident, h01, h23, f32x4_t{c, c, c, c});
-        float w[4] = {D * qf[0], D * qf[1], D * qf[2], D * qf[3]};
-        if constexpr (HAS_MIN) {
+        float w[4];
+        if constexpr (FUSED && HAS_MIN) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) w[e] = w[e] - DM;
+            for (int e = 0; e < 4; e++) w[e] = __builtin_fmaf(D, qf[e], -DM);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) w[e] = D * qf[e];
+            if constexpr (HAS_MIN) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = w[e] - DM;
+            }
         }
         p01 = pack_bf16(w[0], w[1]);
         p23 = pack_bf16(w[2], w[3]);
@@ -272,7 +294,7 @@ __device__ __forceinline__ void decode_q3_k(half4_t ident, const uint8_t* row, i
 // values are bit-identical; it takes a quarter of the decode's vector instructions away.  Must be called by all
 // 64 lanes.
 template <int NUM, int HALF>
-__device__ __forceinline__ void q4k_pairs(const u32x4_t& head, int g, typename Num<NUM>::T (&D)[4], typename Num<NUM>::T (&DM)[4]) {
+__device__ __forceinline__ bool q4k_pairs(const u32x4_t& head, int g, typename Num<NUM>::T (&D)[4], typename Num<NUM>::T (&DM)[4]) {
     typedef Num<NUM> A;
     uint32_t sc, mn;
     if constexpr (HALF == 0) {
@@ -295,23 +317,23 @@ __device__ __forceinline__ void q4k_pairs(const u32x4_t& head, int g, typename N
             D[jj] = got[0];
             DM[jj] = got[1];
         }
+        // every |d * scale| of the wavefront below 64 (0x5400): the fused form of kq_dword_bf16 is exact
+        return __builtin_amdgcn_ballot_w64(((uint32_t)bits & 0x7FFFu) >= 0x5400u) == 0;
     } else {
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             D[jj] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(self + 64 * jj, __builtin_bit_cast(int, mine_d)));
             DM[jj] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(self + 64 * jj, __builtin_bit_cast(int, mine_m)));
         }
+        return true;
     }
 }
 
 // The four A operands of half a super-block (sub-blocks 4 HALF .. 4 HALF + 3) of one row, fed to
 // `emit(jj, a)` with jj = 0..3.  `row` points at the row's super-block in the slab; g = lane / 16.
-template <int NUM, int HALF, typename Emit>
-__device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
-    typedef Num<NUM> A;
-    const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
-    typename A::T Ds[4], DMs[4];
-    q4k_pairs<NUM, HALF>(head, g, Ds, DMs);
+template <int NUM, int HALF, bool FUSED, typename Emit>
+__device__ __forceinline__ void decode_q4_k_body(half4_t ident, const uint8_t* row, int g, const typename Num<NUM>::T (&Ds)[4],
+                                                 const typename Num<NUM>::T (&DMs)[4], Emit&& emit) {
 #pragma unroll
     for (int cc = 0; cc < 2; cc++) {
         const int c = 2 * HALF + cc;
@@ -319,23 +341,28 @@ __device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, i
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
             const int j = 2 * c + hi;
-            const typename A::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
+            const typename Num<NUM>::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
             const uint32_t v0 = (hi ? qs[0] >> 4 : qs[0]) & 0x0F0F0F0Fu, v1 = (hi ? qs[1] >> 4 : qs[1]) & 0x0F0F0F0Fu;
             uint32_t a0, a1, a2, a3;
-            kq_dword_bf16<NUM, true>(ident, v0, 0.f, D, DM, a0, a1);
-            kq_dword_bf16<NUM, true>(ident, v1, 0.f, D, DM, a2, a3);
+            kq_dword_bf16<NUM, true, FUSED>(ident, v0, 0.f, D, DM, a0, a1);
+            kq_dword_bf16<NUM, true, FUSED>(ident, v1, 0.f, D, DM, a2, a3);
             emit(j - 4 * HALF, u32x4_t{a0, a1, a2, a3});
         }
     }
 }
-
-// Q5_K: as Q4_K, the fifth bit of element l of sub-block j is bit j of qh[l]
 template <int NUM, int HALF, typename Emit>
-__device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+__device__ __forceinline__ void decode_q4_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
     typedef Num<NUM> A;
     const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
     typename A::T Ds[4], DMs[4];
-    q4k_pairs<NUM, HALF>(head, g, Ds, DMs);
+    if (q4k_pairs<NUM, HALF>(head, g, Ds, DMs)) decode_q4_k_body<NUM, HALF, true>(ident, row, g, Ds, DMs, emit);
+    else decode_q4_k_body<NUM, HALF, false>(ident, row, g, Ds, DMs, emit);
+}
+
+// Q5_K: as Q4_K, the fifth bit of element l of sub-block j is bit j of qh[l]
+template <int NUM, int HALF, bool FUSED, typename Emit>
+__device__ __forceinline__ void decode_q5_k_body(half4_t ident, const uint8_t* row, int g, const typename Num<NUM>::T (&Ds)[4],
+                                                 const typename Num<NUM>::T (&DMs)[4], Emit&& emit) {
     const u32x2_t qh = *reinterpret_cast<const u32x2_t*>(row + 16 + 8 * g);
 #pragma unroll
     for (int cc = 0; cc < 2; cc++) {
@@ -344,17 +371,25 @@ __device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, i
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
             const int j = 2 * c + hi;
-            const typename A::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
+            const typename Num<NUM>::T D = Ds[j - 4 * HALF], DM = DMs[j - 4 * HALF];
             uint32_t a[4];
 #pragma unroll
             for (int w = 0; w < 2; w++) {
                 const uint32_t lo = (hi ? qs[w] >> 4 : qs[w]) & 0x0F0F0F0Fu;
                 const uint32_t hb = ((qh[w] >> j) & 0x01010101u) << 4;
-                kq_dword_bf16<NUM, true>(ident, lo | hb, 0.f, D, DM, a[2 * w], a[2 * w + 1]);
+                kq_dword_bf16<NUM, true, FUSED>(ident, lo | hb, 0.f, D, DM, a[2 * w], a[2 * w + 1]);
             }
             emit(j - 4 * HALF, u32x4_t{a[0], a[1], a[2], a[3]});
         }
     }
+}
+template <int NUM, int HALF, typename Emit>
+__device__ __forceinline__ void decode_q5_k(half4_t ident, const uint8_t* row, int g, Emit&& emit) {
+    typedef Num<NUM> A;
+    const u32x4_t head = *reinterpret_cast<const u32x4_t*>(row);  // d, dmin, 12 scale bytes
+    typename A::T Ds[4], DMs[4];
+    if (q4k_pairs<NUM, HALF>(head, g, Ds, DMs)) decode_q5_k_body<NUM, HALF, true>(ident, row, g, Ds, DMs, emit);
+    else decode_q5_k_body<NUM, HALF, false>(ident, row, g, Ds, DMs, emit);
 }
 
 template <int NUM, int HALF, typename Emit>

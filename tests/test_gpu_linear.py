@@ -160,6 +160,36 @@ def test_q8_0_fp16_subnormal_products(dev, numerics, m):
         _check(got, want)
 
 
+@pytest.mark.parametrize("qt", [go.Q4_K, go.Q5_K])
+@pytest.mark.parametrize("numerics", [0, 1])
+def test_k_quant_decode_with_scale_products_on_both_sides_of_64(dev, c_oracle, qt, numerics):
+    """The decode kernel of Q4_K / Q5_K forms q * D as one fused multiply-add around the constant -1024 * D where every
+    |D| = |d * scale| of a wavefront is below 64 (so that the constant is exact in fp16), and keeps the separate
+    subtraction and product elsewhere.  Super-block scales d of 2^-10, 1.5 and 24 with the 6-bit sub-scales put D far
+    below 64, on both sides of it within one wavefront, and beyond the range where 1024 * D would still be finite:
+    all must follow the oracle's chain; one and sixteen rows, the plain projection and the gated pair."""
+    import numpy as np
+    print(f"case k-quant scale products qt={qt} numerics={numerics}", flush=True)
+    n, k = 96, 2048
+    for m in (1, 16):
+        for case, d_values in enumerate(([2.0 ** -10], [1.5], [24.0], [2.0 ** -10, 1.5, 24.0])):
+            mats = []
+            for which in range(2):
+                raw = synthetic.make_packed(qt, n, k, seed=7 * case + which + m).numpy().copy()
+                blocks = raw.reshape(n, k // 256, -1)
+                rng = np.random.default_rng(case + which)
+                d = rng.choice(np.array(d_values, dtype=np.float16), size=(n, k // 256))
+                blocks[..., 0:2] = d.view(np.uint16)[..., None].view(np.uint8)
+                blocks[..., 2:4] = np.array([0.25], dtype=np.float16).view(np.uint8)      # dmin
+                mats.append(torch.from_numpy(raw))
+            x = (synthetic.make_activations(m, k, seed=case + 3).float() / 64).to(torch.bfloat16)
+            want = go.gguf_linear_forward(x, mats[0], qt, None, numerics=numerics)
+            assert bool(torch.isfinite(want.float()).all()) and want.float().abs().max() > 0
+            _check(ops.linear(x.to(dev), mats[0].to(dev), qt, None, numerics).cpu(), want)
+            up = go.gguf_linear_forward(x, mats[1], qt, None, numerics=numerics)
+            _check(ops.gate_up_silu(x.to(dev), mats[0].to(dev), mats[1].to(dev), qt, numerics).cpu(), c_oracle.silu_mul(want, up))
+
+
 def test_gemv_fp64_bruteforce_tiny(dev):
     """Independent of torch's matmul: exact fp64 dot products on the bf16-rounded weights."""
     print("case gemv fp64", flush=True)
