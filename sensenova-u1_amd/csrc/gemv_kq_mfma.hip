@@ -29,27 +29,6 @@ namespace sngguf {
 namespace {
 
 
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-
-// fp16 -> fp32 on the matrix core.  With A = the 16 x 16 identity, v_mfma_f32_16x16x16_f16 computes
-// D = I . B + C, and because a lane's B elements (column lane % 16, rows 4 (lane / 16) .. + 3) sit
-// at the same positions as its D elements, every lane gets back its own four fp16 values as
-// exact fp32 (+ c).  The K-quant decode is bound by the vector ALU while the matrix cores are
-// nearly idle, so this takes one conversion per element off the busy unit.  fp16 subnormals are
-// widened exactly; a signed zero comes back as + 0, and a non-finite element (a scale product
-// beyond the fp16 range) turns the other values of its weight row in that instruction into NaN
-// (0 . inf) - the row's dot product is non-finite either way.
-__device__ __forceinline__ half4_t identity_row(int lane) {
-    half4_t a;
-#pragma unroll
-    for (int e = 0; e < 4; e++) a[e] = (4 * (lane >> 4) + e == (lane & 15)) ? (_Float16)1.0f : (_Float16)0.0f;
-    return a;
-}
-__device__ __forceinline__ f32x4_t widen_f16x4(half4_t ident, half2_t lo, half2_t hi, f32x4_t c) {
-    const half4_t b = {lo[0], lo[1], hi[0], hi[1]};
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(ident, b, c, 0, 0, 0);
-}
-
 // Four small unsigned integers (one per byte of v, each < 256) -> (v - zero) * D - DM as two packed
 // bf16 pairs.  NUM 1: every operation rounds to fp16 (0x6400 | b is the half 1024 + b, so the
 // integer is formed without a convert); NUM 0: exact fp32 products, one rounding in the subtraction

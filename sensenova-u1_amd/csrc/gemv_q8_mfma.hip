@@ -736,6 +736,7 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     // (this wavefront's ring is its own again; the vector ALU has room while other wavefronts wait for memory, and once
     // the activations are there only the 32 matrix instructions are left)
     u32x4_t afrag[kSteps * CB];
+    const half4_t ident = identity_row(lane);
     auto decode = [&](int i) {
         const uint8_t* sl = slab0;
         const uint8_t* lrow = sl + r * kRowStep + 8 * g;
@@ -754,8 +755,15 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
                 q1 = w[1];
             }
             uint32_t a0, a1, a2, a3;
-            q8_dword_bf16<NUM>(d, q0, a0, a1);
-            q8_dword_bf16<NUM>(d, q1, a2, a3);
+            // the fp16 -> fp32 step of the decode on the matrix cores: this phase is bound by the vector ALU (36.3 ->
+            // 35.1 us for the launch; in the first phase, which waits for memory, and in the separate launches it gains
+            // nothing or loses)
+            const uint32_t d2 = (uint32_t)d | ((uint32_t)d << 16);
+            q8_dword_bf16_widened<NUM>(ident, d2, q0, a0, a1);
+            q8_dword_bf16_widened<NUM>(ident, d2, q1, a2, a3);
+            // (pinned here: left alone, the compiler moves the roundings down to the matrix instructions behind the wait
+            // and keeps the widened values, twice the registers, across it)
+            asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
             afrag[i * CB + b] = u32x4_t{a0, a1, a2, a3};
         }
     };

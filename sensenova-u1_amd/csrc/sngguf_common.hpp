@@ -358,6 +358,48 @@ __device__ __forceinline__ void q8_dword_bf16_d2(uint32_t d2_bits, uint32_t dw, 
         p23 = pack_bf16(d * (float)(int8_t)((dw >> 16) & 0xFF), d * (float)(int8_t)(dw >> 24));
     }
 }
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+// fp16 -> fp32 on the matrix core.  With A = the 16 x 16 identity, v_mfma_f32_16x16x16_f16 computes
+// D = I . B + C, and because a lane's B elements (column lane % 16, rows 4 (lane / 16) .. + 3) sit
+// at the same positions as its D elements, every lane gets back its own four fp16 values as
+// exact fp32 (+ c).  The K-quant decode is bound by the vector ALU while the matrix cores are
+// nearly idle, so this takes one conversion per element off the busy unit.  fp16 subnormals are
+// widened exactly; a signed zero comes back as + 0, and a non-finite element (a scale product
+// beyond the fp16 range) turns the other values of its weight row in that instruction into NaN
+// (0 . inf) - the row's dot product is non-finite either way.
+__device__ __forceinline__ half4_t identity_row(int lane) {
+    half4_t a;
+#pragma unroll
+    for (int e = 0; e < 4; e++) a[e] = (4 * (lane >> 4) + e == (lane & 15)) ? (_Float16)1.0f : (_Float16)0.0f;
+    return a;
+}
+__device__ __forceinline__ f32x4_t widen_f16x4(half4_t ident, half2_t lo, half2_t hi, f32x4_t c) {
+    const half4_t b = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(ident, b, c, 0, 0, 0);
+}
+
+// q8_dword_bf16_d2 with the fp16 -> fp32 step on the matrix core (all 64 lanes must call it): two vector instructions
+// per weight instead of three.  NUM 0: the widening instruction's accumulator input takes the 1024 + 128 off, so the
+// quant arrives as an exact float without a convert either.
+template <int NUM>
+__device__ __forceinline__ void q8_dword_bf16_widened(half4_t ident, uint32_t d2_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
+    const uint32_t u = dw ^ 0x80808080u;
+    const half2_t h01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u));
+    const half2_t h23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u));
+    if constexpr (NUM == SNGGUF_NUM_UPSTREAM_FP16) {
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const half2_t d2 = __builtin_bit_cast(half2_t, d2_bits);
+        const f32x4_t w = widen_f16x4(ident, (h01 - bias) * d2, (h23 - bias) * d2, f32x4_t{0.f, 0.f, 0.f, 0.f});
+        p01 = pack_bf16(w[0], w[1]);
+        p23 = pack_bf16(w[2], w[3]);
+    } else {
+        const float d = f16_to_f32((uint16_t)(d2_bits & 0xFFFF));
+        const f32x4_t qf = widen_f16x4(ident, h01, h23, f32x4_t{-1152.f, -1152.f, -1152.f, -1152.f});
+        p01 = pack_bf16(d * qf[0], d * qf[1]);
+        p23 = pack_bf16(d * qf[2], d * qf[3]);
+    }
+}
 // Same with the scale as the 16 bits of the block header.
 template <int NUM>
 __device__ __forceinline__ void q8_dword_bf16(uint16_t d_bits, uint32_t dw, uint32_t& p01, uint32_t& p23) {
