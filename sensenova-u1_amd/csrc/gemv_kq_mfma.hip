@@ -753,16 +753,17 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
 // the phase: a wavefront leaves its partial sums in LDS and counts itself in for its row group; the group's storing
 // wavefront waits for that count only.  Phase B: 16 rows of the down matrix, K = inter split over the twelve
 // wavefronts, four super-blocks each; two of them are requested the moment the wavefront leaves phase A's loop, the
-// other two after one workgroup barrier (requested earlier, their traffic slows phase A's last wavefronts, which the
-// whole device waits for), and all four wait as raw bytes in registers; the first is decoded into matrix-core operands
+// other two when every wavefront of the workgroup has left it (a count in LDS; requested earlier, their traffic slows
+// phase A's last wavefronts, which the whole device waits for), and all four wait as raw bytes in registers; the first is decoded into matrix-core operands
 // while the activations are on their way.  Then the wavefront polls the flags of the 64 row groups its K range needs,
 // reads the tagged words (every tag checked), contracts the decoded super-block, decodes and contracts the other three,
 // and the twelve partial sums are added.  Bounded wait, status word, generation counter and workspace layout as in the
 // Q8_0 kernel (MlpCtl).  Without `gamma` the gated activations are bit-identical to the gated pair's own launch (same
 // fragments, same order of accumulation), and so is the output (the down projection's own launch splits K over eight
 // wavefronts, not twelve: equal up to the order of twelve fp32 additions, which the tests allow for).
-// The decode arithmetic, not memory, bounds these formats: the launch is worth 1 - 3 % over the two separate ones
-// (34.1 against 34.3 us with a Q6_K down projection, 31.9 against 33.0 with Q4_K), where the Q8_0 kernel gains 11 %.
+// The decode arithmetic, not memory, bounds these formats: the launch is level with the two separate ones or up to 3 %
+// ahead by device (33.5 against 34.0 us with a Q6_K down projection, 31.9 - 32.8 against 32.7 - 33.0 with Q4_K), where
+// the Q8_0 kernel gains 10 %.
 template <int QT>
 struct SlabIo {
     typedef Slab<QT> S;
@@ -927,6 +928,9 @@ __global__ __launch_bounds__(64 * kMlpKqWaves) void mlp_kq_decode_kernel(const b
     uint16_t raw_d[kSteps] = {};
     ib.fetch(bbase, sb0, lane, raw[0], raw_d[0]);
     ib.fetch(bbase, sb0 + 1, lane, raw[1], raw_d[1]);
+    // counted as having left the loop: the other two steps are requested when that count is full
+    uint32_t* const left_a = cnt + 8;
+    if (lane == 0) __hip_atomic_fetch_add(left_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 
     // ---- phase A epilogue: partial sums, per-group count, the storing wavefront's SiLU and tagged stores ----
     red_a[wave * 64 + lane] = acc;
@@ -968,7 +972,8 @@ __global__ __launch_bounds__(64 * kMlpKqWaves) void mlp_kq_decode_kernel(const b
     };
     if constexpr (kAhead > 0) decode(0);
     if constexpr (kAhead > 1) decode(1);
-    __syncthreads();   // the whole workgroup has left phase A: now the other two steps' traffic
+    // every wavefront of the workgroup has left phase A's loop: now the other two steps' traffic
+    while (__hip_atomic_load(left_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)kWaves) __builtin_amdgcn_s_sleep(1);
     ib.fetch(bbase, sb0 + 2, lane, raw[2], raw_d[2]);
     ib.fetch(bbase, sb0 + 3, lane, raw[3], raw_d[3]);
     if constexpr (kAhead > 2) decode(2);

@@ -772,7 +772,9 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     // every wavefront fetching and decoding all four steps as soon as it is free, no barrier, 40.4 us (56 us when only
     // the first few to arrive do so); a workgroup barrier before steps 2 and 3 are requested and all decoding behind it
     // 36.6 ... 37.1 us; steps 0 and 1 decoded in front of that barrier by every wavefront 35.5 us (by the first six or
-    // eight to arrive only: 36.4 us).
+    // eight to arrive only: 36.4 us).  The last wavefronts to leave the loop requesting all four steps at once: no gain.
+    // (a counter of the first phase's area that no row group uses: the body zeroes sixteen of them in front of its first barrier)
+    uint32_t* const left_a = reinterpret_cast<uint32_t*>(reinterpret_cast<f32x4_t*>(red_a) + kWaves * 64) + 8;
     __builtin_amdgcn_s_setprio(2);   // the first phase is what every other workgroup waits for
     gemv_q8_span_body<NUM, true, 12, true, false, true>(
         lds, x, M, q_gate, q_up, inter, hidden, nullptr, nullptr, reinterpret_cast<bf16_t*>(ht), gamma, eps, nullptr, 3, 1, bid,
@@ -781,6 +783,8 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
             // the first two down-projection steps, requested the moment this wavefront leaves the loop
             dfetch(s0, pre);
             dfetch(s0 + 1, pre2);
+            // counted as having left the loop: the other two steps are requested when that count is full
+            if (lane == 0) __hip_atomic_fetch_add(left_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         },
         tag, kMlpWaveLds, red_a);
     // a wavefront that wrote a row group's activations also raises that group's flag (behind the data, unordered)
@@ -796,13 +800,16 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     __builtin_amdgcn_s_setprio(0);
     MLP_TRACE(2);
     // steps 0 and 1 move into LDS and are decoded at once, at the lowest priority (this wavefront's partial sums are
-    // counted in: nobody waits for it); steps 2 and 3 are requested only when the whole workgroup has left the first
-    // phase - requested earlier, their traffic slows the first phase's last wavefronts, which every workgroup waits for
+    // counted in: nobody waits for it); steps 2 and 3 are requested only when every wavefront of the workgroup has left
+    // the first phase's loop - requested earlier, their traffic slows the first phase's last wavefronts, which every
+    // workgroup waits for.  (A count that a wavefront joins when it leaves the loop, not a barrier behind the two decode
+    // steps: with the barrier the workgroup's last wavefront held the others' requests back by its own two steps,
+    // 35.0 against 33.5 us for the launch.)
     to_slab(pre);
     decode(0);
     to_slab(pre2);
     decode(1);
-    __syncthreads();
+    while (__hip_atomic_load(left_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)kWaves) __builtin_amdgcn_s_sleep(1);
     dfetch(s0 + 2, pre);
     dfetch(s0 + 3, pre2);
     to_slab(pre);
@@ -815,6 +822,8 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     // ---- wait for this wavefront's K range of the activations ----
     // staged (tags stripped), 2048 bytes per row, behind this wavefront's slab (at most two rows: the launcher checks);
     // fragment (step i, block b) of a row at ((i CB + b) 64 + 16 g)
+    // (Requesting the words in front of the last decode step, on the expectation that they are there, and polling only
+    // if a tag says otherwise, gained nothing: the last activations become visible about when the last weights arrive.)
     constexpr int xrow_b = kSteps * CB * 64;
     auto xw_row = [&](int m) -> uint8_t* { return slab0 + kSlab + m * xrow_b; };
     {
