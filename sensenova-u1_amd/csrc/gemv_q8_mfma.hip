@@ -909,8 +909,10 @@ int64_t mlp_q8_decode_status_offset() { return (int64_t)offsetof(MlpCtl, status)
 // Shapes the one-launch form takes: Q8_0 everywhere; hidden = 4096 (two spans per row: the twelve-wavefront form of
 // the gated pair); inter = 3 hidden (as many 48-row slices of gate / up as 16-row groups of down: one of each per
 // workgroup) and 12 wavefronts x 4 steps x 256 elements of it per row of the down projection; one or two rows (their staged
-// copies fit behind a wavefront's slab; with three and four rows, tried with the copies elsewhere in LDS, the separate
-// launches were 3 - 6 % faster: polling and reading the tagged words grows with the rows); as many compute units as workgroups and the kernel resident on each.
+// copies fit behind a wavefront's slab; three and four rows, staged and contracted two at a time, came out level with
+// the separate launches, 38.7 - 39.9 against 39.1 - 40.7 us: every workgroup reads every row's tagged words, 12.5 MB of
+// coherent reads per row over the device behind the last weights); as many compute units as workgroups and the kernel
+// resident on each.
 bool mlp_q8_decode_fits(int64_t M, int64_t hidden, int64_t inter) {
     if (M < 1 || M > 2 || hidden != 4096 || inter != 3 * hidden || inter != 12 * 4 * 256) return false;
     static const int ok = [] {
