@@ -761,9 +761,10 @@ int launch_qt(const bf16_t* x, int M, const uint8_t* qa, const uint8_t* qb, int6
 // Q8_0 kernel (MlpCtl).  Without `gamma` the gated activations are bit-identical to the gated pair's own launch (same
 // fragments, same order of accumulation), and so is the output (the down projection's own launch splits K over eight
 // wavefronts, not twelve: equal up to the order of twelve fp32 additions, which the tests allow for).
-// The decode arithmetic, not memory, bounds these formats: the launch is level with the two separate ones or up to 3 %
-// ahead by device (33.5 against 34.0 us with a Q6_K down projection, 31.9 - 32.8 against 32.7 - 33.0 with Q4_K), where
-// the Q8_0 kernel gains 10 %.
+// The decode arithmetic, not memory, bounds these formats: the launch is 0 - 5 % ahead of the two separate ones by device
+// and down type (32.3 against 33.9 us with a Q6_K down projection once the down projection's first requests are made
+// behind phase A's epilogue instead of in front of it; 31.9 - 32.8 against 32.7 - 33.0 with Q4_K), where the Q8_0 kernel
+// gains 10 %.
 template <int QT>
 struct SlabIo {
     typedef Slab<QT> S;
@@ -926,13 +927,8 @@ __global__ __launch_bounds__(64 * kMlpKqWaves) void mlp_kq_decode_kernel(const b
     ib.init(lane, brow_bytes);
     u32x4_t raw[kSteps][IB::kLoads];
     uint16_t raw_d[kSteps] = {};
-    ib.fetch(bbase, sb0, lane, raw[0], raw_d[0]);
-    ib.fetch(bbase, sb0 + 1, lane, raw[1], raw_d[1]);
-    // counted as having left the loop: the other two steps are requested when that count is full
-    uint32_t* const left_a = cnt + 8;
-    if (lane == 0) __hip_atomic_fetch_add(left_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-
-    // ---- phase A epilogue: partial sums, per-group count, the storing wavefront's SiLU and tagged stores ----
+    // ---- phase A epilogue: partial sums, per-group count, the storing wavefront's SiLU and tagged stores; the down
+    // projection's first requests come behind it, so that they do not queue in front of what other workgroups wait for ----
     red_a[wave * 64 + lane] = acc;
     if (lane == 0) __hip_atomic_fetch_add(cnt + grp, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (lw == 0) {
@@ -956,6 +952,12 @@ __global__ __launch_bounds__(64 * kMlpKqWaves) void mlp_kq_decode_kernel(const b
         }
         if (lane == 0) __hip_atomic_store(&ctl->flags[3 * bid + grp], tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    ib.fetch(bbase, sb0, lane, raw[0], raw_d[0]);
+    ib.fetch(bbase, sb0 + 1, lane, raw[1], raw_d[1]);
+    // counted as having left the loop: the other two steps are requested when that count is full
+    uint32_t* const left_a = cnt + 8;
+    if (lane == 0) __hip_atomic_fetch_add(left_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+
     __builtin_amdgcn_s_setprio(0);
 
     // ---- phase B: decode the first kAhead super-blocks into matrix-core operands while the activations are on their

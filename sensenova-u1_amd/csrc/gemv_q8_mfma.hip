@@ -301,8 +301,8 @@ constexpr int kSpanBytes = 2176;  // 64 blocks = 17 lines
 // fragment is fetched once for both - with several activation rows those fetches, not the weights, fill the
 // vector memory path (16 rows x 64 bytes per matrix instruction against 544 bytes of weights).
 // The body of the line-aligned kernel for workgroup `bid`.  `after_loop(stores)` is called by every wavefront when it
-// has left its K loop, before the workgroup adds up the partial sums; `stores` tells whether this wavefront will write
-// outputs.  AGENT_STORES: for consumers inside the same launch, and the wavefronts of a workgroup leave the body one by
+// has left its K loop, before the workgroup adds up the partial sums (with AGENT_STORES: when the wavefront has left its
+// own sums in LDS and counted itself in); `stores` tells whether this wavefront will write outputs.  AGENT_STORES: for consumers inside the same launch, and the wavefronts of a workgroup leave the body one by
 // one instead of together (`red_lds` must then be room for the partial sums plus 64 bytes that nothing else uses).
 // y is then an array of 8-byte words, word (m N + n) / 2 = { outputs n, n + 1 of row m as two bf16, tag }, each written
 // with one agent-scope store (it reaches memory that every compute unit of the device reads): a reader that finds
@@ -564,7 +564,7 @@ __device__ __forceinline__ void gemv_q8_span_body(uint8_t* lds, const bf16_t* __
         }
     }
 
-    after_loop(lw == 0 && live);
+    if constexpr (!AGENT_STORES) after_loop(lw == 0 && live);
     // ---- add the wavefronts' partial sums (the rings are dead: reuse them) ---------------------------
     // per row group: [gate partial sums of the W K ranges | up partial sums][64]; the paired mode keeps the up sums of
     // all wavefronts behind the gate sums of all wavefronts
@@ -575,6 +575,7 @@ __device__ __forceinline__ void gemv_q8_span_body(uint8_t* lds, const bf16_t* __
         uint32_t* cnt = reinterpret_cast<uint32_t*>(red + waves * 64) + grp;
         red[lwave * 64 + lane] = acc[0];
         if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        after_loop(lw == 0 && live);   // (behind the partial sums: what it requests must not hold them up)
         if (lw != 0 || !live) return;
         while (__hip_atomic_load(cnt, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)wpg) __builtin_amdgcn_s_sleep(1);
     } else {
@@ -804,7 +805,8 @@ __global__ __launch_bounds__(768) void mlp_q8_decode_kernel(const bf16_t* __rest
     // the first phase's loop - requested earlier, their traffic slows the first phase's last wavefronts, which every
     // workgroup waits for.  (A count that a wavefront joins when it leaves the loop, not a barrier behind the two decode
     // steps: with the barrier the workgroup's last wavefront held the others' requests back by its own two steps,
-    // 35.0 against 33.5 us for the launch.  Each register set refilled the moment it is free, which moves the last two
+    // 35.0 against 33.5 us for the launch.  The requests at the loop's end behind the storing wavefront's whole epilogue
+    // (partners awaited, activations and flag stored first): 34.1 us.  Each register set refilled the moment it is free, which moves the last two
     // requests in front of the first two decode steps: 35.1 us; only one step requested at the loop's end: 34.7 us.)
     to_slab(pre);
     decode(0);
