@@ -31,7 +31,7 @@ HIDDEN, INTER, KV = 4096, 12288, 1024
 # HBM bytes per launch of the dominant kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
 # each scaled by what the same counter reads for the plain 256 MiB elementwise copy that
 # --calibrate-copy runs in the same process; None = not measured for this build.
-MEASURED_TRAFFIC = {"mlp_one_launch_m1": 164846627, "gemv_gate_up_m1": 107641642, "gemm_gate_m4096": 516357081, "gemm_dense_gate_m4096": 705231439}
+MEASURED_TRAFFIC = {"mlp_one_launch_m1": 164774013, "gemv_gate_up_m1": 107629683, "gemm_gate_m4096": 516359845, "gemm_dense_gate_m4096": 705462160}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 Q8_0, Q4_K, Q6_K = 8, 12, 14
